@@ -1,0 +1,374 @@
+"""Pins for the CPU oracle: each oracle function is checked against something that is not the oracle's
+own formula -- the reference's docstring vectors, the literal torch expression the reference evaluates,
+closed forms, library routines (scipy, torch SDPA) and brute force on tiny inputs."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import shareprefill_oracle as O
+
+
+# ----- literal restatements of the reference's torch expressions, used only as checkers -----------
+def literal_cover_topk(x, score):  # utils.py:47-50
+    c = torch.cumsum(torch.sort(x, dim=-1, descending=True, stable=True).values, dim=-1)
+    return int(torch.sum(c <= score, dim=-1)) + 1
+
+
+def literal_cover_idx(x, score):  # utils.py:53-57
+    xs, idx = torch.sort(x, dim=-1, descending=True, stable=True)
+    c = torch.cumsum(xs, dim=-1)
+    return idx[~(c > score)]
+
+
+def literal_each_row(a, score):  # utils.py:60-76
+    xs, idx = torch.sort(a, dim=-1, descending=True, stable=True)
+    c = torch.cumsum(xs, dim=-1)
+    t = (c >= score).float().argmax(dim=-1) + 1
+    keep = torch.zeros_like(a, dtype=torch.bool)
+    for r in range(a.shape[0]):
+        keep[r, idx[r, : int(t[r])]] = True
+    return keep.numpy()
+
+
+def rand_probs(n, seed, sharp=3.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.softmax(torch.randn(n, generator=g) * sharp, dim=-1)
+
+
+# ----- reference docstring vectors ----------------------------------------------------------------
+def test_csr_docstring_vector():
+    # shareprefill_attn.py:235-236
+    assert O.csr_row_pointers(np.array([0, 5, 8, 9, 13, 14]), 4).tolist() == [0, 1, 2, 4, 6]
+
+
+def test_csr_ignores_padding_ids():
+    nb = 4
+    ids = np.array([0, 5, 8, 13, 14, nb * (nb + 1), nb * (nb + 1)])
+    assert O.csr_row_pointers(ids, nb).tolist() == [0, 1, 2, 3, 5]
+
+
+def test_flat_id_docstring_vector():
+    # shareprefill_attn.py:491-492: blocks (0,0),(1,1),(2,0),(3,1),(3,2) <-> [0,5,8,13,14]
+    m = np.zeros((4, 4), dtype=bool)
+    for r, c in [(0, 0), (1, 1), (2, 0), (3, 1), (3, 2)]:
+        m[r, c] = True
+    assert O.mask_to_ids(m).tolist() == [0, 5, 8, 13, 14]
+
+
+# ----- pooling --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [256, 300, 129])
+def test_pool_avg_is_block_mean(n):
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(n, 3, 16, generator=g)
+    y = O.pool_avg(x, 128)
+    nb = -(-n // 128)
+    assert y.shape == (nb, 3, 16)
+    for b in range(nb):
+        ref = x[b * 128: min((b + 1) * 128, n)].double().mean(0)
+        assert torch.allclose(y[b].double(), ref, atol=1e-6)
+
+
+def test_pool_avg_constant_and_linear():
+    x = torch.full((300, 2, 16), 0.375)
+    assert torch.equal(O.pool_avg(x, 128), torch.full((3, 2, 16), 0.375))
+    g = torch.Generator().manual_seed(0)
+    a, b = torch.randn(256, 2, 16, generator=g), torch.randn(256, 2, 16, generator=g)
+    assert torch.allclose(O.pool_avg(a + 2 * b, 128), O.pool_avg(a, 128) + 2 * O.pool_avg(b, 128), atol=1e-5)
+
+
+def test_pool_q_head_tail_rescale():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(300, 16, generator=g)
+    y = O.pool_q_head(x, 128)
+    assert torch.allclose(y[2], x[256:].mean(0), atol=1e-5)
+    assert torch.allclose(y[0], x[:128].mean(0), atol=1e-6)
+
+
+# ----- anti-diagonal sums ---------------------------------------------------------------------------
+def test_diagonal_sums_bruteforce():
+    g = torch.Generator().manual_seed(1)
+    n, m = 8, 40
+    p = torch.rand(n, m, generator=g, dtype=torch.float64)
+    out = O.diagonal_sums(p)
+    ref = torch.zeros(m, dtype=torch.float64)
+    for j in range(m):
+        for i in range(n):
+            c = j + i - (n - 1)
+            if 0 <= c < m:
+                ref[j] += p[i, c]
+    assert torch.allclose(out, ref, atol=1e-12)
+    # last entry is the main diagonal of the trailing n x n square
+    assert math.isclose(out[m - 1].item(), sum(p[i, m - n + i].item() for i in range(n)), rel_tol=1e-12)
+
+
+def test_lastq_scores_invariants_and_bruteforce():
+    g = torch.Generator().manual_seed(2)
+    hq, hkv, n, d, bs = 4, 2, 512, 16, 128
+    q = torch.randn(hq, n, d, generator=g)
+    k = torch.randn(hkv, n, d, generator=g)
+    vert, slash = O.lastq_scores(q, k, bs, logits_in_input_dtype=False)
+    assert torch.allclose(vert.sum(-1), torch.ones(hq), atol=1e-5)
+    assert torch.allclose(slash.sum(-1), torch.ones(hq), atol=1e-5)
+    h = 3
+    s = (q[h, -bs:].double() / math.sqrt(d)) @ k[h // 2].double().T
+    for i in range(bs):
+        s[i, n - bs + i + 1:] = -math.inf
+    p = torch.softmax(s, -1)
+    assert torch.allclose(vert[h].double(), p.mean(0), atol=1e-6)
+    diag = sum(p[i, n - bs + i].item() for i in range(bs)) / bs
+    assert math.isclose(slash[h, n - 1].item(), diag, rel_tol=1e-4)
+    j = 200  # distance n-1-j behind each query
+    ref = sum(p[i, j + i - (bs - 1)].item() for i in range(bs) if 0 <= j + i - (bs - 1) < n) / bs
+    assert math.isclose(slash[h, j].item(), ref, rel_tol=1e-4, abs_tol=1e-9)
+
+
+# ----- cumulative-mass selection -------------------------------------------------------------------
+def test_cover_count_closed_forms():
+    onehot = np.zeros(1000, dtype=np.float32)
+    onehot[123] = 1.0
+    assert O.cover_count(onehot, 0.95) == 1
+    n = 1024  # uniform 2^-10: exactly representable, cumsum exact
+    uni = np.full(n, 1.0 / n, dtype=np.float32)
+    for thr in (0.5, 0.9, 0.95, 0.99):
+        assert O.cover_count(uni, thr) == math.floor(float(np.float32(thr)) * n) + 1
+
+
+@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("thr", [0.9, 0.95, 0.99])
+def test_cover_count_matches_literal_torch(seed, thr):
+    x = rand_probs(4096 + 37 * seed, seed)
+    assert O.cover_count(x.numpy(), thr) == literal_cover_topk(x, thr)
+
+
+def test_cover_count_is_smallest_prefix_exceeding():
+    x = rand_probs(300, 5).numpy()
+    m = O.cover_count(x, 0.9)
+    s = np.sort(x.astype(np.float64))[::-1]
+    assert s[: m - 1].sum() <= 0.9 + 1e-9
+    assert s[:m].sum() > 0.9 - 1e-9
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_cover_keep_le_matches_literal_and_excludes_crossing(seed):
+    nb = 16
+    g = torch.Generator().manual_seed(seed)
+    a = torch.softmax(torch.randn(nb, nb, generator=g) * 2, -1).reshape(-1)
+    score = 0.9 * nb
+    kept = O.cover_keep_le(a.numpy(), score)
+    lit = literal_cover_idx(a, score)
+    assert sorted(kept.tolist()) == sorted(lit.tolist())
+    assert a[kept].double().sum().item() <= score + 1e-6
+    rest = np.setdiff1d(np.arange(nb * nb), kept)
+    assert a[kept].double().sum().item() + a[rest].max().item() > score - 1e-6
+
+
+def test_cover_keep_le_largest_exceeds_score_keeps_nothing():
+    x = np.array([0.7, 0.2, 0.1], dtype=np.float32)
+    assert O.cover_keep_le(x, 0.5).size == 0
+
+
+def test_cover_keep_le_tie_order_is_index_ascending():
+    x = np.array([0.25, 0.25, 0.25, 0.25], dtype=np.float32)
+    assert O.cover_keep_le(x, 0.5).tolist() == [0, 1]
+    assert O.cover_keep_le(x, 0.74).tolist() == [0, 1]
+    assert O.cover_keep_le(x, 0.75).tolist() == [0, 1, 2]
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_cover_keep_rows_matches_literal_and_includes_crossing(seed):
+    g = torch.Generator().manual_seed(100 + seed)
+    a = torch.softmax(torch.randn(12, 20, generator=g) * 2, -1)
+    keep = O.cover_keep_rows_ge(a.numpy(), 0.9)
+    assert np.array_equal(keep, literal_each_row(a, 0.9))
+    for r in range(a.shape[0]):
+        sel = a[r][torch.from_numpy(keep[r])].double()
+        assert sel.sum().item() >= 0.9 - 1e-6
+        assert sel.sum().item() - sel.min().item() < 0.9 + 1e-6
+
+
+def test_cover_keep_rows_never_reaching_keeps_one():
+    a = np.array([[0.3, 0.4, 0.1], [0.5, 0.45, 0.05]], dtype=np.float32)
+    keep = O.cover_keep_rows_ge(a, 0.9)
+    assert keep[0].tolist() == [False, True, False]  # total 0.8 < 0.9: argmax of all-False -> 1 entry
+    assert keep[1].tolist() == [True, True, False]
+
+
+def test_fixed_point_conversion():
+    x = np.array([1.0, 0.5, 2.0 ** -48, 2.0 ** -49, 0.0, -1.0, np.nan, 3.0 * 2.0 ** -30], dtype=np.float32)
+    fx = O.to_fixed(x)
+    assert fx.tolist() == [2 ** 48, 2 ** 47, 1, 0, 0, 0, 0, 3 * 2 ** 18]
+    assert O.thr_le(0.5) == 2 ** 47 and O.thr_lt(0.5) == 2 ** 47 - 1
+
+
+# ----- JS divergence ----------------------------------------------------------------------------------
+def test_sqrt_js_vs_scipy():
+    from scipy.spatial.distance import jensenshannon
+
+    p, q = rand_probs(257, 1, 1.0), rand_probs(257, 2, 1.0)
+    assert math.isclose(O.sqrt_js(p, q).item(), jensenshannon(p.numpy(), q.numpy()), rel_tol=1e-4)
+    assert O.sqrt_js(p, p).item() == 0.0
+    assert math.isclose(O.sqrt_js(p, q).item(), O.sqrt_js(q, p).item(), rel_tol=1e-6)
+
+
+def test_sqrt_js_zero_entry_is_nan_and_compares_false():
+    p = torch.tensor([0.5, 0.5, 0.0])
+    q = torch.tensor([0.25, 0.25, 0.5])
+    v = O.sqrt_js(p, q)
+    assert torch.isnan(v)
+    assert not bool(v < 0.5)
+
+
+# ----- vertical-slash expansion ---------------------------------------------------------------------
+def test_vs_id_list_bruteforce_nb5():
+    ids = O.vs_id_list(cols=[0, 3], dists=[0, 2], nb=5)
+    assert set(ids.tolist()) == {0, 5, 6, 10, 12, 15, 16, 18, 20, 22, 23, 24}
+    assert len(ids) == 5 * 4
+    # layout: slash part first (row-major over r, then d), then the vertical part
+    assert ids[:10].tolist() == [0, 10, 6, 16, 12, 22, 18, 0, 24, 0]
+    assert ids[10:].tolist() == [0, 0, 5, 0, 10, 0, 15, 18, 20, 23]
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_vs_mask_equals_id_set(seed):
+    rng = np.random.default_rng(seed)
+    nb = 11
+    cols = np.concatenate([[0], rng.choice(np.arange(1, nb), 3, replace=False)])
+    dists = np.concatenate([[0], rng.choice(np.arange(1, nb), 2, replace=False)])
+    ids = set(O.vs_id_list(cols, dists, nb).tolist())
+    m = O.vs_mask(cols, dists, nb)
+    assert ids == set(O.mask_to_ids(m).tolist())
+    assert all(m[r, r] and m[r, 0] for r in range(nb))
+    assert not np.triu(m, 1).any()
+
+
+def test_vs_ratio_counts_duplicates_hand_example():
+    # 3x3 map, cols {0,2}, dists {0,1}.  id list (slash | vertical):
+    #   slash: r=0:(0,0)->0,(1,0)->3 ; r=1:(1,1)->4,(2,1)->7 ; r=2:(2,2)->8, pad 0
+    #   vert : r=0: 0, pad 0 ; r=1: 3, pad 0 ; r=2: 6, 8
+    avg = np.array([[1.0, 0, 0], [0.5, 0.5, 0], [0.25, 0.25, 0.5]], dtype=np.float32)
+    ids = O.vs_id_list([0, 2], [0, 1], 3)
+    assert ids.tolist() == [0, 3, 4, 7, 8, 0, 0, 0, 3, 0, 6, 8]
+    lit = avg.reshape(-1)[ids].astype(np.float64).sum() / avg.astype(np.float64).sum()
+    assert math.isclose(lit, (1 + .5 + .5 + .25 + .5 + 1 + 1 + 1 + .5 + 1 + .25 + .5) / 3.0)
+    assert math.isclose(O.vs_ratio(avg, [0, 2], [0, 1]), lit, rel_tol=1e-12)
+    assert O.vs_ratio(avg, [0, 2], [0, 1]) > 1.0
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_vs_ratio_matches_literal_gather(seed):
+    rng = np.random.default_rng(seed)
+    nb = 9
+    avg = np.tril(rng.random((nb, nb))).astype(np.float32)
+    avg /= avg.sum(1, keepdims=True)
+    cols = np.concatenate([[0], rng.choice(np.arange(1, nb), 3, replace=False)])
+    dists = np.concatenate([[0], rng.choice(np.arange(1, nb), 3, replace=False)])
+    ids = O.vs_id_list(cols, dists, nb)
+    lit = avg.reshape(-1)[ids].astype(np.float64).sum() / avg.astype(np.float64).sum()
+    assert math.isclose(O.vs_ratio(avg, cols, dists), lit, rel_tol=1e-9)
+
+
+# ----- masked attention -------------------------------------------------------------------------------
+def test_masked_attention_full_mask_is_sdpa_causal():
+    g = torch.Generator().manual_seed(4)
+    hq, hkv, n, d, bs = 4, 2, 300, 32, 128
+    q, k, v = (torch.randn(h, n, d, generator=g) for h in (hq, hkv, hkv))
+    nb = 3
+    mask = np.tril(np.ones((nb, nb), dtype=bool))[None].repeat(hq, 0)
+    out, avg = O.masked_attention(q, k, v, mask, bs, 1 / math.sqrt(d), want_avg=np.ones(hq, bool))
+    ke, ve = k.repeat_interleave(2, 0), v.repeat_interleave(2, 0)
+    ref = torch.nn.functional.scaled_dot_product_attention(q[None], ke[None], ve[None], is_causal=True)[0]
+    assert torch.allclose(out, ref, atol=2e-5)
+    assert torch.allclose(avg.sum(-1), torch.ones(hq, nb), atol=1e-5)
+    s = (q[1] @ ke[1].T) / math.sqrt(d)
+    s = s.masked_fill(torch.triu(torch.ones(n, n, dtype=torch.bool), 1), -math.inf)
+    p = torch.softmax(s, -1)
+    assert math.isclose(avg[1, 2, 1].item(), p[256:300, 128:256].sum().item() / 44, rel_tol=1e-4)
+
+
+def test_masked_attention_diagonal_mask_is_per_block_causal():
+    g = torch.Generator().manual_seed(5)
+    n, d, bs = 256, 16, 128
+    q, k, v = (torch.randn(1, n, d, generator=g) for _ in range(3))
+    mask = np.eye(2, dtype=bool)[None]
+    out, _ = O.masked_attention(q, k, v, mask, bs, 0.25)
+    for b in range(2):
+        sl = slice(b * bs, (b + 1) * bs)
+        ref = torch.nn.functional.scaled_dot_product_attention(q[:, sl][None], k[:, sl][None], v[:, sl][None],
+                                                               is_causal=True, scale=0.25)[0]
+        assert torch.allclose(out[:, sl], ref, atol=2e-5)
+
+
+# ----- sharing scenarios on a toy table ----------------------------------------------------------------
+def _toy(seed=0, n=1024, hq=4, hkv=2, d=32):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(hq, n, d, generator=g)
+    k = torch.randn(hkv, n, d, generator=g)
+    v = torch.randn(hkv, n, d, generator=g)
+    k[:, :8] *= 3
+    return q, k, v
+
+
+TOY_TABLE = {"clusters": {"a": [[0, 0], [0, 1], [1, 0], [1, 1]], "b": [[0, 2], [0, 3], [1, 2], [1, 3]]},
+             "shared_clusters": ["a"]}
+KW = dict(bs=128, min_budget=128, max_budget=None, pattern_threshold=0.9, similarity_threshold=0.5,
+          fallback_threshold=1e9, queryaware_threshold=0.0)
+
+
+def test_sharing_scenarios():
+    q, k, v = _toy()
+    sh = O.OracleSharing(O.ClusterTable(TOY_TABLE["clusters"], TOY_TABLE["shared_clusters"]))
+    r0 = sh.layer(q, k, v, 0, **KW)
+    # (i) first non-QA head of the shared cluster becomes the dense pivot; (ii) its same-layer sibling does not share
+    assert r0.decision.tolist() == [O.DEC_DENSE, O.DEC_VS, O.DEC_VS, O.DEC_VS]
+    nb = 8
+    assert np.array_equal(r0.mask[0], np.tril(np.ones((nb, nb), bool)))
+    assert sh.state["a"].pivot_head == 0 and sh.state["a"].pattern is not None
+    # (v) the non-shared cluster never elects a pivot
+    assert sh.state["b"].pivot_head is None
+    # every row holds its sink column and its diagonal block
+    for h in range(4):
+        assert all(r0.mask[h, r, 0] and r0.mask[h, r, r] for r in range(nb))
+    # (iii) next layer: identical inputs -> JS = 0 -> both cluster members share (fallback disabled by 1e9)
+    r1 = sh.layer(q, k, v, 1, **KW)
+    assert r1.decision.tolist() == [O.DEC_SHARE, O.DEC_SHARE, O.DEC_VS, O.DEC_VS]
+    assert r1.js_v[0] == 0.0 and r1.js_s[0] == 0.0
+    assert (r1.mask[0] & sh.state["a"].pattern).sum() == sh.state["a"].pattern.sum()
+    assert r1.nv_final[0] == 1 and r1.ns_final[0] == 1
+
+
+def test_sharing_blocked_by_fallback_and_similarity():
+    q, k, v = _toy()
+    sh = O.OracleSharing(O.ClusterTable(TOY_TABLE["clusters"], TOY_TABLE["shared_clusters"]))
+    kw = dict(KW)
+    sh.layer(q, k, v, 0, **kw)
+    kw["fallback_threshold"] = 0.0  # vs_ratio >= 0 always -> never share
+    r1 = sh.layer(q, k, v, 1, **kw)
+    assert O.DEC_SHARE not in r1.decision.tolist()
+    # (iv) a dissimilar head falls back: similarity threshold 0 can never be met (JS >= 0)
+    sh.reset_state()
+    kw = dict(KW, similarity_threshold=0.0)
+    sh.layer(q, k, v, 0, **kw)
+    r1 = sh.layer(q, k, v, 1, **kw)
+    assert O.DEC_SHARE not in r1.decision.tolist()
+
+
+def test_query_aware_head_never_becomes_pivot():
+    q, k, v = _toy()
+    sh = O.OracleSharing(O.ClusterTable(TOY_TABLE["clusters"], TOY_TABLE["shared_clusters"]))
+    kw = dict(KW, queryaware_threshold=10.0)  # every head with a finite JS is query-aware
+    r0 = sh.layer(q, k, v, 0, **kw)
+    assert all(d == O.DEC_QA for d in r0.decision.tolist())
+    assert sh.state["a"].pivot_head is None
+    assert r0.mask[:, 0, 0].all()
+    assert not np.triu(r0.mask[0], 1).any()
+
+
+def test_reset_state_clears_pivots():
+    q, k, v = _toy()
+    sh = O.OracleSharing(O.ClusterTable(TOY_TABLE["clusters"], TOY_TABLE["shared_clusters"]))
+    sh.layer(q, k, v, 0, **KW)
+    sh.reset_state()
+    assert sh.state["a"].pivot_head is None and sh.state["a"].pattern is None
