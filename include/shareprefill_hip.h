@@ -1,0 +1,182 @@
+/*
+ * shareprefill_hip.h -- C ABI of libshareprefill_hip.so (MI355X / gfx950).
+ *
+ * The library is the device side of the SharePrefill prefill-attention layer: block average
+ * pooling, last-block vertical/slash scoring, cumulative-mass block selection, cross-head
+ * pattern sharing and the GQA causal block-sparse flash attention.  The reference implements
+ * this path in Python + Triton; each entry point below names the reference code it replaces
+ * (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the comment says "host";
+ *   - batch size is 1 (shareprefill/attn/attention_sharing.py:42-44);
+ *   - q/k/v are bf16 with explicit element strides for the token and head axes and a
+ *     contiguous head_dim axis, so both [N,H,D] and [H,N,D] storage are accepted as is;
+ *   - all work is enqueued on `stream` (a hipStream_t; NULL = the default stream), nothing
+ *     synchronises the stream, nothing allocates;
+ *   - return value 0 = ok, negative = error (SP_ERR_*), text from sp_last_error();
+ *   - block masks are bit matrices: mask[h][r][w] is a uint64 word, bit (c & 63) of word
+ *     (c >> 6) is block (r, c); nbw = ceil(nb / 64) words per row.  Flat block id of the
+ *     reference = r * nb + c (shareprefill/attn/shareprefill_attn.py:491-492).
+ */
+#ifndef SHAREPREFILL_HIP_H
+#define SHAREPREFILL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SP_OK 0
+#define SP_ERR_INVALID_ARGUMENT (-1)
+#define SP_ERR_UNSUPPORTED (-2)
+#define SP_ERR_HIP (-3)
+#define SP_ERR_WORKSPACE (-4)
+
+/* per-head decision written by sp_share_decide (attention_sharing.py:182-190 use_dense/use_share/use_query_aware) */
+#define SP_DEC_VS 0
+#define SP_DEC_DENSE 1
+#define SP_DEC_SHARE 2
+#define SP_DEC_QA 3
+
+/* flags */
+#define SP_FLAG_LOGITS_BF16 1u /* round pooled / last-block logits to bf16 as the reference's bf16 einsum does */
+
+/* tail handling of sp_pool_avg_bf16 */
+#define SP_POOL_TAIL_TRUE_LENGTH 0 /* divide the ragged last block by its length (attn/utils.py:171,187) */
+#define SP_POOL_TAIL_RESCALE 1     /* mean over bs, then *bs/(bs-pad) in bf16 (attention_sharing.py:350-356) */
+
+typedef void* sp_stream_t;
+
+/* Cross-layer sharing state, one slot per SHARED cluster (attention_sharing.py:41-78).
+ * The struct itself lives in host memory; every member pointer is device memory owned by the caller. */
+typedef struct sp_cluster_state {
+  int32_t n_clusters;
+  int32_t nb;  /* blocks per side the slabs are sized for */
+  int32_t nbw; /* ceil(nb/64) */
+  int32_t reserved;
+  int32_t* info;     /* [C][8]: 0 pivot head (-1 none), 1 has_pattern, 2 pivot nv, 3 pivot ns, 4 pivot layer */
+  double* ratio;     /* [C]     vs_ratio of the pivot (valid once has_pattern) */
+  float* vert;       /* [C][nb] pivot's pooled last-row vertical vector */
+  float* slash;      /* [C][nb] pivot's pooled last-row slash vector */
+  uint8_t* cols;     /* [C][nb] 1 = block column in the pivot's own vertical set */
+  uint8_t* dists;    /* [C][nb] 1 = block distance in the pivot's own slash set */
+  uint64_t* pattern; /* [C][nb][nbw] pivot block pattern */
+  uint64_t* accum;   /* [C][2]  scratch of sp_pivot_update (covered / total mass, fixed point) */
+} sp_cluster_state;
+
+/* ---- library info ------------------------------------------------------------------------- */
+int sp_version(void);
+const char* sp_arch(void);       /* "gfx950" */
+const char* sp_last_error(void); /* host string, valid until the next failing call on this thread */
+
+/* ---- (a) block average pooling --------------------------------------------------------------
+ * Replaces triton_bnhd_pool / bnhd_pool_kernel (attn/utils.py:131-261, "avg" mode) and the torch
+ * .mean used for Q (attention_sharing.py:350-356).
+ * x: bf16 [n][h][d] with strides; y: bf16 [nb][h][d] contiguous.  fp32 accumulation.
+ * head_enable: optional int32[h]; heads with 0 are skipped (their rows of y are left untouched). */
+int sp_pool_avg_bf16(const void* x, void* y, int64_t n, int32_t h, int32_t d, int64_t x_stride_n,
+                     int64_t x_stride_h, int32_t bs, int32_t tail_mode, const int32_t* head_enable,
+                     sp_stream_t stream);
+
+/* ---- last-block scores -> vertical / slash --------------------------------------------------
+ * Replaces attention_sharing.py:127-167 + sum_all_diagonal_matrix (attn/utils.py:79-86) +
+ * torch_bhn_sumpool (attn/utils.py:33-44): softmax over all keys of the last bs queries
+ * (scaled by 1/sqrt(d), causal inside the last bs columns), column mean -> vert_tok[hq][n],
+ * anti-diagonal mean -> slash_tok[hq][n], and their block sums vert_blk / slash_blk [hq][nb].
+ * workspace: sp_lastq_scores_workspace_bytes(...) bytes of device scratch. */
+size_t sp_lastq_scores_workspace_bytes(int64_t n, int32_t hq, int32_t bs);
+int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int32_t hq, int32_t hkv, int32_t d,
+                         int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                         int32_t bs, uint32_t flags, void* workspace, size_t workspace_bytes,
+                         float* vert_tok, float* slash_tok, float* vert_blk, float* slash_blk,
+                         sp_stream_t stream);
+
+/* ---- cumulative-mass primitives (attn/utils.py:47-76) --------------------------------------
+ * Canonical arithmetic: entries ordered by (value desc, index asc); running sums are exact
+ * sums of the values truncated to unsigned 2^-48 fixed point.  Inputs: finite, >= 0, row sum < 2^14.
+ *
+ * sp_cover_count: score_cover_topk (utils.py:47-50): out[v] = count(cumsum <= thr) + 1 for each of
+ * n_vec vectors of length len (row stride = len). */
+int sp_cover_count(const float* x, int32_t n_vec, int64_t len, float thr, int32_t* out, sp_stream_t stream);
+
+/* budgets of attention_sharing.py:169-176: clamp(cover_count(.)/bs + 1, minb, maxb) for both vectors */
+int sp_cover_budgets(const float* vert_tok, const float* slash_tok, int32_t hq, int64_t n, int32_t bs,
+                     float pattern_threshold, int32_t min_blocks, int32_t max_blocks, int32_t* nv, int32_t* ns,
+                     sp_stream_t stream);
+
+/* ---- query-aware test (attention_sharing.py:193-202) ----------------------------------------
+ * avg_qk[h] = softmax_fp32(mean_i(last_q[h]) . kbar[:, h/g]); js_qa[h] = sqrt_JS(avg_qk[h], vert_blk[h]);
+ * use_qa[h] = js_qa[h] < queryaware_threshold (NaN compares false).  kbar: bf16 [nb][hkv][d]. */
+int sp_queryaware_test_bf16(const void* q, const void* kbar, const float* vert_blk, int64_t n, int32_t hq,
+                            int32_t hkv, int32_t d, int64_t q_stride_n, int64_t q_stride_h, int32_t bs,
+                            uint32_t flags, float queryaware_threshold, float* avg_qk, float* js_qa,
+                            int32_t* use_qa, sp_stream_t stream);
+
+/* ---- pivot election / share test (attention_sharing.py:204-301) -----------------------------
+ * Walks the heads in ascending order.  head_cluster[h] = slot of the head's cluster in `state`
+ * for this layer, or -1 when the head is in no shared cluster.  Writes decision[h] (SP_DEC_*),
+ * js_v / js_s (NaN where no share test ran) and the final budgets (min_blocks for QA / sharing heads).
+ * A newly elected pivot stores its pooled vectors, its budgets and its own vertical / slash sets. */
+int sp_share_decide(const sp_cluster_state* state /* host */, const int32_t* head_cluster, int32_t layer_idx,
+                    int32_t hq, const float* vert_blk, const float* slash_blk, const int32_t* use_qa,
+                    const int32_t* nv, const int32_t* ns, int32_t min_blocks, float similarity_threshold,
+                    double fallback_threshold, int32_t* decision, float* js_v, float* js_s, int32_t* nv_final,
+                    int32_t* ns_final, sp_stream_t stream);
+
+/* ---- mask construction (attention_sharing.py:303-337, attn/utils.py:99-128) -----------------
+ * mask[h] = vertical-slash blocks (sink column and main diagonal forced, top-nv columns, top-ns
+ * distances) | all lower-triangular blocks (DENSE) | the cluster pivot's pattern (SHARE).
+ * Overwrites mask[hq][nb][nbw]. */
+int sp_build_mask(const sp_cluster_state* state /* host */, const int32_t* head_cluster, const int32_t* decision,
+                  const float* vert_blk, const float* slash_blk, const int32_t* nv_final, const int32_t* ns_final,
+                  int32_t hq, int32_t nb, uint64_t* mask, sp_stream_t stream);
+
+/* ---- query-aware block selection (attention_sharing.py:339-364, attn/utils.py:53-57) --------
+ * For heads with decision == SP_DEC_QA: probs[h] = softmax rows of (qbar[h]/sqrt(d)) . kbar^T with the
+ * block-causal mask ([nb][nb] fp32, caller scratch [hq][nb][nb]); then the global cumulative-mass
+ * selection at pattern_threshold * nb (crossing entry excluded) is OR-ed into mask[h].
+ * qbar: bf16 [nb][hq][d] (sp_pool_avg_bf16 of q), kbar: bf16 [nb][hkv][d]. */
+int sp_queryaware_select_bf16(const void* qbar, const void* kbar, const int32_t* decision, int32_t hq,
+                              int32_t hkv, int32_t d, int32_t nb, uint32_t flags, float pattern_threshold,
+                              float* probs, uint64_t* mask, sp_stream_t stream);
+
+/* the selection alone, on caller-supplied probabilities: mask[v] |= kept entries of x[v] ([nb][nb] each),
+ * restricted to the lower triangle; vectors with enable[v] == 0 are skipped (enable may be NULL). */
+int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec, int32_t nb, float score,
+                           uint64_t* mask, sp_stream_t stream);
+
+/* ---- GQA causal block-sparse flash attention ------------------------------------------------
+ * Replaces triton_block_wise_prefill_attention / block_wise_prefill_attention_kernel /
+ * count_kernel (shareprefill_attn.py:187-620).  out: bf16 [n][hq][d] contiguous.  Only blocks set in
+ * mask (and c <= r) are computed.  For heads with decision == SP_DEC_DENSE the block-averaged attention
+ * map avg_attn[h][nb][nb] (fp32, pre-zeroed by the caller) is written as well (:425-457).
+ * vt_workspace: sp_attn_workspace_bytes(...) bytes of device scratch (key-major repack of V). */
+size_t sp_attn_workspace_bytes(int64_t n, int32_t hkv, int32_t d, int32_t bs);
+int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,
+                                  int32_t d, int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n,
+                                  int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h, int32_t bs,
+                                  float softmax_scale, const uint64_t* mask, const int32_t* decision, void* out,
+                                  float* avg_attn, void* workspace, size_t workspace_bytes, sp_stream_t stream);
+
+/* ---- pivot state update (attention_sharing.py:94-103, attn/utils.py:60-76) ------------------
+ * For each head with decision == SP_DEC_DENSE: per-row cumulative-mass selection (>= threshold,
+ * crossing entry included) of avg_attn[h] -> state.pattern, the pivot's vs_ratio
+ * (attention_sharing.py:278-286, duplicates counted) -> state.ratio, has_pattern = 1. */
+int sp_pivot_update(const sp_cluster_state* state /* host */, const int32_t* head_cluster, const int32_t* decision,
+                    const float* avg_attn, int32_t hq, int32_t nb, float pattern_threshold, sp_stream_t stream);
+
+/* per-row selection alone: pattern[r] = kept entries of row r of x[nb][nb] (lower triangle, (0,0) set) */
+int sp_cover_select_rows(const float* x, int32_t nb, float thr, uint64_t* pattern, sp_stream_t stream);
+
+/* ---- helpers ----------------------------------------------------------------------------------
+ * CSR row pointers of a mask (triton_column_count_cumsum, shareprefill_attn.py:226-269):
+ * row_ptr[h][r+1] = number of set blocks in rows 0..r of head h; row_ptr[h][0] = 0. */
+int sp_mask_row_pointers(const uint64_t* mask, int32_t hq, int32_t nb, int32_t* row_ptr, sp_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SHAREPREFILL_HIP_H */

@@ -1,0 +1,296 @@
+// Last-block scores: softmax over all keys of the last 128 queries, reduced to the per-token
+// vertical (column mean) and slash (anti-diagonal mean) vectors and their 128-token block sums.
+// Replaces shareprefill/attn/attention_sharing.py:127-167, sum_all_diagonal_matrix
+// (attn/utils.py:79-86) and torch_bhn_sumpool (attn/utils.py:33-44) without ever writing the
+// [Hq,128,N] probability matrix to memory.
+//
+// Three kernels:
+//   stats   : per (head, key chunk) the running row max / row sum of the logits (bf16 MFMA);
+//   combine : folds the chunk partials into one (max, 1/sum) per query row, in chunk order;
+//   probs   : recomputes the logits tile by tile, writes the probabilities of one 128x128 tile to
+//             LDS, and lets 128 threads sum columns (vertical) while the other 128 sum the tile's
+//             anti-diagonals (slash).  A slash bin receives its upper part from the previous key tile;
+//             that part is carried in a register, and each workgroup recomputes one leading tile so
+//             that no cross-workgroup accumulation (and no float atomic) is needed.
+// Every sum runs in a fixed order, so results are reproducible run to run.
+#include "sp_common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+#define LQ_ROWS 128          // query rows (= block size)
+#define LQ_TILE 128          // keys per tile
+#define LQ_D 128             // head dim
+#define LQ_THREADS 256       // 4 waves, wave w owns query rows 32w..32w+31
+#define LQ_STAT_TILES 8      // key tiles per stats workgroup
+#define LQ_PROB_TILES 8      // output key tiles per probs workgroup (plus one leading tile)
+#define LQ_PITCH 136         // LDS row pitch (floats) of the probability tile
+
+// lane's A operand: scaled last-block queries, 8 k-steps x 8 bf16
+__device__ static inline void lq_load_q(const sp_bf16* __restrict__ q, int64_t n, int64_t sq_n, int wave, int lane,
+                                        float inv_sqrt_d, bf16x8 qa[8]) {
+  const int row = wave * 32 + (lane & 31);
+  const sp_bf16* src = q + (n - LQ_ROWS + row) * sq_n + 8 * (lane >> 5);
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    uint4 raw = *reinterpret_cast<const uint4*>(src + 16 * ks);
+    uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      // last_q = bf16(q * (1/sqrt(d))), attention_sharing.py:127
+      uint32_t lo = sp_f32_to_bf16(__uint_as_float(w[j] << 16) * inv_sqrt_d);
+      uint32_t hi = sp_f32_to_bf16(__uint_as_float(w[j] & 0xffff0000u) * inv_sqrt_d);
+      w[j] = lo | (hi << 16);
+    }
+    raw = make_uint4(w[0], w[1], w[2], w[3]);
+    qa[ks] = __builtin_bit_cast(bf16x8, raw);
+  }
+}
+
+// logits of this wave's 32 query rows against the 128 keys of tile `kb`:
+// acc[nt][r] = S[row 32w + 8(r/4) + 4(lane/32) + r%4][key kb + 32nt + lane%32]
+__device__ static inline void lq_tile_logits(const sp_bf16* __restrict__ k, int64_t n, int64_t sk_n, int64_t kb,
+                                             int lane, const bf16x8 qa[8], floatx16 acc[4]) {
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    int64_t key = kb + 32 * nt + (lane & 31);
+    if (key > n - 1) key = n - 1;  // out-of-range keys are masked by the caller
+    const sp_bf16* src = k + key * sk_n + 8 * (lane >> 5);
+    floatx16 c = {0};
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      uint4 raw = *reinterpret_cast<const uint4*>(src + 16 * ks);
+      c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[ks], __builtin_bit_cast(bf16x8, raw), c, 0, 0, 0);
+    }
+    acc[nt] = c;
+  }
+}
+
+__device__ static inline int lq_row_of(int wave, int lane, int r) {
+  return wave * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+}
+
+// ---- kernel 1: chunk partials of the row max / row sum ------------------------------------------
+__global__ __launch_bounds__(LQ_THREADS) void sp_lastq_stats_kernel(
+    const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
+    int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, int n_chunks,
+    float2* __restrict__ partial /* [hq][n_chunks][128] */) {
+  const int h = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const sp_bf16* qh = q + (int64_t)h * sq_h;
+  const sp_bf16* kh = k + (int64_t)(h / group) * sk_h;
+  bf16x8 qa[8];
+  lq_load_q(qh, n, sq_n, wave, lane, inv_sqrt_d, qa);
+
+  float m[16], l[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
+  }
+  const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
+  for (int t = 0; t < LQ_STAT_TILES; ++t) {
+    const int64_t tile = (int64_t)chunk * LQ_STAT_TILES + t;
+    if (tile >= n_tiles) break;
+    const int64_t kb = tile * LQ_TILE;
+    floatx16 acc[4];
+    lq_tile_logits(kh, n, sk_n, kb, lane, qa, acc);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int64_t qpos = n - LQ_ROWS + lq_row_of(wave, lane, r);
+      float s[4];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int64_t key = kb + 32 * nt + (lane & 31);
+        float v = acc[nt][r];
+        if (flags & SP_FLAG_LOGITS_BF16) v = sp_round_bf16(v);
+        v = (key <= qpos && key < n) ? v : -INFINITY;
+        s[nt] = v;
+        tmax = fmaxf(tmax, v);
+      }
+      if (tmax > -INFINITY) {
+        const float mn = fmaxf(m[r], tmax);
+        float add = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) add += __expf(s[nt] - mn);
+        l[r] = l[r] * __expf(m[r] - mn) + add;
+        m[r] = mn;
+      }
+    }
+  }
+  // merge the 32 lanes that share a row (fixed xor tree)
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float mm = m[r], ll = l[r];
+#pragma unroll
+    for (int o = 1; o < 32; o <<= 1) {
+      const float m2 = __shfl_xor(mm, o, SP_WAVE);
+      const float l2 = __shfl_xor(ll, o, SP_WAVE);
+      const float mn = fmaxf(mm, m2);
+      if (mn > -INFINITY) {
+        ll = ll * __expf(mm - mn) + l2 * __expf(m2 - mn);
+      }
+      mm = mn;
+    }
+    if ((lane & 31) == 0) {
+      partial[((int64_t)h * n_chunks + chunk) * LQ_ROWS + lq_row_of(wave, lane, r)] = make_float2(mm, ll);
+    }
+  }
+}
+
+// ---- kernel 2: fold chunk partials ------------------------------------------------------------------
+__global__ __launch_bounds__(LQ_ROWS) void sp_lastq_combine_kernel(const float2* __restrict__ partial, int n_chunks,
+                                                                   float2* __restrict__ rowstat /* [hq][128] */) {
+  const int h = blockIdx.x, row = threadIdx.x;
+  const float2* p = partial + (int64_t)h * n_chunks * LQ_ROWS + row;
+  float m = -INFINITY;
+  for (int c = 0; c < n_chunks; ++c) m = fmaxf(m, p[(int64_t)c * LQ_ROWS].x);
+  float l = 0.f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const float2 v = p[(int64_t)c * LQ_ROWS];
+    if (v.x > -INFINITY) l += v.y * __expf(v.x - m);
+  }
+  rowstat[h * LQ_ROWS + row] = make_float2(m, 1.0f / l);
+}
+
+// ---- kernel 3: probabilities -> vertical / slash ------------------------------------------------------
+__global__ __launch_bounds__(LQ_THREADS) void sp_lastq_probs_kernel(
+    const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
+    int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, const float2* __restrict__ rowstat,
+    float* __restrict__ vert_tok, float* __restrict__ slash_tok, float* __restrict__ vert_blk,
+    float* __restrict__ slash_blk, int64_t nb) {
+  extern __shared__ float lds[];
+  float* P = lds;                           // [128][LQ_PITCH]
+  float* red = lds + LQ_ROWS * LQ_PITCH;    // [4] wave partials of the block sums
+  const int h = blockIdx.y;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const sp_bf16* qh = q + (int64_t)h * sq_h;
+  const sp_bf16* kh = k + (int64_t)(h / group) * sk_h;
+  bf16x8 qa[8];
+  lq_load_q(qh, n, sq_n, wave, lane, inv_sqrt_d, qa);
+  float rm[16], rinv[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float2 st = rowstat[h * LQ_ROWS + lq_row_of(wave, lane, r)];
+    rm[r] = st.x;
+    rinv[r] = st.y;
+  }
+  const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
+  const int64_t first = (int64_t)blockIdx.x * LQ_PROB_TILES;
+  const float inv_rows = 1.0f / (float)LQ_ROWS;
+  float carry = 0.f;  // upper anti-diagonal part handed from the previous tile to bin (u) of this one
+  const int u = threadIdx.x & 127;
+
+  for (int64_t tile = first - 1; tile < first + LQ_PROB_TILES && tile < n_tiles; ++tile) {
+    if (tile < 0) continue;
+    const int64_t kb = tile * LQ_TILE;
+    floatx16 acc[4];
+    lq_tile_logits(kh, n, sk_n, kb, lane, qa, acc);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = lq_row_of(wave, lane, r);
+      const int64_t qpos = n - LQ_ROWS + row;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int c = 32 * nt + (lane & 31);
+        const int64_t key = kb + c;
+        float v = acc[nt][r];
+        if (flags & SP_FLAG_LOGITS_BF16) v = sp_round_bf16(v);
+        const float p = (key <= qpos && key < n) ? __expf(v - rm[r]) * rinv[r] : 0.f;
+        P[row * LQ_PITCH + c] = p;
+      }
+    }
+    __syncthreads();
+    const bool emit = tile >= first;
+    float val;
+    if (threadIdx.x < 128) {
+      // anti-diagonals: element (i, c) belongs to bin kb + c - i + 127; thread u reads P[i][(u+1+i) mod 128]
+      float low = carry, high = 0.f;
+#pragma unroll 8
+      for (int i = 0; i < LQ_ROWS; ++i) {
+        const float p = P[i * LQ_PITCH + ((u + 1 + i) & 127)];
+        if (i <= 126 - u)
+          high += p;  // c = u+1+i > i : bin kb + 128 + u (next tile)
+        else
+          low += p;   // c = u+1+i-128 <= i : bin kb + u
+      }
+      carry = high;
+      val = low * inv_rows;
+      if (emit && kb + u < n) slash_tok[(int64_t)h * n + kb + u] = val;
+    } else {
+      float s = 0.f;
+#pragma unroll 8
+      for (int i = 0; i < LQ_ROWS; ++i) s += P[i * LQ_PITCH + u];
+      val = s * inv_rows;
+      if (emit && kb + u < n) vert_tok[(int64_t)h * n + kb + u] = val;
+    }
+    // block sums (the tile is one 128-token block): wave tree, then two waves per vector in fixed order
+    if (kb + u >= n) val = 0.f;
+    const float ws = sp_wave_sum(val);
+    if (lane == 0) red[wave] = ws;
+    __syncthreads();
+    if (emit && threadIdx.x == 0) slash_blk[(int64_t)h * nb + tile] = red[0] + red[1];
+    if (emit && threadIdx.x == 128) vert_blk[(int64_t)h * nb + tile] = red[2] + red[3];
+    // the next iteration's P writes are ordered after these reads by the barrier above plus the one below
+    __syncthreads();
+  }
+}
+
+// ---- host -------------------------------------------------------------------------------------------------
+static inline int lq_chunks(int64_t n) { return (int)sp_ceil_div(sp_ceil_div(n, LQ_TILE), LQ_STAT_TILES); }
+
+extern "C" size_t sp_lastq_scores_workspace_bytes(int64_t n, int32_t hq, int32_t bs) {
+  (void)bs;
+  if (n <= 0 || hq <= 0) return 0;
+  size_t partial = (size_t)hq * lq_chunks(n) * LQ_ROWS * sizeof(float2);
+  size_t rowstat = (size_t)hq * LQ_ROWS * sizeof(float2);
+  return partial + rowstat;
+}
+
+extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int32_t hq, int32_t hkv, int32_t d,
+                                    int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                                    int32_t bs, uint32_t flags, void* workspace, size_t workspace_bytes,
+                                    float* vert_tok, float* slash_tok, float* vert_blk, float* slash_blk,
+                                    sp_stream_t stream) {
+  SP_REQUIRE(q && k && vert_tok && slash_tok && vert_blk && slash_blk && workspace, SP_ERR_INVALID_ARGUMENT,
+             "sp_lastq_scores_bf16: null pointer");
+  SP_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0, SP_ERR_INVALID_ARGUMENT,
+             "sp_lastq_scores_bf16: hq=%d must be a positive multiple of hkv=%d", hq, hkv);
+  SP_REQUIRE(bs == LQ_ROWS, SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: block size %d unsupported (only 128)", bs);
+  SP_REQUIRE(d == LQ_D, SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: head_dim %d unsupported (only 128)", d);
+  SP_REQUIRE(n >= bs, SP_ERR_INVALID_ARGUMENT, "sp_lastq_scores_bf16: seq_len %lld is shorter than one block",
+             (long long)n);
+  SP_REQUIRE(q_stride_n % 8 == 0 && q_stride_h % 8 == 0 && k_stride_n % 8 == 0 && k_stride_h % 8 == 0 &&
+                 ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0,
+             SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: q/k must be 16-byte aligned with strides multiple of 8");
+  SP_REQUIRE(workspace_bytes >= sp_lastq_scores_workspace_bytes(n, hq, bs), SP_ERR_WORKSPACE,
+             "sp_lastq_scores_bf16: workspace too small");
+  const int n_chunks = lq_chunks(n);
+  const int64_t nb = sp_ceil_div(n, bs);
+  float2* partial = (float2*)workspace;
+  float2* rowstat = partial + (size_t)hq * n_chunks * LQ_ROWS;
+  const float inv_sqrt_d = 1.0f / sqrtf((float)d);
+  const int group = hq / hkv;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(sp_lastq_stats_kernel, dim3(n_chunks, hq), dim3(LQ_THREADS), 0, s, (const sp_bf16*)q,
+                     (const sp_bf16*)k, n, hkv, group, q_stride_n, q_stride_h, k_stride_n, k_stride_h, inv_sqrt_d,
+                     flags, n_chunks, partial);
+  SP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sp_lastq_combine_kernel, dim3(hq), dim3(LQ_ROWS), 0, s, partial, n_chunks, rowstat);
+  SP_LAUNCH_CHECK();
+  const size_t lds_bytes = (LQ_ROWS * LQ_PITCH + 4) * sizeof(float);
+  static bool attr_set = false;
+  if (!attr_set) {
+    SP_HIP(hipFuncSetAttribute((const void*)sp_lastq_probs_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)lds_bytes));
+    attr_set = true;
+  }
+  const int grid_x = (int)sp_ceil_div(nb, LQ_PROB_TILES);
+  hipLaunchKernelGGL(sp_lastq_probs_kernel, dim3(grid_x, hq), dim3(LQ_THREADS), lds_bytes, s, (const sp_bf16*)q,
+                     (const sp_bf16*)k, n, hkv, group, q_stride_n, q_stride_h, k_stride_n, k_stride_h, inv_sqrt_d,
+                     flags, rowstat, vert_tok, slash_tok, vert_blk, slash_blk, nb);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}

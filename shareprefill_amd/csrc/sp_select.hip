@@ -1,0 +1,879 @@
+// Block selection and cross-head pattern sharing on the device, with no host synchronisation.
+// Replaces the torch-op chains of shareprefill/attn/attention_sharing.py:169-364 and :94-103 and the
+// helpers of shareprefill/attn/utils.py:26-128.
+//
+// Canonical arithmetic shared with the CPU oracle:
+//   * order = (value descending, index ascending), compared on the fp32 bit pattern (sp_sort_key);
+//   * cumulative mass = exact integer sums of values truncated to 2^-48 fixed point (sp_to_fixed),
+//     so every comparison against a threshold is independent of summation order (integer atomics
+//     and scans may associate freely).
+// Two primitives:
+//   * radix mass descent for long vectors (per-token vectors of length N, the nb*nb pooled map):
+//     three passes over the data building (count, mass) histograms over 11/11/10 key bits;
+//   * rank sort for short vectors (rows of length nb): rank by pairwise comparison in LDS, scatter to
+//     sorted order, integer prefix scan -- a literal sort / cumsum / threshold.
+#include "sp_common.h"
+
+#define SEL_THREADS 1024
+#define SEL_BINS 2048
+
+// ------------------------------------------------------------------------------------------------
+// radix mass descent (one workgroup of SEL_THREADS threads per vector)
+// ------------------------------------------------------------------------------------------------
+struct MassCut {
+  uint32_t key;        // boundary key k*: every element with key > k* is in the prefix
+  uint32_t n_equal;    // elements with key == k*
+  uint32_t n_take;     // how many of them (lowest indices first) are in the prefix
+  uint32_t n_above;    // elements with key > k*
+  int32_t all;         // 1 when the whole vector is in the prefix
+};
+
+struct SelShared {
+  unsigned long long sum[SEL_BINS];
+  uint32_t cnt[SEL_BINS];
+  unsigned long long sum_above;
+  uint32_t cnt_above;
+  int32_t bin;
+  uint32_t bin_cnt;
+  unsigned long long bin_sum;
+};
+
+// suffix-inclusive scan of sh.sum over SEL_BINS bins (bin b <- sum of bins >= b)
+__device__ static void sel_suffix_scan(SelShared& sh) {
+  const int t = threadIdx.x;
+  for (int off = 1; off < SEL_BINS; off <<= 1) {
+    unsigned long long a0 = 0, a1 = 0;
+    if (t + off < SEL_BINS) a0 = sh.sum[t + off];
+    if (t + SEL_THREADS + off < SEL_BINS) a1 = sh.sum[t + SEL_THREADS + off];
+    __syncthreads();
+    sh.sum[t] += a0;
+    sh.sum[t + SEL_THREADS] += a1;
+    __syncthreads();
+  }
+}
+
+// One descent level: histogram the elements whose key matches `prefix` on the bits above
+// (shift+width), pick the bin in which the running mass (high keys first) first exceeds `budget`.
+// Returns false when no bin crosses (only possible at the top level).
+__device__ static bool sel_level(const float* __restrict__ x, int64_t len, uint32_t prefix, int prefix_shift,
+                                 int shift, int width, unsigned long long budget, SelShared& sh) {
+  const int t = threadIdx.x;
+  sh.sum[t] = 0;
+  sh.sum[t + SEL_THREADS] = 0;
+  sh.cnt[t] = 0;
+  sh.cnt[t + SEL_THREADS] = 0;
+  if (t == 0) {
+    sh.bin = -1;
+    sh.cnt_above = 0;
+  }
+  __syncthreads();
+  const uint32_t maskw = (1u << width) - 1u;
+  for (int64_t i = t; i < len; i += SEL_THREADS) {
+    const float v = x[i];
+    const uint32_t key = sp_sort_key(v);
+    if (prefix_shift < 32 && (key >> prefix_shift) != prefix) continue;
+    const uint32_t b = (key >> shift) & maskw;
+    atomicAdd(&sh.cnt[b], 1u);
+    const unsigned long long fx = sp_to_fixed(v);
+    if (fx) atomicAdd(&sh.sum[b], fx);
+  }
+  __syncthreads();
+  // keep the per-bin mass of the candidate bins before the scan overwrites it
+  const unsigned long long own0 = sh.sum[t], own1 = sh.sum[t + SEL_THREADS];
+  __syncthreads();
+  sel_suffix_scan(sh);
+  const int nbins = 1 << width;
+#pragma unroll
+  for (int rep = 0; rep < 2; ++rep) {
+    const int b = t + rep * SEL_THREADS;
+    if (b < nbins) {
+      const unsigned long long incl = sh.sum[b];
+      const unsigned long long excl = (b + 1 < SEL_BINS) ? sh.sum[b + 1] : 0ull;
+      if (incl > budget && excl <= budget) {
+        sh.bin = b;
+        sh.sum_above = excl;
+        sh.bin_sum = rep ? own1 : own0;
+        sh.bin_cnt = sh.cnt[b];
+      }
+    }
+  }
+  __syncthreads();
+  const int bin = sh.bin;
+  if (bin < 0) return false;
+  // count of the bins above the chosen one
+  uint32_t c = 0;
+#pragma unroll
+  for (int rep = 0; rep < 2; ++rep) {
+    const int b = t + rep * SEL_THREADS;
+    if (b < nbins && b > bin) c += sh.cnt[b];
+  }
+  if (c) atomicAdd(&sh.cnt_above, c);
+  __syncthreads();
+  return true;
+}
+
+// prefix of sort_desc(x) whose running mass stays <= budget
+__device__ static MassCut sel_mass_cut(const float* __restrict__ x, int64_t len, unsigned long long budget,
+                                       SelShared& sh) {
+  MassCut cut;
+  cut.all = 0;
+  if (!sel_level(x, len, 0u, 32, 21, 11, budget, sh)) {
+    cut.all = 1;
+    cut.key = 0;
+    cut.n_equal = 0;
+    cut.n_take = 0;
+    cut.n_above = (uint32_t)len;
+    return cut;
+  }
+  uint32_t prefix = (uint32_t)sh.bin;
+  uint32_t above = sh.cnt_above;
+  unsigned long long rem = budget - sh.sum_above;
+  __syncthreads();
+  sel_level(x, len, prefix, 21, 10, 11, rem, sh);
+  prefix = (prefix << 11) | (uint32_t)sh.bin;
+  above += sh.cnt_above;
+  rem -= sh.sum_above;
+  __syncthreads();
+  sel_level(x, len, prefix, 10, 0, 10, rem, sh);
+  cut.key = (prefix << 10) | (uint32_t)sh.bin;
+  above += sh.cnt_above;
+  rem -= sh.sum_above;
+  cut.n_equal = sh.bin_cnt;
+  cut.n_above = above;
+  const unsigned long long each = sh.bin_sum / (sh.bin_cnt ? sh.bin_cnt : 1u);
+  unsigned long long take = each ? rem / each : (unsigned long long)cut.n_equal;
+  if (take > cut.n_equal) take = cut.n_equal;
+  cut.n_take = (uint32_t)take;
+  __syncthreads();
+  return cut;
+}
+
+// ---- score_cover_topk (attn/utils.py:47-50) ---------------------------------------------------------
+__global__ __launch_bounds__(SEL_THREADS) void sp_cover_count_kernel(const float* __restrict__ x, int64_t len,
+                                                                     long long t_le, int32_t* __restrict__ out,
+                                                                     int bs, int minb, int maxb) {
+  __shared__ SelShared sh;
+  const float* v = x + (int64_t)blockIdx.x * len;
+  long long m = 0;
+  if (t_le >= 0) {
+    MassCut cut = sel_mass_cut(v, len, (unsigned long long)t_le, sh);
+    m = cut.all ? (long long)len : (long long)cut.n_above + cut.n_take;
+  }
+  if (threadIdx.x == 0) {
+    long long r = m + 1;
+    if (bs > 0) {  // budgets: tokens // bs + 1, clamped (attention_sharing.py:169-176)
+      r = r / bs + 1;
+      if (r < minb) r = minb;
+      if (r > maxb) r = maxb;
+    }
+    out[blockIdx.x] = (int32_t)r;
+  }
+}
+
+extern "C" int sp_cover_count(const float* x, int32_t n_vec, int64_t len, float thr, int32_t* out,
+                              sp_stream_t stream) {
+  SP_REQUIRE(x && out && n_vec > 0 && len > 0, SP_ERR_INVALID_ARGUMENT, "sp_cover_count: bad arguments");
+  hipLaunchKernelGGL(sp_cover_count_kernel, dim3(n_vec), dim3(SEL_THREADS), 0, (hipStream_t)stream, x, len,
+                     (long long)sp_thr_le(thr), out, 0, 0, 0);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_cover_budgets(const float* vert_tok, const float* slash_tok, int32_t hq, int64_t n, int32_t bs,
+                                float pattern_threshold, int32_t min_blocks, int32_t max_blocks, int32_t* nv,
+                                int32_t* ns, sp_stream_t stream) {
+  SP_REQUIRE(vert_tok && slash_tok && nv && ns && hq > 0 && n > 0 && bs > 0, SP_ERR_INVALID_ARGUMENT,
+             "sp_cover_budgets: bad arguments");
+  const long long t = (long long)sp_thr_le(pattern_threshold);
+  hipLaunchKernelGGL(sp_cover_count_kernel, dim3(hq), dim3(SEL_THREADS), 0, (hipStream_t)stream, vert_tok, n, t, nv,
+                     bs, min_blocks, max_blocks);
+  SP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sp_cover_count_kernel, dim3(hq), dim3(SEL_THREADS), 0, (hipStream_t)stream, slash_tok, n, t, ns,
+                     bs, min_blocks, max_blocks);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+// ---- score_cover_idx (attn/utils.py:53-57) on [nb][nb] maps, written into bit masks -----------------
+__global__ __launch_bounds__(SEL_THREADS) void sp_cover_select_global_kernel(
+    const float* __restrict__ x, const int32_t* __restrict__ enable, int enable_match, int nb, int nbw,
+    long long t_le, uint64_t* __restrict__ mask) {
+  __shared__ SelShared sh;
+  __shared__ uint32_t wave_cnt[SEL_THREADS / SP_WAVE];
+  __shared__ uint32_t running;
+  const int v = blockIdx.x;
+  if (enable) {
+    const int e = enable[v];
+    if (enable_match < 0 ? (e == 0) : (e != enable_match)) return;
+  }
+  const int64_t len = (int64_t)nb * nb;
+  const float* xv = x + (int64_t)v * len;
+  uint32_t* mv = reinterpret_cast<uint32_t*>(mask + (int64_t)v * nb * nbw);
+  if (threadIdx.x == 0) atomicOr(&mv[0], 1u);  // block (0,0): the padding id of the reference
+  if (t_le < 0) return;
+  MassCut cut = sel_mass_cut(xv, len, (unsigned long long)t_le, sh);
+  const bool ranked = !cut.all && cut.n_take > 0 && cut.n_take < cut.n_equal;
+  if (threadIdx.x == 0) running = 0;
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int64_t base = 0; base < len; base += SEL_THREADS) {
+    const int64_t i = base + threadIdx.x;
+    bool sel = false;
+    bool eq = false;
+    int r = 0, c = 0;
+    if (i < len) {
+      r = (int)(i / nb);
+      c = (int)(i - (int64_t)r * nb);
+      const uint32_t key = sp_sort_key(xv[i]);
+      if (cut.all || key > cut.key)
+        sel = true;
+      else if (key == cut.key) {
+        if (cut.n_take >= cut.n_equal)
+          sel = true;
+        else
+          eq = cut.n_take > 0;
+      }
+    }
+    if (ranked) {  // ties at the boundary: the n_take lowest indices win
+      const unsigned long long bal = __ballot(eq);
+      const uint32_t before = __popcll(bal & ((1ull << lane) - 1ull));
+      if (lane == 0) wave_cnt[wave] = __popcll(bal);
+      __syncthreads();
+      uint32_t off = running;
+      for (int w = 0; w < wave; ++w) off += wave_cnt[w];
+      if (eq && off + before < cut.n_take) sel = true;
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        uint32_t tot = 0;
+        for (int w = 0; w < SEL_THREADS / SP_WAVE; ++w) tot += wave_cnt[w];
+        running += tot;
+      }
+      __syncthreads();
+    }
+    if (sel && c <= r) atomicOr(&mv[((int64_t)r * nbw + (c >> 6)) * 2 + ((c >> 5) & 1)], 1u << (c & 31));
+  }
+}
+
+extern "C" int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec, int32_t nb, float score,
+                                      uint64_t* mask, sp_stream_t stream) {
+  SP_REQUIRE(x && mask && n_vec > 0 && nb > 0, SP_ERR_INVALID_ARGUMENT, "sp_cover_select_global: bad arguments");
+  const int nbw = (nb + 63) / 64;
+  hipLaunchKernelGGL(sp_cover_select_global_kernel, dim3(n_vec), dim3(SEL_THREADS), 0, (hipStream_t)stream, x, enable,
+                     -1, nb, nbw, (long long)sp_thr_le(score), mask);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// rank sort for short vectors (length <= RS_MAX), one workgroup of RS_THREADS threads
+// ------------------------------------------------------------------------------------------------
+#define RS_THREADS 256
+#define RS_MAX 4096
+
+// rank[i] = position of element i in (key desc, index asc) order; keys[] in LDS
+__device__ static void rs_ranks(const uint32_t* keys, int n, uint16_t* rank) {
+  for (int i = threadIdx.x; i < n; i += RS_THREADS) {
+    const uint32_t ki = keys[i];
+    int r = 0;
+    for (int j = 0; j < n; ++j) {
+      const uint32_t kj = keys[j];
+      r += (kj > ki) || (kj == ki && j < i);
+    }
+    rank[i] = (uint16_t)r;
+  }
+}
+
+// ---- score_cover_idx_each_row (attn/utils.py:60-76) -------------------------------------------------
+// keep[r] = first (count(cumsum < thr) + 1) entries of the sorted row, or exactly one if thr is never reached
+struct RowShared {
+  uint32_t keys[RS_MAX];
+  uint16_t rank[RS_MAX];
+  unsigned long long sorted_fx[RS_MAX];
+  unsigned long long chunk_sum[RS_THREADS];
+  uint32_t below;
+};
+
+__device__ static int rs_row_keep(const float* __restrict__ row, int n, long long t_lt, RowShared& sh) {
+  for (int i = threadIdx.x; i < n; i += RS_THREADS) sh.keys[i] = sp_sort_key(row[i]);
+  if (threadIdx.x == 0) sh.below = 0;
+  __syncthreads();
+  rs_ranks(sh.keys, n, sh.rank);
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += RS_THREADS) sh.sorted_fx[sh.rank[i]] = sp_to_fixed(row[i]);
+  __syncthreads();
+  // inclusive scan of sorted_fx in contiguous per-thread chunks
+  const int per = (n + RS_THREADS - 1) / RS_THREADS;
+  const int lo = threadIdx.x * per, hi = min(lo + per, n);
+  unsigned long long s = 0;
+  for (int i = lo; i < hi; ++i) s += sh.sorted_fx[i];
+  sh.chunk_sum[threadIdx.x] = s;
+  __syncthreads();
+  unsigned long long off = 0;
+  for (int t = 0; t < (int)threadIdx.x; ++t) off += sh.chunk_sum[t];
+  uint32_t cnt = 0;
+  if (t_lt >= 0) {
+    for (int i = lo; i < hi; ++i) {
+      off += sh.sorted_fx[i];
+      cnt += (off <= (unsigned long long)t_lt);
+    }
+  }
+  if (cnt) atomicAdd(&sh.below, cnt);
+  __syncthreads();
+  const int c = (int)sh.below;
+  return c < n ? c + 1 : 1;
+}
+
+__global__ __launch_bounds__(RS_THREADS) void sp_cover_select_rows_kernel(const float* __restrict__ x, int nb, int nbw,
+                                                                          long long t_lt,
+                                                                          uint64_t* __restrict__ pattern) {
+  __shared__ RowShared sh;
+  const int r = blockIdx.x;
+  const int keep = rs_row_keep(x + (int64_t)r * nb, nb, t_lt, sh);
+  uint32_t* prow = reinterpret_cast<uint32_t*>(pattern + (int64_t)r * nbw);
+  for (int w = threadIdx.x; w < nbw * 2; w += RS_THREADS) {
+    uint32_t bits = 0;
+    for (int b = 0; b < 32; ++b) {
+      const int c = w * 32 + b;
+      if (c < nb && c <= r && sh.rank[c] < keep) bits |= 1u << b;
+    }
+    if (r == 0 && w == 0) bits |= 1u;
+    prow[w] = bits;
+  }
+}
+
+extern "C" int sp_cover_select_rows(const float* x, int32_t nb, float thr, uint64_t* pattern, sp_stream_t stream) {
+  SP_REQUIRE(x && pattern && nb > 0, SP_ERR_INVALID_ARGUMENT, "sp_cover_select_rows: bad arguments");
+  SP_REQUIRE(nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_cover_select_rows: nb=%d exceeds %d", nb, RS_MAX);
+  hipLaunchKernelGGL(sp_cover_select_rows_kernel, dim3(nb), dim3(RS_THREADS), 0, (hipStream_t)stream, x, nb,
+                     (nb + 63) / 64, (long long)sp_thr_lt(thr), pattern);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// sqrt Jensen-Shannon divergence (attn/utils.py:26-30), one wave, fixed summation order
+// ------------------------------------------------------------------------------------------------
+__device__ static float wave_sqrt_js(const float* __restrict__ p, const float* __restrict__ q, int n, int lane) {
+  float sp = 0.f, sq = 0.f;
+  for (int i = lane; i < n; i += SP_WAVE) {
+    const float a = p[i], b = q[i];
+    const float m = (a + b) / 2.f;
+    sp += a * logf(a / m);
+    sq += b * logf(b / m);
+  }
+  sp = sp_wave_sum(sp);
+  sq = sp_wave_sum(sq);
+  return sqrtf(0.5f * sp + 0.5f * sq);
+}
+
+// ------------------------------------------------------------------------------------------------
+// query-aware test (attention_sharing.py:193-202)
+// ------------------------------------------------------------------------------------------------
+#define QA_THREADS 256
+__global__ __launch_bounds__(QA_THREADS) void sp_queryaware_test_kernel(
+    const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ kbar, const float* __restrict__ vert_blk, int64_t n,
+    int hq, int hkv, int d, int64_t sq_n, int64_t sq_h, int bs, int nb, uint32_t flags, float inv_sqrt_d, float thr,
+    float* __restrict__ avg_qk, float* __restrict__ js_qa, int32_t* __restrict__ use_qa) {
+  extern __shared__ float qa_lds[];
+  float* qmean = qa_lds;       // [d]
+  float* logit = qa_lds + d;   // [nb]
+  __shared__ float red[QA_THREADS / SP_WAVE];
+  __shared__ float bcast;
+  const int h = blockIdx.x;
+  const int kvh = h / (hq / hkv);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // mean over the last bs queries of bf16(q / sqrt(d)), rounded to bf16 (last_q.mean(1), :197-199)
+  for (int c = threadIdx.x; c < d; c += QA_THREADS) {
+    const sp_bf16* src = q + (int64_t)h * sq_h + (n - bs) * sq_n + c;
+    float s = 0.f;
+    for (int i = 0; i < bs; ++i) s += sp_round_bf16(sp_bf16_to_f32(src[(int64_t)i * sq_n]) * inv_sqrt_d);
+    qmean[c] = sp_round_bf16(s / (float)bs);
+  }
+  __syncthreads();
+  float lmax = -INFINITY;
+  for (int b = threadIdx.x; b < nb; b += QA_THREADS) {
+    const sp_bf16* kr = kbar + ((int64_t)b * hkv + kvh) * d;
+    float s = 0.f;
+    for (int c = 0; c < d; c += 8) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(kr + c);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s += qmean[c + 2 * j] * __uint_as_float(w[j] << 16);
+        s += qmean[c + 2 * j + 1] * __uint_as_float(w[j] & 0xffff0000u);
+      }
+    }
+    if (flags & SP_FLAG_LOGITS_BF16) s = sp_round_bf16(s);
+    logit[b] = s;
+    lmax = fmaxf(lmax, s);
+  }
+  lmax = sp_wave_max(lmax);
+  if (lane == 0) red[wave] = lmax;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = red[0];
+    for (int w = 1; w < QA_THREADS / SP_WAVE; ++w) m = fmaxf(m, red[w]);
+    bcast = m;
+  }
+  __syncthreads();
+  const float gmax = bcast;
+  float lsum = 0.f;
+  for (int b = threadIdx.x; b < nb; b += QA_THREADS) {
+    const float e = expf(logit[b] - gmax);
+    logit[b] = e;
+    lsum += e;
+  }
+  lsum = sp_wave_sum(lsum);
+  __syncthreads();
+  if (lane == 0) red[wave] = lsum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+    for (int w = 0; w < QA_THREADS / SP_WAVE; ++w) s += red[w];
+    bcast = s;
+  }
+  __syncthreads();
+  const float gsum = bcast;
+  for (int b = threadIdx.x; b < nb; b += QA_THREADS) {
+    const float p = logit[b] / gsum;
+    logit[b] = p;
+    avg_qk[(int64_t)h * nb + b] = p;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    const float js = wave_sqrt_js(logit, vert_blk + (int64_t)h * nb, nb, lane);
+    if (lane == 0) {
+      js_qa[h] = js;
+      use_qa[h] = (js < thr) ? 1 : 0;  // NaN compares false
+    }
+  }
+}
+
+extern "C" int sp_queryaware_test_bf16(const void* q, const void* kbar, const float* vert_blk, int64_t n, int32_t hq,
+                                       int32_t hkv, int32_t d, int64_t q_stride_n, int64_t q_stride_h, int32_t bs,
+                                       uint32_t flags, float queryaware_threshold, float* avg_qk, float* js_qa,
+                                       int32_t* use_qa, sp_stream_t stream) {
+  SP_REQUIRE(q && kbar && vert_blk && avg_qk && js_qa && use_qa, SP_ERR_INVALID_ARGUMENT,
+             "sp_queryaware_test_bf16: null pointer");
+  SP_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0 && d % 8 == 0 && n >= bs && bs > 0, SP_ERR_INVALID_ARGUMENT,
+             "sp_queryaware_test_bf16: bad shape");
+  const int nb = (int)sp_ceil_div(n, bs);
+  const size_t lds = (size_t)(d + nb) * sizeof(float);
+  SP_REQUIRE(lds <= 60000, SP_ERR_UNSUPPORTED, "sp_queryaware_test_bf16: nb=%d too large", nb);
+  hipLaunchKernelGGL(sp_queryaware_test_kernel, dim3(hq), dim3(QA_THREADS), lds, (hipStream_t)stream,
+                     (const sp_bf16*)q, (const sp_bf16*)kbar, vert_blk, n, hq, hkv, d, q_stride_n, q_stride_h, bs, nb,
+                     flags, 1.0f / sqrtf((float)d), queryaware_threshold, avg_qk, js_qa, use_qa);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// top-k sets of the pooled vertical / slash vectors (attention_sharing.py:231-251, :303-329)
+// cols[c] = 1 for the nv best columns (column 0 forced), dists[dd] = 1 for the ns best distances
+// (distance 0 forced); slash index i holds distance nb-1-i.
+// ------------------------------------------------------------------------------------------------
+__device__ static void vs_sets(const float* __restrict__ vert, const float* __restrict__ slash, int nb, int nv,
+                               int ns, uint32_t* keys /* LDS [nb] */, uint8_t* cols, uint8_t* dists, int nthreads) {
+  const uint32_t inf_key = 0x7f800000u;
+  for (int i = threadIdx.x; i < nb; i += nthreads) keys[i] = (i == 0) ? inf_key : sp_sort_key(vert[i]);
+  __syncthreads();
+  for (int i = threadIdx.x; i < nb; i += nthreads) {
+    const uint32_t ki = keys[i];
+    int r = 0;
+    for (int j = 0; j < nb; ++j) r += (keys[j] > ki) || (keys[j] == ki && j < i);
+    cols[i] = r < nv;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < nb; i += nthreads) keys[i] = (i == nb - 1) ? inf_key : sp_sort_key(slash[i]);
+  __syncthreads();
+  for (int i = threadIdx.x; i < nb; i += nthreads) {
+    const uint32_t ki = keys[i];
+    int r = 0;
+    for (int j = 0; j < nb; ++j) r += (keys[j] > ki) || (keys[j] == ki && j < i);
+    dists[nb - 1 - i] = r < ns;
+  }
+  __syncthreads();
+}
+
+// ------------------------------------------------------------------------------------------------
+// pivot election / share test (attention_sharing.py:204-301), single workgroup
+// ------------------------------------------------------------------------------------------------
+#define DEC_THREADS 256
+#define DEC_MAX_HEADS 256
+__global__ __launch_bounds__(DEC_THREADS) void sp_share_decide_kernel(
+    sp_cluster_state st, const int32_t* __restrict__ head_cluster, int layer_idx, int hq,
+    const float* __restrict__ vert_blk, const float* __restrict__ slash_blk, const int32_t* __restrict__ use_qa,
+    const int32_t* __restrict__ nv, const int32_t* __restrict__ ns, int minb, float sim_thr, double fb_thr,
+    int32_t* __restrict__ decision, float* __restrict__ js_v, float* __restrict__ js_s, int32_t* __restrict__ nv_f,
+    int32_t* __restrict__ ns_f) {
+  __shared__ float s_jv[DEC_MAX_HEADS], s_js[DEC_MAX_HEADS];
+  __shared__ int32_t s_new[DEC_MAX_HEADS];
+  __shared__ uint32_t s_keys[RS_MAX];
+  const int nb = st.nb;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // similarity of every candidate head against its cluster's stored pivot (pivots of EARLIER layers only)
+  for (int h = wave; h < hq; h += DEC_THREADS / SP_WAVE) {
+    float jv = NAN, js = NAN;
+    const int c = head_cluster[h];
+    if (c >= 0 && !use_qa[h] && st.info[c * 8 + 0] >= 0 && st.info[c * 8 + 1] != 0) {
+      jv = wave_sqrt_js(st.vert + (int64_t)c * nb, vert_blk + (int64_t)h * nb, nb, lane);
+      js = wave_sqrt_js(st.slash + (int64_t)c * nb, slash_blk + (int64_t)h * nb, nb, lane);
+    }
+    if (lane == 0) {
+      s_jv[h] = jv;
+      s_js[h] = js;
+      js_v[h] = jv;
+      js_s[h] = js;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int h = 0; h < hq; ++h) {
+      int dec = SP_DEC_VS;
+      s_new[h] = 0;
+      if (use_qa[h]) {
+        dec = SP_DEC_QA;
+      } else {
+        const int c = head_cluster[h];
+        if (c >= 0) {
+          if (st.info[c * 8 + 0] < 0) {
+            st.info[c * 8 + 0] = h;
+            st.info[c * 8 + 2] = nv[h];
+            st.info[c * 8 + 3] = ns[h];
+            st.info[c * 8 + 4] = layer_idx;
+            dec = SP_DEC_DENSE;
+            s_new[h] = 1;
+          } else if (st.info[c * 8 + 1] != 0) {
+            if (s_jv[h] < sim_thr && s_js[h] < sim_thr && st.ratio[c] < fb_thr) dec = SP_DEC_SHARE;
+          }
+        }
+      }
+      decision[h] = dec;
+      const bool reset = (dec == SP_DEC_QA || dec == SP_DEC_SHARE);
+      nv_f[h] = reset ? minb : nv[h];
+      ns_f[h] = reset ? minb : ns[h];
+    }
+  }
+  __syncthreads();
+  // newly elected pivots keep their pooled vectors and their own vertical-slash sets (:223-263)
+  for (int h = 0; h < hq; ++h) {
+    if (!s_new[h]) continue;
+    const int c = head_cluster[h];
+    for (int i = threadIdx.x; i < nb; i += DEC_THREADS) {
+      st.vert[(int64_t)c * nb + i] = vert_blk[(int64_t)h * nb + i];
+      st.slash[(int64_t)c * nb + i] = slash_blk[(int64_t)h * nb + i];
+    }
+    vs_sets(vert_blk + (int64_t)h * nb, slash_blk + (int64_t)h * nb, nb, nv[h], ns[h], s_keys,
+            st.cols + (int64_t)c * nb, st.dists + (int64_t)c * nb, DEC_THREADS);
+  }
+}
+
+static int check_state(const sp_cluster_state* st, int nb, const char* who) {
+  SP_REQUIRE(st != nullptr, SP_ERR_INVALID_ARGUMENT, "%s: null cluster state", who);
+  SP_REQUIRE(st->n_clusters >= 0 && st->nb == nb && st->nbw == (nb + 63) / 64, SP_ERR_INVALID_ARGUMENT,
+             "%s: cluster state sized for nb=%d, call uses nb=%d", who, st->nb, nb);
+  if (st->n_clusters > 0) {
+    SP_REQUIRE(st->info && st->ratio && st->vert && st->slash && st->cols && st->dists && st->pattern && st->accum,
+               SP_ERR_INVALID_ARGUMENT, "%s: cluster state has null slabs", who);
+  }
+  return SP_OK;
+}
+
+extern "C" int sp_share_decide(const sp_cluster_state* state, const int32_t* head_cluster, int32_t layer_idx,
+                               int32_t hq, const float* vert_blk, const float* slash_blk, const int32_t* use_qa,
+                               const int32_t* nv, const int32_t* ns, int32_t min_blocks, float similarity_threshold,
+                               double fallback_threshold, int32_t* decision, float* js_v, float* js_s,
+                               int32_t* nv_final, int32_t* ns_final, sp_stream_t stream) {
+  SP_REQUIRE(state, SP_ERR_INVALID_ARGUMENT, "sp_share_decide: null cluster state");
+  int rc = check_state(state, state->nb, "sp_share_decide");
+  if (rc) return rc;
+  SP_REQUIRE(head_cluster && vert_blk && slash_blk && use_qa && nv && ns && decision && js_v && js_s && nv_final &&
+                 ns_final,
+             SP_ERR_INVALID_ARGUMENT, "sp_share_decide: null pointer");
+  SP_REQUIRE(hq > 0 && hq <= DEC_MAX_HEADS, SP_ERR_UNSUPPORTED, "sp_share_decide: hq=%d unsupported (max %d)", hq,
+             DEC_MAX_HEADS);
+  SP_REQUIRE(state->nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_share_decide: nb=%d exceeds %d", state->nb, RS_MAX);
+  hipLaunchKernelGGL(sp_share_decide_kernel, dim3(1), dim3(DEC_THREADS), 0, (hipStream_t)stream, *state, head_cluster,
+                     layer_idx, hq, vert_blk, slash_blk, use_qa, nv, ns, min_blocks, similarity_threshold,
+                     fallback_threshold, decision, js_v, js_s, nv_final, ns_final);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// mask construction (attention_sharing.py:303-337 and attn/utils.py:99-128 as a set)
+// ------------------------------------------------------------------------------------------------
+#define MASK_THREADS 256
+__global__ __launch_bounds__(MASK_THREADS) void sp_build_mask_kernel(
+    sp_cluster_state st, const int32_t* __restrict__ head_cluster, const int32_t* __restrict__ decision,
+    const float* __restrict__ vert_blk, const float* __restrict__ slash_blk, const int32_t* __restrict__ nv_f,
+    const int32_t* __restrict__ ns_f, int nb, int nbw, uint64_t* __restrict__ mask) {
+  __shared__ uint32_t s_keys[RS_MAX];
+  __shared__ uint8_t s_cols[RS_MAX], s_dists[RS_MAX];
+  const int h = blockIdx.x;
+  const int dec = decision[h];
+  vs_sets(vert_blk + (int64_t)h * nb, slash_blk + (int64_t)h * nb, nb, nv_f[h], ns_f[h], s_keys, s_cols, s_dists,
+          MASK_THREADS);
+  const uint64_t* pat = nullptr;
+  if (dec == SP_DEC_SHARE) pat = st.pattern + (int64_t)head_cluster[h] * nb * nbw;
+  uint64_t* mh = mask + (int64_t)h * nb * nbw;
+  for (int idx = threadIdx.x; idx < nb * nbw; idx += MASK_THREADS) {
+    const int r = idx / nbw, w = idx - r * nbw;
+    uint64_t bits = 0;
+    const int c0 = w * 64;
+    const int cend = min(c0 + 64, r + 1);
+    if (dec == SP_DEC_DENSE) {
+      for (int c = c0; c < cend; ++c) bits |= 1ull << (c - c0);
+    } else {
+      for (int c = c0; c < cend; ++c) {
+        if (s_cols[c] | s_dists[r - c]) bits |= 1ull << (c - c0);
+      }
+      if (pat) bits |= pat[idx];
+    }
+    if (idx == 0) bits |= 1ull;
+    mh[idx] = bits;
+  }
+}
+
+extern "C" int sp_build_mask(const sp_cluster_state* state, const int32_t* head_cluster, const int32_t* decision,
+                             const float* vert_blk, const float* slash_blk, const int32_t* nv_final,
+                             const int32_t* ns_final, int32_t hq, int32_t nb, uint64_t* mask, sp_stream_t stream) {
+  int rc = check_state(state, nb, "sp_build_mask");
+  if (rc) return rc;
+  SP_REQUIRE(head_cluster && decision && vert_blk && slash_blk && nv_final && ns_final && mask,
+             SP_ERR_INVALID_ARGUMENT, "sp_build_mask: null pointer");
+  SP_REQUIRE(hq > 0 && nb > 0 && nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_build_mask: nb=%d unsupported (max %d)", nb,
+             RS_MAX);
+  hipLaunchKernelGGL(sp_build_mask_kernel, dim3(hq), dim3(MASK_THREADS), 0, (hipStream_t)stream, *state, head_cluster,
+                     decision, vert_blk, slash_blk, nv_final, ns_final, nb, (nb + 63) / 64, mask);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// query-aware heads: pooled block probabilities (attention_sharing.py:350-360)
+// ------------------------------------------------------------------------------------------------
+#define BP_THREADS 256
+__global__ __launch_bounds__(BP_THREADS) void sp_block_probs_kernel(
+    const sp_bf16* __restrict__ qbar, const sp_bf16* __restrict__ kbar, const int32_t* __restrict__ decision, int hq,
+    int hkv, int d, int nb, uint32_t flags, float inv_sqrt_d, float* __restrict__ probs) {
+  extern __shared__ float bp_lds[];
+  float* qs = bp_lds;          // [d]
+  float* logit = bp_lds + d;   // [nb]
+  __shared__ float red[BP_THREADS / SP_WAVE];
+  __shared__ float bcast;
+  const int r = blockIdx.x, h = blockIdx.y;
+  if (decision[h] != SP_DEC_QA) return;
+  const int kvh = h / (hq / hkv);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int c = threadIdx.x; c < d; c += BP_THREADS)
+    qs[c] = sp_round_bf16(sp_bf16_to_f32(qbar[((int64_t)r * hq + h) * d + c]) * inv_sqrt_d);
+  __syncthreads();
+  float lmax = -INFINITY;
+  for (int b = threadIdx.x; b <= r; b += BP_THREADS) {
+    const sp_bf16* kr = kbar + ((int64_t)b * hkv + kvh) * d;
+    float s = 0.f;
+    for (int c = 0; c < d; c += 8) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(kr + c);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s += qs[c + 2 * j] * __uint_as_float(w[j] << 16);
+        s += qs[c + 2 * j + 1] * __uint_as_float(w[j] & 0xffff0000u);
+      }
+    }
+    if (flags & SP_FLAG_LOGITS_BF16) s = sp_round_bf16(s);
+    logit[b] = s;
+    lmax = fmaxf(lmax, s);
+  }
+  lmax = sp_wave_max(lmax);
+  if (lane == 0) red[wave] = lmax;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = red[0];
+    for (int w = 1; w < BP_THREADS / SP_WAVE; ++w) m = fmaxf(m, red[w]);
+    bcast = m;
+  }
+  __syncthreads();
+  const float gmax = bcast;
+  float lsum = 0.f;
+  for (int b = threadIdx.x; b <= r; b += BP_THREADS) {
+    const float e = expf(logit[b] - gmax);
+    logit[b] = e;
+    lsum += e;
+  }
+  lsum = sp_wave_sum(lsum);
+  __syncthreads();
+  if (lane == 0) red[wave] = lsum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+    for (int w = 0; w < BP_THREADS / SP_WAVE; ++w) s += red[w];
+    bcast = s;
+  }
+  __syncthreads();
+  const float gsum = bcast;
+  float* out = probs + ((int64_t)h * nb + r) * nb;
+  for (int b = threadIdx.x; b < nb; b += BP_THREADS) out[b] = (b <= r) ? logit[b] / gsum : 0.f;
+}
+
+extern "C" int sp_queryaware_select_bf16(const void* qbar, const void* kbar, const int32_t* decision, int32_t hq,
+                                         int32_t hkv, int32_t d, int32_t nb, uint32_t flags, float pattern_threshold,
+                                         float* probs, uint64_t* mask, sp_stream_t stream) {
+  SP_REQUIRE(qbar && kbar && decision && probs && mask, SP_ERR_INVALID_ARGUMENT,
+             "sp_queryaware_select_bf16: null pointer");
+  SP_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0 && d % 8 == 0 && nb > 0, SP_ERR_INVALID_ARGUMENT,
+             "sp_queryaware_select_bf16: bad shape");
+  const size_t lds = (size_t)(d + nb) * sizeof(float);
+  SP_REQUIRE(lds <= 60000, SP_ERR_UNSUPPORTED, "sp_queryaware_select_bf16: nb=%d too large", nb);
+  hipLaunchKernelGGL(sp_block_probs_kernel, dim3(nb, hq), dim3(BP_THREADS), lds, (hipStream_t)stream,
+                     (const sp_bf16*)qbar, (const sp_bf16*)kbar, decision, hq, hkv, d, nb, flags,
+                     1.0f / sqrtf((float)d), probs);
+  SP_LAUNCH_CHECK();
+  // score = pattern_threshold * nb evaluated in double, then taken to fp32 as a tensor comparison would
+  const float score = (float)((double)pattern_threshold * (double)nb);
+  hipLaunchKernelGGL(sp_cover_select_global_kernel, dim3(hq), dim3(SEL_THREADS), 0, (hipStream_t)stream, probs,
+                     decision, SP_DEC_QA, nb, (nb + 63) / 64, (long long)sp_thr_le(score), mask);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// pivot state update (attention_sharing.py:94-103 and the vs_ratio of :278-286, computed eagerly)
+// ------------------------------------------------------------------------------------------------
+struct PivotRowShared {
+  RowShared row;
+  unsigned long long cov, tot;
+};
+
+__global__ __launch_bounds__(RS_THREADS) void sp_pivot_rows_kernel(sp_cluster_state st,
+                                                                   const int32_t* __restrict__ head_cluster,
+                                                                   const int32_t* __restrict__ decision,
+                                                                   const float* __restrict__ avg_attn, int nb,
+                                                                   int nbw, long long t_lt,
+                                                                   unsigned long long* __restrict__ accum) {
+  __shared__ PivotRowShared sh;
+  const int r = blockIdx.x, h = blockIdx.y;
+  if (decision[h] != SP_DEC_DENSE) return;
+  const int c = head_cluster[h];
+  const float* row = avg_attn + ((int64_t)h * nb + r) * nb;
+  const int keep = rs_row_keep(row, nb, t_lt, sh.row);
+  uint32_t* prow = reinterpret_cast<uint32_t*>(st.pattern + ((int64_t)c * nb + r) * nbw);
+  for (int w = threadIdx.x; w < nbw * 2; w += RS_THREADS) {
+    uint32_t bits = 0;
+    for (int b = 0; b < 32; ++b) {
+      const int col = w * 32 + b;
+      if (col < nb && col <= r && sh.row.rank[col] < keep) bits |= 1u << b;
+    }
+    if (r == 0 && w == 0) bits |= 1u;
+    prow[w] = bits;
+  }
+  // vs_ratio pieces: mass under the pivot's own vertical / slash sets (a block in both counts twice) and the total
+  if (threadIdx.x == 0) {
+    sh.cov = 0;
+    sh.tot = 0;
+  }
+  __syncthreads();
+  const uint8_t* cols = st.cols + (int64_t)c * nb;
+  const uint8_t* dists = st.dists + (int64_t)c * nb;
+  unsigned long long cov = 0, tot = 0;
+  for (int col = threadIdx.x; col < nb; col += RS_THREADS) {
+    const unsigned long long fx = sp_to_fixed(row[col]);
+    tot += fx;
+    if (col <= r) cov += fx * (unsigned long long)((cols[col] ? 1 : 0) + (dists[r - col] ? 1 : 0));
+  }
+  if (cov) atomicAdd(&sh.cov, cov);
+  if (tot) atomicAdd(&sh.tot, tot);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (sh.cov) atomicAdd(&accum[c * 2 + 0], sh.cov);
+    if (sh.tot) atomicAdd(&accum[c * 2 + 1], sh.tot);
+  }
+}
+
+__global__ void sp_pivot_zero_kernel(const int32_t* __restrict__ head_cluster, const int32_t* __restrict__ decision,
+                                     int hq, unsigned long long* __restrict__ accum) {
+  const int h = threadIdx.x;
+  if (h < hq && decision[h] == SP_DEC_DENSE) {
+    const int c = head_cluster[h];
+    accum[c * 2 + 0] = 0;
+    accum[c * 2 + 1] = 0;
+  }
+}
+
+__global__ void sp_pivot_finish_kernel(sp_cluster_state st, const int32_t* __restrict__ head_cluster,
+                                       const int32_t* __restrict__ decision, const float* __restrict__ avg_attn,
+                                       int hq, int nb, const unsigned long long* __restrict__ accum) {
+  const int h = threadIdx.x;
+  if (h >= hq || decision[h] != SP_DEC_DENSE) return;
+  const int c = head_cluster[h];
+  // every out-of-range slash / vertical slot of the reference's id list is the padding id 0
+  unsigned long long pad = 0;
+  for (int i = 0; i < nb; ++i) {
+    if (st.cols[(int64_t)c * nb + i]) pad += (unsigned long long)i;
+    if (st.dists[(int64_t)c * nb + i]) pad += (unsigned long long)i;
+  }
+  const unsigned long long a00 = sp_to_fixed(avg_attn[(int64_t)h * nb * nb]);
+  const double cov = (double)accum[c * 2 + 0] + (double)pad * (double)a00;
+  const double tot = (double)accum[c * 2 + 1];
+  st.ratio[c] = tot > 0.0 ? cov / tot : (double)NAN;
+  __threadfence();
+  st.info[c * 8 + 1] = 1;
+}
+
+extern "C" int sp_pivot_update(const sp_cluster_state* state, const int32_t* head_cluster, const int32_t* decision,
+                               const float* avg_attn, int32_t hq, int32_t nb, float pattern_threshold,
+                               sp_stream_t stream) {
+  int rc = check_state(state, nb, "sp_pivot_update");
+  if (rc) return rc;
+  SP_REQUIRE(head_cluster && decision && avg_attn, SP_ERR_INVALID_ARGUMENT, "sp_pivot_update: null pointer");
+  SP_REQUIRE(hq > 0 && hq <= 1024 && nb > 0 && nb <= RS_MAX, SP_ERR_UNSUPPORTED,
+             "sp_pivot_update: hq=%d nb=%d unsupported", hq, nb);
+  if (state->n_clusters == 0) return SP_OK;
+  unsigned long long* accum = reinterpret_cast<unsigned long long*>(state->accum);
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(sp_pivot_zero_kernel, dim3(1), dim3(1024), 0, s, head_cluster, decision, hq, accum);
+  SP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sp_pivot_rows_kernel, dim3(nb, hq), dim3(RS_THREADS), 0, s, *state, head_cluster, decision,
+                     avg_attn, nb, (nb + 63) / 64, (long long)sp_thr_lt(pattern_threshold), accum);
+  SP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sp_pivot_finish_kernel, dim3(1), dim3(1024), 0, s, *state, head_cluster, decision, avg_attn, hq,
+                     nb, accum);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// CSR row pointers of a mask (triton_column_count_cumsum, shareprefill_attn.py:226-269)
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void sp_mask_row_pointers_kernel(const uint64_t* __restrict__ mask, int nb, int nbw,
+                                                                   int32_t* __restrict__ row_ptr) {
+  __shared__ int32_t cnt[RS_MAX];
+  const int h = blockIdx.x;
+  const uint64_t* mh = mask + (int64_t)h * nb * nbw;
+  for (int r = threadIdx.x; r < nb; r += 256) {
+    int c = 0;
+    for (int w = 0; w < nbw; ++w) c += __popcll(mh[(int64_t)r * nbw + w]);
+    cnt[r] = c;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t* out = row_ptr + (int64_t)h * (nb + 1);
+    int acc = 0;
+    out[0] = 0;
+    for (int r = 0; r < nb; ++r) {
+      acc += cnt[r];
+      out[r + 1] = acc;
+    }
+  }
+}
+
+extern "C" int sp_mask_row_pointers(const uint64_t* mask, int32_t hq, int32_t nb, int32_t* row_ptr,
+                                    sp_stream_t stream) {
+  SP_REQUIRE(mask && row_ptr && hq > 0 && nb > 0, SP_ERR_INVALID_ARGUMENT, "sp_mask_row_pointers: bad arguments");
+  SP_REQUIRE(nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_mask_row_pointers: nb=%d exceeds %d", nb, RS_MAX);
+  hipLaunchKernelGGL(sp_mask_row_pointers_kernel, dim3(hq), dim3(256), 0, (hipStream_t)stream, mask, nb,
+                     (nb + 63) / 64, row_ptr);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}

@@ -1,0 +1,288 @@
+"""Torch-tensor front ends of the C-ABI entry points (include/shareprefill_hip.h).
+
+Each function validates shapes on the host, allocates the outputs with torch, and enqueues the HIP
+kernels on torch's current stream.  Tensors follow the library's conventions: token-major or
+head-major q/k/v given as [H, N, D] views with arbitrary token / head strides and contiguous head_dim.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import ClusterStateStruct
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> C.c_void_p:
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _check_hnd(t: torch.Tensor, name: str):
+    if t.dim() != 3:
+        raise ValueError(f"{name} must be [H, N, D], got {tuple(t.shape)}")
+    if t.dtype != torch.bfloat16:
+        raise AssertionError(f"{name} must be bfloat16, got {t.dtype}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU")
+    if t.stride(2) != 1:
+        raise ValueError(f"{name} must have a contiguous head_dim axis")
+
+
+def pool_avg(x: torch.Tensor, block_size: int, tail_mode: int = _lib.SP_POOL_TAIL_TRUE_LENGTH,
+             head_enable: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x: bf16 [H, N, D] view -> bf16 [nb, H, D] block means (reference: triton_bnhd_pool, attn/utils.py:211-261)."""
+    lib = _lib.load()
+    _check_hnd(x, "x")
+    h, n, d = x.shape
+    nb = -(-n // block_size)
+    if out is None:
+        out = torch.empty(nb, h, d, dtype=torch.bfloat16, device=x.device)
+    st = lib.sp_pool_avg_bf16(_ptr(x), _ptr(out), n, h, d, x.stride(1), x.stride(0), block_size, tail_mode,
+                              _ptr(head_enable), _stream())
+    _lib.check(st, "sp_pool_avg_bf16")
+    return out
+
+
+_workspaces = {}
+
+
+def _workspace(tag: str, nbytes: int, device) -> torch.Tensor:
+    """Grow-only scratch buffers keyed by purpose and device (reused across layers)."""
+    key = (tag, str(device))
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def lastq_scores(q: torch.Tensor, k: torch.Tensor, block_size: int, flags: int = _lib.SP_FLAG_LOGITS_BF16):
+    """q [Hq,N,D], k [Hkv,N,D] -> (vert_tok [Hq,N], slash_tok [Hq,N], vert_blk [Hq,nb], slash_blk [Hq,nb]) fp32.
+
+    Reference: attention_sharing.py:127-180 (Step A and the block sum-pool)."""
+    lib = _lib.load()
+    _check_hnd(q, "q")
+    _check_hnd(k, "k")
+    hq, n, d = q.shape
+    hkv = k.shape[0]
+    nb = -(-n // block_size)
+    dev = q.device
+    vert_tok = torch.empty(hq, n, dtype=torch.float32, device=dev)
+    slash_tok = torch.empty(hq, n, dtype=torch.float32, device=dev)
+    vert_blk = torch.empty(hq, nb, dtype=torch.float32, device=dev)
+    slash_blk = torch.empty(hq, nb, dtype=torch.float32, device=dev)
+    need = lib.sp_lastq_scores_workspace_bytes(n, hq, block_size)
+    ws = _workspace("lastq", need, dev)
+    st = lib.sp_lastq_scores_bf16(_ptr(q), _ptr(k), n, hq, hkv, d, q.stride(1), q.stride(0), k.stride(1), k.stride(0),
+                                  block_size, flags, _ptr(ws), ws.numel(), _ptr(vert_tok), _ptr(slash_tok),
+                                  _ptr(vert_blk), _ptr(slash_blk), _stream())
+    _lib.check(st, "sp_lastq_scores_bf16")
+    return vert_tok, slash_tok, vert_blk, slash_blk
+
+
+def cover_count(x: torch.Tensor, thr: float) -> torch.Tensor:
+    """x fp32 [V, L] -> int32 [V] = count(cumsum(sort_desc(x)) <= thr) + 1 (attn/utils.py:47-50)."""
+    lib = _lib.load()
+    assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and x.is_cuda
+    out = torch.empty(x.shape[0], dtype=torch.int32, device=x.device)
+    _lib.check(lib.sp_cover_count(_ptr(x), x.shape[0], x.shape[1], thr, _ptr(out), _stream()), "sp_cover_count")
+    return out
+
+
+def cover_budgets(vert_tok, slash_tok, block_size, pattern_threshold, min_blocks, max_blocks):
+    """Per-head vertical / slash block budgets, int32 [Hq] each (attention_sharing.py:169-176)."""
+    lib = _lib.load()
+    assert vert_tok.is_contiguous() and slash_tok.is_contiguous() and vert_tok.dtype == torch.float32
+    hq, n = vert_tok.shape
+    nv = torch.empty(hq, dtype=torch.int32, device=vert_tok.device)
+    ns = torch.empty(hq, dtype=torch.int32, device=vert_tok.device)
+    st = lib.sp_cover_budgets(_ptr(vert_tok), _ptr(slash_tok), hq, n, block_size, pattern_threshold, min_blocks,
+                              max_blocks, _ptr(nv), _ptr(ns), _stream())
+    _lib.check(st, "sp_cover_budgets")
+    return nv, ns
+
+
+def queryaware_test(q, kbar, vert_blk, block_size, queryaware_threshold, flags=_lib.SP_FLAG_LOGITS_BF16):
+    """-> (avg_qk [Hq,nb] fp32, js_qa [Hq] fp32, use_qa [Hq] int32) (attention_sharing.py:193-202)."""
+    lib = _lib.load()
+    _check_hnd(q, "q")
+    hq, n, d = q.shape
+    nb, hkv, _ = kbar.shape
+    assert kbar.is_contiguous() and kbar.dtype == torch.bfloat16 and vert_blk.is_contiguous()
+    dev = q.device
+    avg_qk = torch.empty(hq, nb, dtype=torch.float32, device=dev)
+    js = torch.empty(hq, dtype=torch.float32, device=dev)
+    use = torch.empty(hq, dtype=torch.int32, device=dev)
+    st = lib.sp_queryaware_test_bf16(_ptr(q), _ptr(kbar), _ptr(vert_blk), n, hq, hkv, d, q.stride(1), q.stride(0),
+                                     block_size, flags, queryaware_threshold, _ptr(avg_qk), _ptr(js), _ptr(use),
+                                     _stream())
+    _lib.check(st, "sp_queryaware_test_bf16")
+    return avg_qk, js, use
+
+
+class ClusterState:
+    """Device slabs of the cross-layer sharing state for C shared clusters (struct sp_cluster_state)."""
+
+    def __init__(self, n_clusters: int, nb: int, device):
+        self.n_clusters, self.nb, self.nbw, self.device = n_clusters, nb, (nb + 63) // 64, device
+        c = max(n_clusters, 1)
+        self.info = torch.zeros(c, 8, dtype=torch.int32, device=device)
+        self.ratio = torch.zeros(c, dtype=torch.float64, device=device)
+        self.vert = torch.zeros(c, nb, dtype=torch.float32, device=device)
+        self.slash = torch.zeros(c, nb, dtype=torch.float32, device=device)
+        self.cols = torch.zeros(c, nb, dtype=torch.uint8, device=device)
+        self.dists = torch.zeros(c, nb, dtype=torch.uint8, device=device)
+        self.pattern = torch.zeros(c, nb, self.nbw, dtype=torch.int64, device=device)
+        self.accum = torch.zeros(c, 2, dtype=torch.int64, device=device)
+        self.struct = ClusterStateStruct(n_clusters, nb, self.nbw, 0, self.info.data_ptr(), self.ratio.data_ptr(),
+                                         self.vert.data_ptr(), self.slash.data_ptr(), self.cols.data_ptr(),
+                                         self.dists.data_ptr(), self.pattern.data_ptr(), self.accum.data_ptr())
+        self.reset()
+
+    def reset(self):
+        """No pivot, no pattern (attention_sharing.py:41-78); enqueued on the current stream."""
+        self.info.zero_()
+        self.info[:, 0] = -1
+
+    def ref(self):
+        return C.byref(self.struct)
+
+
+def share_decide(state: ClusterState, head_cluster, layer_idx, vert_blk, slash_blk, use_qa, nv, ns, min_blocks,
+                 similarity_threshold, fallback_threshold):
+    """-> (decision, js_v, js_s, nv_final, ns_final) (attention_sharing.py:204-301)."""
+    lib = _lib.load()
+    hq = vert_blk.shape[0]
+    dev = vert_blk.device
+    decision = torch.empty(hq, dtype=torch.int32, device=dev)
+    js_v = torch.empty(hq, dtype=torch.float32, device=dev)
+    js_s = torch.empty(hq, dtype=torch.float32, device=dev)
+    nv_f = torch.empty(hq, dtype=torch.int32, device=dev)
+    ns_f = torch.empty(hq, dtype=torch.int32, device=dev)
+    st = lib.sp_share_decide(state.ref(), _ptr(head_cluster), layer_idx, hq, _ptr(vert_blk), _ptr(slash_blk),
+                             _ptr(use_qa), _ptr(nv), _ptr(ns), min_blocks, similarity_threshold, fallback_threshold,
+                             _ptr(decision), _ptr(js_v), _ptr(js_s), _ptr(nv_f), _ptr(ns_f), _stream())
+    _lib.check(st, "sp_share_decide")
+    return decision, js_v, js_s, nv_f, ns_f
+
+
+def build_mask(state: ClusterState, head_cluster, decision, vert_blk, slash_blk, nv_f, ns_f) -> torch.Tensor:
+    """-> bit mask int64 [Hq, nb, nbw] (attention_sharing.py:303-337)."""
+    lib = _lib.load()
+    hq, nb = vert_blk.shape
+    mask = torch.empty(hq, nb, (nb + 63) // 64, dtype=torch.int64, device=vert_blk.device)
+    st = lib.sp_build_mask(state.ref(), _ptr(head_cluster), _ptr(decision), _ptr(vert_blk), _ptr(slash_blk),
+                           _ptr(nv_f), _ptr(ns_f), hq, nb, _ptr(mask), _stream())
+    _lib.check(st, "sp_build_mask")
+    return mask
+
+
+def queryaware_select(qbar, kbar, decision, mask, pattern_threshold, flags=_lib.SP_FLAG_LOGITS_BF16,
+                      probs: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """ORs the query-aware selection into mask for heads with decision == QA; returns the probs scratch."""
+    lib = _lib.load()
+    nb, hq, d = qbar.shape
+    hkv = kbar.shape[1]
+    if probs is None:
+        probs = torch.empty(hq, nb, nb, dtype=torch.float32, device=qbar.device)
+    st = lib.sp_queryaware_select_bf16(_ptr(qbar), _ptr(kbar), _ptr(decision), hq, hkv, d, nb, flags,
+                                       pattern_threshold, _ptr(probs), _ptr(mask), _stream())
+    _lib.check(st, "sp_queryaware_select_bf16")
+    return probs
+
+
+def cover_select_global(x: torch.Tensor, score: float, mask: torch.Tensor, enable: Optional[torch.Tensor] = None):
+    """x fp32 [V, nb, nb]; ORs the kept lower-triangular entries into mask int64 [V, nb, nbw] (attn/utils.py:53-57)."""
+    lib = _lib.load()
+    assert x.dtype == torch.float32 and x.is_contiguous() and mask.is_contiguous()
+    v, nb, _ = x.shape
+    st = lib.sp_cover_select_global(_ptr(x), _ptr(enable), v, nb, score, _ptr(mask), _stream())
+    _lib.check(st, "sp_cover_select_global")
+    return mask
+
+
+def cover_select_rows(x: torch.Tensor, thr: float) -> torch.Tensor:
+    """x fp32 [nb, nb] -> pattern int64 [nb, nbw] (attn/utils.py:60-76)."""
+    lib = _lib.load()
+    assert x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
+    nb = x.shape[0]
+    pat = torch.empty(nb, (nb + 63) // 64, dtype=torch.int64, device=x.device)
+    _lib.check(lib.sp_cover_select_rows(_ptr(x), nb, thr, _ptr(pat), _stream()), "sp_cover_select_rows")
+    return pat
+
+
+def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=None, avg_attn=None):
+    """q [Hq,N,D], k/v [Hkv,N,D] views, mask int64 [Hq,nb,nbw] -> out bf16 [N,Hq,D] contiguous.
+
+    Reference: triton_block_wise_prefill_attention (shareprefill_attn.py:474-620).  avg_attn (fp32 [Hq,nb,nb],
+    zero-filled) receives the block-averaged attention map of the heads whose decision is DENSE."""
+    lib = _lib.load()
+    _check_hnd(q, "q")
+    _check_hnd(k, "k")
+    _check_hnd(v, "v")
+    hq, n, d = q.shape
+    hkv = k.shape[0]
+    assert q.shape[1] == k.shape[1] == v.shape[1], "q_len must equal k_len"
+    assert mask.is_contiguous() and mask.dtype == torch.int64
+    dev = q.device
+    out = torch.empty(n, hq, d, dtype=torch.bfloat16, device=dev)
+    need = lib.sp_attn_workspace_bytes(n, hkv, d, block_size)
+    ws = _workspace("attn_vt", need, dev)
+    st = lib.sp_block_sparse_attn_fwd_bf16(_ptr(q), _ptr(k), _ptr(v), n, hq, hkv, d, q.stride(1), q.stride(0),
+                                           k.stride(1), k.stride(0), v.stride(1), v.stride(0), block_size,
+                                           softmax_scale, _ptr(mask), _ptr(decision), _ptr(out), _ptr(avg_attn),
+                                           _ptr(ws), ws.numel(), _stream())
+    _lib.check(st, "sp_block_sparse_attn_fwd_bf16")
+    return out
+
+
+def pivot_update(state: ClusterState, head_cluster, decision, avg_attn, pattern_threshold):
+    """Stores pattern / vs_ratio of this layer's pivots into the state (attention_sharing.py:94-103)."""
+    lib = _lib.load()
+    hq, nb, _ = avg_attn.shape
+    st = lib.sp_pivot_update(state.ref(), _ptr(head_cluster), _ptr(decision), _ptr(avg_attn), hq, nb,
+                             pattern_threshold, _stream())
+    _lib.check(st, "sp_pivot_update")
+
+
+def mask_row_pointers(mask: torch.Tensor) -> torch.Tensor:
+    """CSR row pointers int32 [Hq, nb+1] of a bit mask (shareprefill_attn.py:226-269)."""
+    lib = _lib.load()
+    hq, nb, _ = mask.shape
+    out = torch.empty(hq, nb + 1, dtype=torch.int32, device=mask.device)
+    _lib.check(lib.sp_mask_row_pointers(_ptr(mask), hq, nb, _ptr(out), _stream()), "sp_mask_row_pointers")
+    return out
+
+
+# ---- mask format helpers (host side, synchronising; for tests and inspection) ---------------------------
+def mask_to_bool(mask: torch.Tensor, nb: int) -> torch.Tensor:
+    """bit mask int64 [..., nb, nbw] -> bool [..., nb, nb]."""
+    shifts = torch.arange(64, device=mask.device, dtype=torch.int64)
+    bits = (mask.unsqueeze(-1) >> shifts) & 1
+    return bits.reshape(*mask.shape[:-1], -1)[..., :nb].bool()
+
+
+def bool_to_mask(b: torch.Tensor) -> torch.Tensor:
+    """bool [..., nb, nb] -> bit mask int64 [..., nb, nbw]."""
+    nb = b.shape[-1]
+    nbw = (nb + 63) // 64
+    pad = nbw * 64 - nb
+    x = torch.nn.functional.pad(b.to(torch.int64), (0, pad)).reshape(*b.shape[:-1], nbw, 64)
+    lo = (x[..., :63] << torch.arange(63, device=b.device, dtype=torch.int64)).sum(-1)
+    hi = torch.where(x[..., 63] != 0, torch.tensor(-(2 ** 63), dtype=torch.int64, device=b.device),
+                     torch.tensor(0, dtype=torch.int64, device=b.device))
+    return (lo | hi).contiguous()
+
+
+def mask_to_block_idx(mask: torch.Tensor, nb: int):
+    """bit mask [Hq, nb, nbw] -> list[Hq] of sorted unique flat ids (row*nb+col), the reference's block_idx."""
+    b = mask_to_bool(mask, nb)
+    return [torch.nonzero(b[h].reshape(-1)).reshape(-1) for h in range(b.shape[0])]

@@ -1,0 +1,59 @@
+"""GPU parity: last-block scores (vertical / slash vectors and their block sums) against the CPU oracle."""
+
+import pytest
+import torch
+
+from oracle import shareprefill_oracle as O
+from shareprefill_amd import synthetic
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(hq, hkv, n, seed):
+    q, k, _ = synthetic.planted_qkv(hq, hkv, n, 128, seed, q_head_gain=1.0)
+    return q[0], k[0]  # [H, N, D] views of token-major storage
+
+
+@pytest.mark.parametrize("hq,hkv,n", [(4, 2, 1024), (8, 2, 4096), (4, 4, 1000), (2, 1, 128), (4, 1, 2304)])
+@pytest.mark.parametrize("bf16_logits", [False, True])
+def test_lastq_scores_match_oracle(gpu_device, hq, hkv, n, bf16_logits):
+    from shareprefill_amd import _lib, ops
+
+    q, k = _inputs(hq, hkv, n, 11 + n)
+    vref, sref = O.lastq_scores(q, k, 128, logits_in_input_dtype=bf16_logits)
+    flags = _lib.SP_FLAG_LOGITS_BF16 if bf16_logits else 0
+    vt, st, vb, sb = ops.lastq_scores(q.to(gpu_device), k.to(gpu_device), 128, flags)
+    vt, st, vb, sb = vt.cpu(), st.cpu(), vb.cpu(), sb.cpu()
+    # a logit that lands on the other side of a bf16 rounding boundary (MFMA vs CPU summation order) moves one
+    # probability by 2^-8 relative; with fp32 logits only exp/sum rounding remains
+    rtol, atol = (3e-2, 1e-6) if bf16_logits else (2e-4, 1e-8)
+    assert torch.allclose(vt, vref, rtol=rtol, atol=atol)
+    assert torch.allclose(st, sref, rtol=rtol, atol=atol)
+    assert torch.allclose(vt.sum(-1), torch.ones(hq), atol=1e-4)
+    assert torch.allclose(st.sum(-1), torch.ones(hq), atol=1e-4)
+    # block sums are the right-padded 128-token sums of the token vectors the kernel itself wrote
+    assert torch.allclose(vb, O.block_sum(vt, 128), rtol=1e-5, atol=1e-9)
+    assert torch.allclose(sb, O.block_sum(st, 128), rtol=1e-5, atol=1e-9)
+
+
+def test_lastq_scores_head_major_layout_and_determinism(gpu_device):
+    from shareprefill_amd import ops
+
+    q, k = _inputs(4, 2, 2048, 5)
+    qg, kg = q.to(gpu_device), k.to(gpu_device)
+    a = ops.lastq_scores(qg, kg, 128)
+    b = ops.lastq_scores(qg.contiguous(), kg.contiguous(), 128)  # [H,N,D] contiguous storage
+    c = ops.lastq_scores(qg, kg, 128)
+    for x, y, z in zip(a, b, c):
+        assert torch.equal(x, y) and torch.equal(x, z)
+
+
+def test_lastq_scores_rejects_unsupported(gpu_device):
+    from shareprefill_amd import ops
+
+    q = torch.zeros(2, 256, 64, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(NotImplementedError):
+        ops.lastq_scores(q, q, 128)
+    q = torch.zeros(2, 64, 128, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(ValueError):
+        ops.lastq_scores(q, q, 128)

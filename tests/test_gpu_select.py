@@ -1,0 +1,163 @@
+"""GPU parity (bit-exact): cumulative-mass selection, budgets, top-k sets and masks against the CPU oracle
+on identical fp32 score inputs."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import shareprefill_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _probs(rows, n, seed, sharp=3.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.softmax(torch.randn(rows, n, generator=g) * sharp, dim=-1)
+
+
+@pytest.mark.parametrize("n", [1000, 8192, 131072])
+@pytest.mark.parametrize("thr", [0.5, 0.9, 0.95, 0.99])
+def test_cover_count_bit_exact(gpu_device, n, thr):
+    from shareprefill_amd import ops
+
+    x = _probs(6, n, n, sharp=4.0)
+    x[1] = 1.0 / n                       # all ties
+    x[2] = 0.0
+    x[2, 17] = 1.0                       # one-hot
+    x[3, : n // 2] = 0.0                 # exact zeros
+    x[3] /= x[3].sum()
+    got = ops.cover_count(x.to(gpu_device).contiguous(), thr).cpu().tolist()
+    want = [O.cover_count(x[i].numpy(), thr) for i in range(x.shape[0])]
+    assert got == want
+
+
+def test_cover_count_threshold_edges(gpu_device):
+    from shareprefill_amd import ops
+
+    x = _probs(2, 4096, 3).to(gpu_device).contiguous()
+    assert ops.cover_count(x, -1.0).cpu().tolist() == [1, 1]
+    assert ops.cover_count(x, 2.0).cpu().tolist() == [4097, 4097]   # never exceeded: every entry counted
+    assert ops.cover_count(x, 0.0).cpu().tolist() == [O.cover_count(x[i].cpu().numpy(), 0.0) for i in range(2)]
+
+
+@pytest.mark.parametrize("hq,n", [(8, 8192), (4, 1000)])
+def test_budgets_bit_exact(gpu_device, hq, n):
+    from shareprefill_amd import ops
+
+    v, s = _probs(hq, n, 1, 5.0), _probs(hq, n, 2, 2.0)
+    nb = -(-n // 128)
+    nv, ns = ops.cover_budgets(v.to(gpu_device), s.to(gpu_device), 128, 0.95, 8, nb)
+
+    def want(x):
+        return [min(max(O.cover_count(x[h].numpy(), 0.95) // 128 + 1, 8), nb) for h in range(hq)]
+
+    assert nv.cpu().tolist() == want(v) and ns.cpu().tolist() == want(s)
+
+
+@pytest.mark.parametrize("nb", [16, 64, 100, 256])
+@pytest.mark.parametrize("thr", [0.9, 0.95])
+def test_cover_select_global_bit_exact(gpu_device, nb, thr):
+    from shareprefill_amd import ops
+
+    g = torch.Generator().manual_seed(nb)
+    logits = torch.randn(3, nb, nb, generator=g) * 2
+    tri = torch.tril(torch.ones(nb, nb, dtype=torch.bool))
+    a = torch.softmax(logits.masked_fill(~tri, float("-inf")), dim=-1)
+    a[2] = torch.softmax(torch.zeros(nb, nb).masked_fill(~tri, float("-inf")), dim=-1)  # uniform rows: heavy ties
+    score = float(np.float32(thr * nb))
+    mask = torch.zeros(3, nb, (nb + 63) // 64, dtype=torch.int64, device=gpu_device)
+    en = torch.tensor([1, 1, 1], dtype=torch.int32, device=gpu_device)
+    ops.cover_select_global(a.to(gpu_device).contiguous(), score, mask, en)
+    got = ops.mask_to_bool(mask, nb).cpu().numpy()
+    for v in range(3):
+        kept = O.cover_keep_le(a[v].numpy().reshape(-1), score)
+        want = np.zeros(nb * nb, dtype=bool)
+        want[kept] = True
+        want = want.reshape(nb, nb) & tri.numpy()
+        want[0, 0] = True
+        assert np.array_equal(got[v], want), f"vector {v}"
+
+
+def test_cover_select_global_skips_disabled(gpu_device):
+    from shareprefill_amd import ops
+
+    a = torch.softmax(torch.zeros(2, 16, 16), -1).to(gpu_device)
+    mask = torch.zeros(2, 16, 1, dtype=torch.int64, device=gpu_device)
+    ops.cover_select_global(a, 8.0, mask, torch.tensor([0, 1], dtype=torch.int32, device=gpu_device))
+    assert int(mask[0].abs().sum()) == 0 and int(mask[1].abs().sum()) != 0
+
+
+@pytest.mark.parametrize("nb", [8, 64, 100, 1024])
+def test_cover_select_rows_bit_exact(gpu_device, nb):
+    from shareprefill_amd import ops
+
+    g = torch.Generator().manual_seed(nb + 1)
+    tri = torch.tril(torch.ones(nb, nb, dtype=torch.bool))
+    a = torch.softmax((torch.randn(nb, nb, generator=g) * 3).masked_fill(~tri, float("-inf")), dim=-1)
+    a[nb // 2] *= 0.5                     # a row that never reaches the threshold keeps one entry
+    a[nb - 1] = a[nb - 1].mean()          # all ties
+    got = ops.mask_to_bool(ops.cover_select_rows(a.to(gpu_device).contiguous(), 0.9), nb).cpu().numpy()
+    want = O.cover_keep_rows_ge(a.numpy(), 0.9) & tri.numpy()
+    want[0, 0] = True
+    assert np.array_equal(got, want)
+
+
+def _table_tensor(table, layer, hq, gpu):
+    ids = {cid: i for i, cid in enumerate(sorted(table["shared_clusters"]))}
+    hc = torch.full((hq,), -1, dtype=torch.int32)
+    for cid, pairs in table["clusters"].items():
+        for lay, h in pairs:
+            if lay == layer and cid in ids:
+                hc[h] = ids[cid]
+    return hc.to(gpu), ids
+
+
+def test_decide_and_mask_match_oracle_on_identical_scores(gpu_device):
+    """Feeds the same pooled vectors / budgets to sp_share_decide + sp_build_mask and to the oracle."""
+    from shareprefill_amd import ops
+
+    hq, nb, minb = 8, 40, 3
+    g = torch.Generator().manual_seed(9)
+    vert = torch.softmax(torch.randn(hq, nb, generator=g) * 2, -1)
+    slash = torch.softmax(torch.randn(hq, nb, generator=g) * 2, -1)
+    nv = torch.randint(minb, 12, (hq,), generator=g, dtype=torch.int32)
+    ns = torch.randint(minb, 12, (hq,), generator=g, dtype=torch.int32)
+    use_qa = torch.tensor([0, 0, 1, 0, 0, 0, 0, 1], dtype=torch.int32)
+    table = {"clusters": {"a": [[0, 0], [0, 1], [0, 2]], "b": [[0, 3], [0, 4]], "c": [[0, 5], [0, 6], [0, 7]]},
+             "shared_clusters": ["a", "c"]}
+    hc, ids = _table_tensor(table, 0, hq, gpu_device)
+    state = ops.ClusterState(len(ids), nb, gpu_device)
+    dev = lambda t: t.to(gpu_device).contiguous()
+    dec, jv, js, nvf, nsf = ops.share_decide(state, hc, 0, dev(vert), dev(slash), dev(use_qa), dev(nv), dev(ns),
+                                             minb, 0.5, 0.9)
+    # heads 0 and 5 are the first non-query-aware heads of the shared clusters -> dense pivots
+    assert dec.cpu().tolist() == [O.DEC_DENSE, O.DEC_VS, O.DEC_QA, O.DEC_VS, O.DEC_VS, O.DEC_DENSE, O.DEC_VS, O.DEC_QA]
+    assert nvf.cpu().tolist() == [int(nv[h]) if h not in (2, 7) else minb for h in range(hq)]
+    mask = ops.mask_to_bool(ops.build_mask(state, hc, dec, dev(vert), dev(slash), nvf, nsf), nb).cpu().numpy()
+    for h in range(hq):
+        if dec[h] == O.DEC_DENSE:
+            want = np.tril(np.ones((nb, nb), bool))
+        else:
+            cols, dists = O.OracleSharing._vs_sets(vert[h], slash[h], int(nvf[h]), int(nsf[h]), nb)
+            want = O.vs_mask(cols, dists, nb)
+        assert np.array_equal(mask[h], want), f"head {h}"
+    # the pivot's stored sets are its own top-k sets with its own budgets
+    for cid, h in (("a", 0), ("c", 5)):
+        cols, dists = O.OracleSharing._vs_sets(vert[h], slash[h], int(nv[h]), int(ns[h]), nb)
+        c = ids[cid]
+        assert sorted(torch.nonzero(state.cols[c]).reshape(-1).cpu().tolist()) == sorted(cols.tolist())
+        assert sorted(torch.nonzero(state.dists[c]).reshape(-1).cpu().tolist()) == sorted(dists.tolist())
+        assert torch.equal(state.vert[c].cpu(), vert[h])
+        assert state.info[c].cpu().tolist()[:5] == [h, 0, int(nv[h]), int(ns[h]), 0]
+
+
+def test_row_pointers_docstring_vector(gpu_device):
+    """shareprefill_attn.py:235-236: ids [0,5,8,9,13,14] on a 4x4 grid -> [0,1,2,4,6]."""
+    from shareprefill_amd import ops
+
+    b = torch.zeros(1, 4, 4, dtype=torch.bool)
+    for i in [0, 5, 8, 9, 13, 14]:
+        b[0, i // 4, i % 4] = True
+    m = ops.bool_to_mask(b).to(gpu_device)
+    assert ops.mask_row_pointers(m).cpu().tolist() == [[0, 1, 2, 4, 6]]
+    assert ops.mask_to_block_idx(m, 4)[0].cpu().tolist() == [0, 5, 8, 9, 13, 14]
