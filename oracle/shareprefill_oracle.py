@@ -229,7 +229,9 @@ def vs_ratio(avg: np.ndarray, cols, dists) -> float:
     """attention_sharing.py:278-286: sum of avg over vs_id_list WITH multiplicity / sum(avg).
 
     Closed form: S(slash set) + S(vertical set) + (sum(dists) + sum(cols)) * avg[0,0]
-    (each out-of-range slash / vertical slot is the padding id 0).  Exact fixed-point sums.
+    (each out-of-range slash / vertical slot is the padding id 0).  The two set sums and the total are exact
+    fixed-point integers; the final combination is evaluated in double as
+    (double(S_sets) + double(pad) * double(avg00)) / double(total), one IEEE operation at a time.
     """
     nb = avg.shape[0]
     fx = to_fixed(avg).astype(object)
@@ -242,10 +244,10 @@ def vs_ratio(avg: np.ndarray, cols, dists) -> float:
     for c in cols:
         r = rr[rr >= c]
         cov += int(fx[r, c].sum())
-    cov += (int(np.sum(dists)) + int(np.sum(cols))) * int(fx[0, 0])
+    pad = int(np.sum(dists)) + int(np.sum(cols))
     if tot == 0:
         return float("nan")
-    return float(cov) / float(tot)
+    return (float(cov) + float(pad) * float(int(fx[0, 0]))) / float(tot)
 
 
 # --------------------------------------------------------------------------- #

@@ -814,9 +814,10 @@ __global__ void sp_pivot_finish_kernel(sp_cluster_state st, const int32_t* __res
     if (st.dists[(int64_t)c * nb + i]) pad += (unsigned long long)i;
   }
   const unsigned long long a00 = sp_to_fixed(avg_attn[(int64_t)h * nb * nb]);
-  const double cov = (double)accum[c * 2 + 0] + (double)pad * (double)a00;
+  // one IEEE operation at a time (no fused multiply-add), so the value is reproducible on a CPU
+  const double cov = __dadd_rn((double)accum[c * 2 + 0], __dmul_rn((double)pad, (double)a00));
   const double tot = (double)accum[c * 2 + 1];
-  st.ratio[c] = tot > 0.0 ? cov / tot : (double)NAN;
+  st.ratio[c] = tot > 0.0 ? __ddiv_rn(cov, tot) : (double)NAN;
   __threadfence();
   st.info[c * 8 + 1] = 1;
 }

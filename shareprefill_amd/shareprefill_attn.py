@@ -1,0 +1,86 @@
+"""The patched attention function (Hugging Face attention-interface signature).
+
+Mirror of shareprefill/attn/shareprefill_attn.py:87-184 of the reference.  Differences, all on purpose:
+  * K / V are not expanded to the query-head count and nothing is transposed to contiguous: the HIP
+    kernels take the [B, H, N, D] views Hugging Face hands over with their real strides;
+  * selection and attention run as a fixed sequence of kernel launches on the current stream, without
+    host synchronisation;
+  * there is no CPU path: tensors must be on a GPU and the HIP library must be built.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib, ops
+from .attention_sharing import budget_blocks
+
+
+def _dense_causal_mask(hq: int, nb: int, device) -> torch.Tensor:
+    tri = torch.tril(torch.ones(nb, nb, dtype=torch.bool, device=device))
+    return ops.bool_to_mask(tri).unsqueeze(0).expand(hq, -1, -1).contiguous()
+
+
+def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: torch.Tensor,
+                                value_states: torch.Tensor, *, gqa_interleave: bool = False
+                                ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """query_states [B, Hq, N, D], key/value_states [B, Hkv, Nk, D] -> (attn_output [B, Hq, N, D], avg_attn).
+
+    Prefill (N != 1): vertical/slash estimation, block selection and sharing, block-sparse attention,
+    pivot update (shareprefill_attn.py:110-144).  Decode (N == 1): dense attention of the one query over
+    all keys (:146-155)."""
+    bsz, num_heads, q_len, head_dim = query_states.shape
+    config = module.config
+    softmax_scale = getattr(module, "scaling", 1.0 / math.sqrt(head_dim))
+    if gqa_interleave:
+        raise NotImplementedError("gqa_interleave=True (query head h -> kv head h % Hkv) is not supported")
+
+    if q_len == 1:
+        out = torch.nn.functional.scaled_dot_product_attention(
+            query_states, key_states, value_states, dropout_p=0.0, is_causal=False, scale=softmax_scale,
+            enable_gqa=key_states.shape[1] != num_heads)
+        return out, None
+
+    if bsz != 1:
+        raise ValueError("SharePrefill prefill keeps per-cluster state for batch size 1 only")
+    assert query_states.dtype == torch.bfloat16, "SharePrefill attention expects bfloat16 q/k/v"
+    assert key_states.shape[2] == q_len, "prefill expects q_len == k_len (no cached prefix)"
+    _lib.load()
+
+    q, k, v = query_states[0], key_states[0], value_states[0]
+    block_size = config.block_size
+    nb = -(-q_len // block_size)
+    sharing = module.attention_sharing
+    avg_attn = torch.zeros(1, num_heads, nb, nb, dtype=torch.float32, device=q.device)
+    if q_len < block_size:
+        # shorter than one block: a single diagonal block, nothing to select (the reference cannot run here)
+        mask = _dense_causal_mask(num_heads, nb, q.device)
+        out = ops.block_sparse_attention(q, k, v, mask, block_size, softmax_scale)
+        return out.unsqueeze(0).transpose(1, 2), avg_attn
+
+    minb, maxb = budget_blocks(config.min_budget, config.max_budget, block_size)
+    plan = sharing.plan_layer(q, k, module.layer_idx, block_size, minb, maxb, config.pattern_threshold,
+                              config.similarity_threshold, config.fallback_threshold, config.queryaware_threshold)
+    out = ops.block_sparse_attention(q, k, v, plan.mask, block_size, softmax_scale, decision=plan.decision,
+                                     avg_attn=avg_attn[0])
+    sharing.update_pivotal_attns(module.layer_idx, avg_attn, plan.decision, config.pattern_threshold)
+    return out.unsqueeze(0).transpose(1, 2), avg_attn
+
+
+def shareprefill_attention_forward(module, query_states: torch.Tensor, key_states: torch.Tensor,
+                                   value_states: torch.Tensor, attention_mask: Optional[torch.Tensor], *,
+                                   scaling: float, dropout: float = 0.0, **kwargs
+                                   ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Attention-interface entry (shareprefill_attn.py:158-184): returns (attn_output [B, N, Hq, D] contiguous,
+    attn_weights), attn_weights being the block-average map [B, Hq, nb, nb] on prefill and None on decode.
+    As in the reference, attention_mask / scaling / dropout are ignored (module.scaling is used) and a
+    sliding window is rejected."""
+    if kwargs.pop("sliding_window", None) is not None:
+        raise NotImplementedError("SharePrefill attention does not support sliding-window mode yet.")
+    gqa_interleave = kwargs.pop("gqa_interleave", False)
+    attn_output, attn_weights = shareprefill_attention_core(module, query_states, key_states, value_states,
+                                                            gqa_interleave=gqa_interleave)
+    return attn_output.transpose(1, 2).contiguous(), attn_weights

@@ -1,0 +1,232 @@
+"""GPU parity of the whole SharePrefill layer (scores -> budgets -> query-aware test -> pivot / share
+decision -> mask -> block-sparse attention -> pivot update) through the patched attention function.
+
+Two comparisons per layer:
+  * forced: the oracle's integer logic is fed the float intermediates the GPU produced; decisions, budgets,
+    masks, pivot patterns and coverage ratios must then be IDENTICAL (bit-exact selection on identical scores);
+  * free: the oracle computes everything itself; float stages agree to tolerance, and on these seeded inputs
+    (no value sits on a decision boundary) the decisions and masks agree as well.
+Attention outputs are checked against the fp32 masked-attention oracle on the GPU's mask.
+"""
+
+import json
+import math
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import shareprefill_oracle as O
+from shareprefill_amd import synthetic
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_REL = 2e-2, 2.5e-3  # see tests/test_gpu_attention.py for the mean-rel floor of a bf16 result
+
+
+class FakeAttention:
+    """The attributes the attention function reads from a Hugging Face attention module."""
+
+    def __init__(self, cfg, sharing, layer_idx, head_dim, hq, hkv):
+        self.config = cfg
+        self.attention_sharing = sharing
+        self.layer_idx = layer_idx
+        self.scaling = head_dim ** -0.5
+        self.num_heads = hq
+        self.num_key_value_groups = hq // hkv
+        self.training = False
+        self.attention_dropout = 0.0
+
+
+def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, **thr):
+    from shareprefill_amd import AttentionSharing, shareprefill_attention_forward, ops
+
+    kw = dict(block_size=128, min_budget=1024, max_budget=None, pattern_threshold=0.95, similarity_threshold=0.5,
+              fallback_threshold=0.9, queryaware_threshold=0.1)
+    kw.update(thr)
+    table = synthetic.random_cluster_table(hq, n_clusters, n_layers, seed)
+    path = synthetic.write_cluster_table(table, str(tmp_path / "table.json"))
+    q, k, v = synthetic.planted_qkv(hq, hkv, n, 128, seed, q_head_gain=1.0)
+    sharing = AttentionSharing(path)
+    sharing.keep_debug = True
+    cfg = types.SimpleNamespace(**kw)
+    oracle_forced = O.OracleSharing(O.ClusterTable(table["clusters"], table["shared_clusters"]))
+    oracle_free = O.OracleSharing(O.ClusterTable(table["clusters"], table["shared_clusters"]))
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    nb = -(-n // 128)
+    results = []
+    for layer in range(n_layers):
+        mod = FakeAttention(cfg, sharing, layer, 128, hq, hkv)
+        out, avg = shareprefill_attention_forward(mod, qg, kg, vg, None, scaling=mod.scaling)
+        plan = sharing.plans[-1]
+        assert out.shape == (1, n, hq, 128) and out.is_contiguous() and out.dtype == torch.bfloat16
+        assert avg.shape == (1, hq, nb, nb) and avg.dtype == torch.float32
+        gpu_mask = ops.mask_to_bool(plan.mask, nb).cpu().numpy()
+        dec = plan.decision.cpu().numpy()
+        inject = dict(vert_tok=plan.vert_tok.cpu(), slash_tok=plan.slash_tok.cpu(), vert_blk=plan.vert_blk.cpu(),
+                      slash_blk=plan.slash_blk.cpu(), avg_qk=plan.avg_qk.cpu(), js_qa=plan.js_qa.cpu(),
+                      js_v=plan.js_v.cpu().numpy(), js_s=plan.js_s.cpu().numpy(),
+                      qa_probs={h: plan.qa_probs[h].cpu() for h in range(hq)})
+        okw = dict(bs=128, min_budget=kw["min_budget"], max_budget=kw["max_budget"],
+                   pattern_threshold=kw["pattern_threshold"], similarity_threshold=kw["similarity_threshold"],
+                   fallback_threshold=kw["fallback_threshold"], queryaware_threshold=kw["queryaware_threshold"])
+        forced = oracle_forced.layer(q[0], k[0], v[0], layer, compute_attention=False, inject=inject, **okw)
+        oracle_forced.update_pivots(layer, forced.decision, avg[0].cpu().numpy(), kw["pattern_threshold"])
+        free = oracle_free.layer(q[0], k[0], v[0], layer, compute_attention=False, **okw)
+        oracle_free.update_pivots(layer, free.decision, avg[0].cpu().numpy(), kw["pattern_threshold"])
+        results.append(dict(layer=layer, out=out.cpu(), avg=avg.cpu(), plan=plan, mask=gpu_mask, dec=dec,
+                            forced=forced, free=free))
+    return dict(q=q[0], k=k[0], v=v[0], table=table, sharing=sharing, oracle_forced=oracle_forced,
+                oracle_free=oracle_free, layers=results, nb=nb, kw=kw)
+
+
+def check_forced(run):
+    sharing = run["sharing"]
+    for L in run["layers"]:
+        plan, forced = L["plan"], L["forced"]
+        assert plan.nv.cpu().tolist() == forced.nv.tolist(), "vertical budgets"
+        assert plan.ns.cpu().tolist() == forced.ns.tolist(), "slash budgets"
+        assert L["dec"].tolist() == forced.decision.tolist(), "decisions"
+        assert plan.nv_final.cpu().tolist() == forced.nv_final.tolist()
+        assert plan.ns_final.cpu().tolist() == forced.ns_final.tolist()
+        for h in range(L["mask"].shape[0]):
+            assert np.array_equal(L["mask"][h], forced.mask[h]), f"layer {L['layer']} head {h}: mask differs"
+    # pivot state after the last layer: pattern bits and coverage ratio
+    summary = sharing.pivot_summary()
+    state = sharing._state
+    for cid, st in run["oracle_forced"].state.items():
+        if cid not in sharing._slot:
+            continue
+        got = summary[cid]
+        assert got["pivot_head"] == (-1 if st.pivot_head is None else st.pivot_head)
+        if st.pattern is not None:
+            from shareprefill_amd import ops
+
+            pat = ops.mask_to_bool(state.pattern[sharing._slot[cid]], run["nb"]).cpu().numpy()
+            assert np.array_equal(pat, st.pattern), f"cluster {cid}: pattern differs"
+            assert got["vs_ratio"] == O.vs_ratio(st.avg, st.cols, st.dists), f"cluster {cid}: vs_ratio"
+
+
+def check_free(run, expect_same_masks=True):
+    for L in run["layers"]:
+        plan, free = L["plan"], L["free"]
+        assert torch.allclose(plan.vert_tok.cpu(), free.vert_tok, rtol=3e-2, atol=1e-6)
+        assert torch.allclose(plan.slash_tok.cpu(), free.slash_tok, rtol=3e-2, atol=1e-6)
+        assert torch.allclose(plan.vert_blk.cpu(), free.vert_blk, rtol=1e-2, atol=1e-6)
+        assert torch.allclose(plan.avg_qk.cpu(), free.avg_qk, rtol=2e-2, atol=1e-7)
+        assert torch.allclose(plan.js_qa.cpu(), free.js_qa, rtol=2e-2, atol=1e-4)
+        kb, kr = plan.kbar.cpu().float(), free.kbar.float()
+        assert (kb - kr).abs().max().item() <= 2 ** -8 * max(1.0, kr.abs().max().item())
+        if expect_same_masks:
+            assert L["dec"].tolist() == free.decision.tolist()
+            differing = sum(int((L["mask"][h] != free.mask[h]).sum()) for h in range(L["mask"].shape[0]))
+            assert differing <= 0.002 * L["mask"].sum(), f"{differing} mask bits differ from the free-running oracle"
+
+
+def check_outputs(run):
+    q, k, v = run["q"], run["k"], run["v"]
+    for L in run["layers"]:
+        want = L["dec"] == O.DEC_DENSE
+        ref, avg_ref = O.masked_attention(q, k, v, L["mask"], 128, 128 ** -0.5, want_avg=want)
+        out = L["out"][0].transpose(0, 1).float()
+        assert (out - ref).abs().max().item() <= MAX_ABS
+        assert ((out - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL
+        for h in np.nonzero(want)[0]:
+            assert torch.allclose(L["avg"][0, h], avg_ref[h], rtol=3e-2, atol=2e-5)
+            assert torch.allclose(L["avg"][0, h].sum(-1), torch.ones(run["nb"]), atol=2e-3)
+        for h in np.nonzero(~want)[0]:
+            assert float(L["avg"][0, h].abs().sum()) == 0.0
+
+
+def test_layer_default_thresholds_small(gpu_device, tmp_path):
+    run = run_layers(gpu_device, tmp_path, hq=8, hkv=2, n=2048, seed=21, n_clusters=2)
+    check_forced(run)
+    check_free(run)
+    check_outputs(run)
+    d0 = run["layers"][0]["dec"]
+    assert (d0 == O.DEC_DENSE).sum() == 2  # one pivot per shared cluster in the first layer
+
+
+def test_layer_c1_shape(gpu_device, tmp_path):
+    """B1 Hq8 Hkv2 D128 N8192, 2 clusters of 4: the CPU-runnable parity configuration (inputs in bf16)."""
+    w = synthetic.WORKLOADS["C1"]
+    run = run_layers(gpu_device, tmp_path, hq=w.hq, hkv=w.hkv, n=w.seq_len, seed=w.seed, n_clusters=w.n_clusters,
+                     pattern_threshold=w.pattern_threshold)
+    check_forced(run)
+    check_free(run)
+    check_outputs(run)
+
+
+def test_layer_sharing_and_query_aware_paths(gpu_device, tmp_path):
+    """fallback_threshold lifted so similar heads DO share in layer 1; queryaware_threshold set between the
+    heads' JS values so that some heads take the query-aware path."""
+    probe = run_layers(gpu_device, tmp_path, hq=8, hkv=2, n=4096, seed=33, n_clusters=2, n_layers=1)
+    js = np.sort(probe["layers"][0]["plan"].js_qa.cpu().numpy())
+    qat = float((js[2] + js[3]) / 2)  # three heads below the threshold
+    run = run_layers(gpu_device, tmp_path, hq=8, hkv=2, n=4096, seed=33, n_clusters=2, fallback_threshold=1e9,
+                     queryaware_threshold=qat)
+    check_forced(run)
+    check_free(run)
+    check_outputs(run)
+    d0, d1 = run["layers"][0]["dec"], run["layers"][1]["dec"]
+    assert (d0 == O.DEC_QA).sum() == 3 and (d1 == O.DEC_QA).sum() == 3
+    assert (d0 == O.DEC_SHARE).sum() == 0          # a fresh pivot's siblings cannot share in the same layer
+    assert (d1 == O.DEC_SHARE).sum() >= 1          # next layer: same inputs -> JS = 0 -> shared
+    hist = run["sharing"].decision_histogram()
+    assert hist["dense_pivot"] == 2 and hist["shared"] == int((d1 == O.DEC_SHARE).sum())
+
+
+def test_layer_ragged_length(gpu_device, tmp_path):
+    run = run_layers(gpu_device, tmp_path, hq=4, hkv=2, n=1000, seed=5, n_clusters=2, fallback_threshold=1e9,
+                     min_budget=256)
+    check_forced(run)
+    check_free(run, expect_same_masks=False)
+    check_outputs(run)
+
+
+def test_reference_style_interfaces(gpu_device, tmp_path):
+    """get_active_blocks / update_pivotal_attns with the reference's argument layout, and the id-list view."""
+    from shareprefill_amd import AttentionSharing, ops
+
+    hq, hkv, n = 4, 2, 1024
+    table = synthetic.random_cluster_table(hq, 2, 2, 3)
+    path = synthetic.write_cluster_table(table, str(tmp_path / "t.json"))
+    q, k, v = synthetic.planted_qkv(hq, hkv, n, 128, 3)
+    sharing = AttentionSharing(path)
+    qn, kn = q.transpose(1, 2).to(gpu_device), k.transpose(1, 2).to(gpu_device)  # [B, N, H, D]
+    mask, use_dense = sharing.get_active_blocks(qn, kn, 0, hq, 128, 8, 2 ** 24, 0.9, 0.5, 0.9, 0.1)
+    assert mask.shape == (1, hq, 8, 1) and use_dense.shape == (1, hq) and use_dense.dtype == torch.bool
+    ids = sharing.plans[-1].block_idx()[0]
+    dense_heads = torch.nonzero(use_dense[0]).reshape(-1).cpu().tolist()
+    assert len(dense_heads) == 2
+    for h in dense_heads:  # all lower-triangular ids, attention_sharing.py:217-219
+        assert ids[h].cpu().tolist() == [r * 8 + c for r in range(8) for c in range(r + 1)]
+    with pytest.raises(NotImplementedError):
+        sharing.get_active_blocks(qn, kn, 0, hq, 128, 8, 2 ** 24, gqa_interleave=True)
+    with pytest.raises(ValueError):
+        sharing.get_active_blocks(qn.expand(2, -1, -1, -1), kn.expand(2, -1, -1, -1), 0, hq, 128, 8, 2 ** 24)
+    sharing.reset_state()
+    assert all(v["pivot_head"] == -1 for v in sharing.pivot_summary().values())
+
+
+def test_forward_rejects_sliding_window_and_handles_short_and_decode(gpu_device, tmp_path):
+    from shareprefill_amd import AttentionSharing, shareprefill_attention_forward
+
+    table = synthetic.random_cluster_table(4, 2, 1, 0)
+    path = synthetic.write_cluster_table(table, str(tmp_path / "t.json"))
+    cfg = types.SimpleNamespace(block_size=128, min_budget=1024, max_budget=None, pattern_threshold=0.9,
+                                similarity_threshold=0.5, fallback_threshold=0.9, queryaware_threshold=0.1)
+    mod = FakeAttention(cfg, AttentionSharing(path), 0, 128, 4, 2)
+    g = torch.Generator().manual_seed(0)
+    mk = lambda h, n: torch.randn(1, n, h, 128, generator=g).to(torch.bfloat16).transpose(1, 2).to(gpu_device)
+    q, k, v = mk(4, 100), mk(2, 100), mk(2, 100)
+    with pytest.raises(NotImplementedError):
+        shareprefill_attention_forward(mod, q, k, v, None, scaling=1.0, sliding_window=4096)
+    out, w = shareprefill_attention_forward(mod, q, k, v, None, scaling=1.0)   # shorter than a block: dense causal
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float().repeat_interleave(2, 1),
+                                                           v.float().repeat_interleave(2, 1), is_causal=True)
+    assert (out.transpose(1, 2).float() - ref).abs().max().item() <= MAX_ABS
+    out1, w1 = shareprefill_attention_forward(mod, q[:, :, -1:], k, v, None, scaling=1.0)  # decode step
+    assert w1 is None and out1.shape == (1, 1, 4, 128)
+    assert (out1[0, 0].float() - ref[0, :, -1].float()).abs().max().item() <= MAX_ABS
