@@ -1,0 +1,279 @@
+"""Benchmark of the SharePrefill prefill-attention layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--pattern-threshold 0.95]
+
+A step is one pass of the whole layer (last-block scores, budgets, K pooling, query-aware test, pivot /
+share decision, mask build, Q pooling + query-aware selection, V repack, block-sparse attention, pivot
+update) over one synthetic Q/K/V batch that is already resident in HBM.  The layer timed is layer 1, after
+one untimed call of layer 0 has elected the cluster pivots (sharing can only start in the layer after the
+pivot's, shareprefill/attn/shareprefill_attn.py:141-143).  Prints ONE JSON line.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import tempfile
+import time
+import types
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+FLOP_PER_BLOCK = 4 * 128 * 128 * 128       # QK^T + PV of one kept 128x128 block at head_dim 128
+PEAK_BF16_TFLOPS = 2500.0                  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C5"])
+    ap.add_argument("--pattern-threshold", type=float, default=None)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the stage breakdown / dense baseline / sweep")
+    ap.add_argument("--sweep", action="store_true", help="also time pattern_threshold 0.9 and 0.99")
+    return ap.parse_args()
+
+
+def event_ms(fn, reps=3):
+    import torch
+
+    fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        ts.append(a.elapsed_time(b))
+    return sum(ts) / len(ts)
+
+
+def cpu_baseline(w, q, k, v, mask_bool, decision, kept_blocks, pt):
+    """Times the CPU oracle (torch-CPU restatement of the reference mask logic + block-sparse attention over
+    kept blocks) on a bounded sample and scales it to one layer: the selection float work on 2 of the heads,
+    the attention on 6 (head, query-block) rows spread over the heads and the sequence."""
+    import numpy as np
+    import torch
+
+    from oracle import shareprefill_oracle as O
+
+    hq, n, bs = w.hq, w.seq_len, w.block_size
+    nb = n // bs
+    g = hq // w.hkv
+    heads = [0, hq - 1]
+    qc = q[0][heads].cpu()
+    kc = k[0][[h // g for h in heads]].cpu()
+    t0 = time.perf_counter()
+    for i in range(len(heads)):
+        vt, st = O.lastq_scores(qc[i:i + 1], kc[i:i + 1], bs)
+        O.cover_count(vt[0].numpy(), pt)
+        O.cover_count(st[0].numpy(), pt)
+        O.block_sum(vt, bs), O.block_sum(st, bs)
+        O.pool_avg(kc[i].unsqueeze(1), bs)
+    t_sel = (time.perf_counter() - t0) / len(heads) * hq
+    # attention sample: rows at 1/6, 2/6 ... of the sequence, heads spread
+    rows = [(int(hq * (i + 0.5) / 6), int(nb * (i + 1) / 6) - 1) for i in range(6)]
+    blocks = 0
+    t_att = 0.0
+    for h, r in rows:
+        qh = q[0][h:h + 1, r * bs:(r + 1) * bs].cpu()
+        kh, vh = k[0][h // g:h // g + 1, : (r + 1) * bs].cpu(), v[0][h // g:h // g + 1, : (r + 1) * bs].cpu()
+        cols = np.nonzero(mask_bool[h, r, : r + 1])[0]
+        t1 = time.perf_counter()
+        kidx = torch.cat([torch.arange(c * bs, (c + 1) * bs) for c in cols])
+        s = (qh[0].float() @ kh[0][kidx].float().T) * (w.head_dim ** -0.5)
+        pos = torch.arange(r * bs, (r + 1) * bs)
+        s = s.masked_fill(kidx[None, :] > pos[:, None], float("-inf"))
+        p = torch.softmax(s, -1)
+        _ = p @ vh[0][kidx].float()
+        t_att += time.perf_counter() - t1
+        blocks += len(cols)
+    per_block = t_att / max(blocks, 1)
+    total_ms = (t_sel + per_block * kept_blocks) * 1e3
+    return {"value": round(total_ms, 1), "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"selection float stages on heads {heads} (x{hq // len(heads)}), fp32 block-sparse attention on "
+                      f"{len(rows)} (head, query-block) rows = {blocks} kept blocks at {per_block * 1e3:.3f} ms/block, "
+                      f"scaled to {kept_blocks} kept blocks; extrapolated"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU only (the SharePrefill layer has no multi-GPU path); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from shareprefill_amd import AttentionSharing, _lib, ops, shareprefill_attention_forward, synthetic
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    _lib.load()
+    dev = torch.device("cuda:0")
+    w = synthetic.WORKLOADS[args.workload]
+    pt = w.pattern_threshold if args.pattern_threshold is None else args.pattern_threshold
+    q, k, v = synthetic.workload_inputs(w, device=dev)
+    table = synthetic.random_cluster_table(w.hq, w.n_clusters, 2, w.seed)
+    with tempfile.TemporaryDirectory() as tmp:
+        sharing = AttentionSharing(synthetic.write_cluster_table(table, os.path.join(tmp, "table.json")))
+    nb = w.seq_len // w.block_size
+
+    def make_cfg(thr):
+        return types.SimpleNamespace(block_size=w.block_size, min_budget=w.min_budget, max_budget=None,
+                                     pattern_threshold=thr, similarity_threshold=w.similarity_threshold,
+                                     fallback_threshold=w.fallback_threshold,
+                                     queryaware_threshold=w.queryaware_threshold)
+
+    def module(layer, thr):
+        return types.SimpleNamespace(config=make_cfg(thr), attention_sharing=sharing, layer_idx=layer,
+                                     scaling=w.head_dim ** -0.5)
+
+    def run_layer(layer, thr):
+        return shareprefill_attention_forward(module(layer, thr), q, k, v, None, scaling=w.head_dim ** -0.5)
+
+    def prime(thr):
+        sharing.reset_state()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        run_layer(0, thr)
+        b.record()
+        b.synchronize()
+        return a.elapsed_time(b)
+
+    # ---- layer 0 once (pivot election), then W warm-up and K timed steps of layer 1 -----------------
+    layer0_ms = prime(pt)
+    plan0 = sharing.plans[-1]
+    for _ in range(args.warmup):
+        run_layer(1, pt)
+    torch.cuda.synchronize()
+    timer = ops.KernelTimer()
+    ops.kernel_timer = timer
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_layer(1, pt)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ops.kernel_timer = None
+    ms_per_step = elapsed / args.steps * 1e3
+    plan = sharing.plans[-1]
+    kept = int(ops.mask_row_pointers(plan.mask)[:, -1].sum())
+    tri = w.hq * nb * (nb + 1) // 2
+    density = kept / tri
+    attn_ms = timer.durations_ms("attn")
+    attn_avg_ms = sum(attn_ms) / len(attn_ms)
+    flop = kept * FLOP_PER_BLOCK
+    attn_tflops = flop / (attn_avg_ms * 1e-3) / 1e12
+    layer_tflops = flop / (ms_per_step * 1e-3) / 1e12
+    hist = {}
+    names = {0: "vertical_slash", 1: "dense_pivot", 2: "shared", 3: "query_aware"}
+    for code, cnt in zip(*torch.unique(plan.decision.cpu(), return_counts=True)):
+        hist[names[int(code)]] = int(cnt)
+    hist0 = {}
+    for code, cnt in zip(*torch.unique(plan0.decision.cpu(), return_counts=True)):
+        hist0[names[int(code)]] = int(cnt)
+    kept0 = int(ops.mask_row_pointers(plan0.mask)[:, -1].sum())
+
+    line = {
+        "metric": "sparse_attn_prefill_ms_per_layer_128k" if args.workload == "C3" else
+                  f"sparse_attn_prefill_ms_per_layer_{args.workload}",
+        "value": round(ms_per_step, 3), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{w.name}: B1 Hq{w.hq} Hkv{w.hkv} D{w.head_dim} N{w.seq_len} bf16, block 128, "
+                               f"min_budget {w.min_budget}, pattern_threshold {pt}, similarity {w.similarity_threshold}, "
+                               f"fallback {w.fallback_threshold}, queryaware {w.queryaware_threshold}, "
+                               f"{w.n_clusters} shared clusters; layer 1 timed after pivot-election layer 0",
+                   "generator": f"seed {w.seed}, sink {synthetic.SINK_TOKENS} tok x{synthetic.SINK_SCALE}, band "
+                                f"{synthetic.BAND_PAIRS} rotary pairs beta {synthetic.BAND_BETA} width "
+                                f"{synthetic.BAND_WIDTH}, head gain {synthetic.HEAD_GAIN}"},
+        "kept_blocks": kept, "density": round(density, 4), "decisions": hist,
+        "layer_tflops_on_kept_blocks": round(layer_tflops, 1),
+        "layer_frac_of_bf16_peak": round(layer_tflops / PEAK_BF16_TFLOPS, 4),
+        "layer0": {"ms": round(layer0_ms, 3), "decisions": hist0,
+                   "density": round(kept0 / tri, 4)},
+        "roofline": {"bound": "mfma", "kernel": "sp_attn_fwd_kernel", "achieved": round(attn_tflops, 1),
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
+                     "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms), "traffic": None},
+    }
+
+    if not args.no_extras:
+        qh, kh, vh = q[0], k[0], v[0]
+        stages = {}
+        stages["lastq_scores"] = event_ms(lambda: ops.lastq_scores(qh, kh, 128))
+        vt, st_, vb, sb = ops.lastq_scores(qh, kh, 128)
+        stages["cover_budgets"] = event_ms(lambda: ops.cover_budgets(vt, st_, 128, pt, 8, nb))
+        stages["pool_k"] = event_ms(lambda: ops.pool_avg(kh, 128))
+        stages["pool_q_all_heads"] = event_ms(lambda: ops.pool_avg(qh, 128))
+        kbar = ops.pool_avg(kh, 128)
+        stages["queryaware_test"] = event_ms(lambda: ops.queryaware_test(qh, kbar, vb, 128, w.queryaware_threshold))
+        ws = ops._workspace("attn_vt", _lib.load().sp_attn_workspace_bytes(w.seq_len, w.hkv, w.head_dim, 128), dev)
+        lib = _lib.load()
+        stages["repack_v"] = event_ms(lambda: lib.sp_attn_repack_v_bf16(
+            vh.data_ptr(), w.seq_len, w.hkv, w.head_dim, vh.stride(1), vh.stride(0), 128, ws.data_ptr(), ws.numel(),
+            torch.cuda.current_stream().cuda_stream))
+        stages["attention"] = attn_avg_ms
+        stages["other_selection_and_host"] = max(0.0, ms_per_step - sum(
+            stages[x] for x in ("lastq_scores", "cover_budgets", "pool_k", "queryaware_test", "repack_v", "attention")))
+        line["stage_ms"] = {a: round(b, 3) for a, b in stages.items()}
+        kbytes = w.seq_len * w.hkv * w.head_dim * 2 + nb * w.hkv * w.head_dim * 2
+        qbytes = w.seq_len * w.hq * w.head_dim * 2 + nb * w.hq * w.head_dim * 2
+        line["pooling"] = {"k_GBps": round(kbytes / stages["pool_k"] / 1e6, 1),
+                           "q_GBps": round(qbytes / stages["pool_q_all_heads"] / 1e6, 1),
+                           "peak_GBps": PEAK_HBM_GBS,
+                           "q_frac": round(qbytes / stages["pool_q_all_heads"] / 1e6 / PEAK_HBM_GBS, 4)}
+        # dense causal baseline at the same shape (every lower-triangular block kept)
+        dense_mask = torch.tril(torch.ones(nb, nb, dtype=torch.bool, device=dev))
+        dense_mask = ops.bool_to_mask(dense_mask).unsqueeze(0).expand(w.hq, -1, -1).contiguous()
+        tm = ops.KernelTimer()
+        ops.kernel_timer = tm
+        for _ in range(2):
+            ops.block_sparse_attention(qh, kh, vh, dense_mask, 128, w.head_dim ** -0.5)
+        torch.cuda.synchronize()
+        ops.kernel_timer = None
+        dms = tm.durations_ms("attn")[-1]
+        line["dense_causal_baseline"] = {"ms": round(dms, 3), "blocks": tri,
+                                         "tflops": round(tri * FLOP_PER_BLOCK / dms / 1e9, 1),
+                                         "frac": round(tri * FLOP_PER_BLOCK / dms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+        if args.sweep:
+            sweep = []
+            for thr in (0.9, 0.95, 0.99):
+                prime(thr)
+                run_layer(1, thr)
+                torch.cuda.synchronize()
+                tm = ops.KernelTimer()
+                ops.kernel_timer = tm
+                t1 = time.perf_counter()
+                for _ in range(3):
+                    run_layer(1, thr)
+                torch.cuda.synchronize()
+                ms = (time.perf_counter() - t1) / 3 * 1e3
+                ops.kernel_timer = None
+                kb = int(ops.mask_row_pointers(sharing.plans[-1].mask)[:, -1].sum())
+                ams = sum(tm.durations_ms("attn")) / 3
+                sweep.append({"pattern_threshold": thr, "density": round(kb / tri, 4), "layer_ms": round(ms, 3),
+                              "attn_ms": round(ams, 3), "attn_tflops": round(kb * FLOP_PER_BLOCK / ams / 1e9, 1),
+                              "layer_frac_of_peak": round(kb * FLOP_PER_BLOCK / ms / 1e9 / PEAK_BF16_TFLOPS, 4)})
+            line["threshold_sweep"] = sweep
+
+    if not args.no_cpu_baseline:
+        mask_bool = ops.mask_to_bool(plan.mask, nb).cpu().numpy()
+        line["cpu_baseline"] = cpu_baseline(w, q, k, v, mask_bool, plan.decision.cpu().numpy(), kept, pt)
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

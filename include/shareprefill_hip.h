@@ -152,14 +152,21 @@ int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec,
  * Replaces triton_block_wise_prefill_attention / block_wise_prefill_attention_kernel /
  * count_kernel (shareprefill_attn.py:187-620).  out: bf16 [n][hq][d] contiguous.  Only blocks set in
  * mask (and c <= r) are computed.  For heads with decision == SP_DEC_DENSE the block-averaged attention
- * map avg_attn[h][nb][nb] (fp32, pre-zeroed by the caller) is written as well (:425-457).
- * vt_workspace: sp_attn_workspace_bytes(...) bytes of device scratch (key-major repack of V). */
+ * map avg_attn[h][nb][nb] (fp32, pre-zeroed by the caller) is written as well (:425-457); decision and
+ * avg_attn may both be NULL.
+ * workspace: sp_attn_workspace_bytes(...) bytes of device scratch holding the key-major repack of V.
+ * sp_attn_repack_v_bf16 fills it; sp_block_sparse_attn_fwd_bf16 calls it first unless flags has
+ * SP_ATTN_V_REPACKED (the caller already repacked this v into this workspace). */
+#define SP_ATTN_V_REPACKED 1u
 size_t sp_attn_workspace_bytes(int64_t n, int32_t hkv, int32_t d, int32_t bs);
+int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n, int64_t v_stride_h,
+                          int32_t bs, void* workspace, size_t workspace_bytes, sp_stream_t stream);
 int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,
                                   int32_t d, int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n,
                                   int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h, int32_t bs,
                                   float softmax_scale, const uint64_t* mask, const int32_t* decision, void* out,
-                                  float* avg_attn, void* workspace, size_t workspace_bytes, sp_stream_t stream);
+                                  float* avg_attn, void* workspace, size_t workspace_bytes, uint32_t flags,
+                                  sp_stream_t stream);
 
 /* ---- pivot state update (attention_sharing.py:94-103, attn/utils.py:60-76) ------------------
  * For each head with decision == SP_DEC_DENSE: per-row cumulative-mass selection (>= threshold,

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "lib
 SP_DEC_VS, SP_DEC_DENSE, SP_DEC_SHARE, SP_DEC_QA = 0, 1, 2, 3
 SP_FLAG_LOGITS_BF16 = 1
 SP_POOL_TAIL_TRUE_LENGTH, SP_POOL_TAIL_RESCALE = 0, 1
+SP_ATTN_V_REPACKED = 1
 
 
 class ClusterStateStruct(C.Structure):
@@ -47,8 +48,9 @@ SIGNATURES = {
     "sp_queryaware_select_bf16": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _U32, _F, _P, _P, _P]),
     "sp_cover_select_global": (_I32, [_P, _P, _I32, _I32, _F, _P, _P]),
     "sp_attn_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32]),
+    "sp_attn_repack_v_bf16": (_I32, [_P, _I64, _I32, _I32, _I64, _I64, _I32, _P, _SZ, _P]),
     "sp_block_sparse_attn_fwd_bf16": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I64, _I64,
-                                             _I32, _F, _P, _P, _P, _P, _P, _SZ, _P]),
+                                             _I32, _F, _P, _P, _P, _P, _P, _SZ, _U32, _P]),
     "sp_pivot_update": (_I32, [_ST, _P, _P, _P, _I32, _I32, _F, _P]),
     "sp_cover_select_rows": (_I32, [_P, _I32, _F, _P, _P]),
     "sp_mask_row_pointers": (_I32, [_P, _I32, _I32, _P, _P]),

@@ -310,13 +310,32 @@ extern "C" size_t sp_attn_workspace_bytes(int64_t n, int32_t hkv, int32_t d, int
   return (size_t)hkv * nb * bs * d * sizeof(sp_bf16);
 }
 
+extern "C" int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n,
+                                     int64_t v_stride_h, int32_t bs, void* workspace, size_t workspace_bytes,
+                                     sp_stream_t stream) {
+  SP_REQUIRE(v && workspace, SP_ERR_INVALID_ARGUMENT, "sp_attn_repack_v_bf16: null pointer");
+  SP_REQUIRE(n > 0 && hkv > 0, SP_ERR_INVALID_ARGUMENT, "sp_attn_repack_v_bf16: bad shape");
+  SP_REQUIRE(bs == AT_BS && d == AT_D, SP_ERR_UNSUPPORTED,
+             "sp_attn_repack_v_bf16: block size %d / head_dim %d unsupported (only 128 / 128)", bs, d);
+  SP_REQUIRE(v_stride_n % 8 == 0 && v_stride_h % 8 == 0 && ((uintptr_t)v % 16) == 0 &&
+                 ((uintptr_t)workspace % 16) == 0,
+             SP_ERR_UNSUPPORTED, "sp_attn_repack_v_bf16: v must be 16-byte aligned, strides multiple of 8");
+  SP_REQUIRE(workspace_bytes >= sp_attn_workspace_bytes(n, hkv, d, bs), SP_ERR_WORKSPACE,
+             "sp_attn_repack_v_bf16: workspace too small");
+  const int64_t nb = sp_ceil_div(n, bs);
+  hipLaunchKernelGGL(sp_repack_v_kernel, dim3((unsigned)nb, hkv), dim3(AT_THREADS), 0, (hipStream_t)stream,
+                     (const sp_bf16*)v, (sp_bf16*)workspace, n, v_stride_n, v_stride_h, nb);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
 extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq,
                                              int32_t hkv, int32_t d, int64_t q_stride_n, int64_t q_stride_h,
                                              int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n,
                                              int64_t v_stride_h, int32_t bs, float softmax_scale,
                                              const uint64_t* mask, const int32_t* decision, void* out,
                                              float* avg_attn, void* workspace, size_t workspace_bytes,
-                                             sp_stream_t stream) {
+                                             uint32_t flags, sp_stream_t stream) {
   SP_REQUIRE(q && k && v && mask && out && workspace, SP_ERR_INVALID_ARGUMENT,
              "sp_block_sparse_attn_fwd_bf16: null pointer");
   SP_REQUIRE(n > 0 && hq > 0 && hkv > 0 && hq % hkv == 0, SP_ERR_INVALID_ARGUMENT,
@@ -325,21 +344,21 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
              bs);
   SP_REQUIRE(d == AT_D, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: head_dim %d unsupported (only 128)", d);
   SP_REQUIRE(q_stride_n % 8 == 0 && q_stride_h % 8 == 0 && k_stride_n % 8 == 0 && k_stride_h % 8 == 0 &&
-                 v_stride_n % 8 == 0 && v_stride_h % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 &&
-                 ((uintptr_t)v % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)workspace % 16) == 0,
+                 ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)out % 16) == 0,
              SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: tensors must be 16-byte aligned, strides multiple of 8");
   SP_REQUIRE(workspace_bytes >= sp_attn_workspace_bytes(n, hkv, d, bs), SP_ERR_WORKSPACE,
              "sp_block_sparse_attn_fwd_bf16: workspace too small");
   const int64_t nb = sp_ceil_div(n, bs);
   SP_REQUIRE(nb * hq < (1ll << 31), SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: grid too large");
-  hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_repack_v_kernel, dim3((unsigned)nb, hkv), dim3(AT_THREADS), 0, s, (const sp_bf16*)v,
-                     (sp_bf16*)workspace, n, v_stride_n, v_stride_h, nb);
-  SP_LAUNCH_CHECK();
+  if (!(flags & SP_ATTN_V_REPACKED)) {
+    int rc = sp_attn_repack_v_bf16(v, n, hkv, d, v_stride_n, v_stride_h, bs, workspace, workspace_bytes, stream);
+    if (rc != SP_OK) return rc;
+  }
   const float scale_log2 = softmax_scale * 1.4426950408889634f;
-  hipLaunchKernelGGL(sp_attn_fwd_kernel, dim3((unsigned)(nb * hq)), dim3(AT_THREADS), 0, s, (const sp_bf16*)q,
-                     (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out, avg_attn, n, hq, hkv,
-                     q_stride_n, q_stride_h, k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2);
+  hipLaunchKernelGGL(sp_attn_fwd_kernel, dim3((unsigned)(nb * hq)), dim3(AT_THREADS), 0, (hipStream_t)stream,
+                     (const sp_bf16*)q, (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out,
+                     avg_attn, n, hq, hkv, q_stride_n, q_stride_h, k_stride_n, k_stride_h, (int)nb,
+                     (int)((nb + 63) / 64), scale_log2);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

@@ -236,12 +236,45 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
     out = torch.empty(n, hq, d, dtype=torch.bfloat16, device=dev)
     need = lib.sp_attn_workspace_bytes(n, hkv, d, block_size)
     ws = _workspace("attn_vt", need, dev)
+    st = lib.sp_attn_repack_v_bf16(_ptr(v), n, hkv, d, v.stride(1), v.stride(0), block_size, _ptr(ws), ws.numel(),
+                                   _stream())
+    _lib.check(st, "sp_attn_repack_v_bf16")
+    timer = kernel_timer
+    if timer is not None:
+        timer.start("attn")
     st = lib.sp_block_sparse_attn_fwd_bf16(_ptr(q), _ptr(k), _ptr(v), n, hq, hkv, d, q.stride(1), q.stride(0),
                                            k.stride(1), k.stride(0), v.stride(1), v.stride(0), block_size,
                                            softmax_scale, _ptr(mask), _ptr(decision), _ptr(out), _ptr(avg_attn),
-                                           _ptr(ws), ws.numel(), _stream())
+                                           _ptr(ws), ws.numel(), _lib.SP_ATTN_V_REPACKED, _stream())
+    if timer is not None:
+        timer.stop("attn")
     _lib.check(st, "sp_block_sparse_attn_fwd_bf16")
     return out
+
+
+class KernelTimer:
+    """Brackets kernel launches with events on the stream they are launched on (torch's current stream).
+    Set ops.kernel_timer to an instance to collect; durations are read after a synchronise."""
+
+    def __init__(self):
+        self.events = {}
+        self._open = {}
+
+    def start(self, name: str):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record(torch.cuda.current_stream())
+        self._open[name] = ev
+
+    def stop(self, name: str):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record(torch.cuda.current_stream())
+        self.events.setdefault(name, []).append((self._open.pop(name), ev))
+
+    def durations_ms(self, name: str):
+        return [a.elapsed_time(b) for a, b in self.events.get(name, [])]
+
+
+kernel_timer: Optional[KernelTimer] = None
 
 
 def pivot_update(state: ClusterState, head_cluster, decision, avg_attn, pattern_threshold):
