@@ -218,7 +218,7 @@ def main():
         stages["pool_q_all_heads"] = event_ms(lambda: ops.pool_avg(qh, 128))
         kbar = ops.pool_avg(kh, 128)
         stages["queryaware_test"] = event_ms(lambda: ops.queryaware_test(qh, kbar, vb, 128, w.queryaware_threshold))
-        ws = ops._workspace("attn_vt", _lib.load().sp_attn_workspace_bytes(w.seq_len, w.hkv, w.head_dim, 128), dev)
+        ws = ops._workspace("attn_vt", _lib.load().sp_attn_workspace_bytes(w.seq_len, w.hq, w.hkv, w.head_dim, 128), dev)
         lib = _lib.load()
         stages["repack_v"] = event_ms(lambda: lib.sp_attn_repack_v_bf16(
             vh.data_ptr(), w.seq_len, w.hkv, w.head_dim, vh.stride(1), vh.stride(0), 128, ws.data_ptr(), ws.numel(),

@@ -154,11 +154,12 @@ int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec,
  * mask (and c <= r) are computed.  For heads with decision == SP_DEC_DENSE the block-averaged attention
  * map avg_attn[h][nb][nb] (fp32, pre-zeroed by the caller) is written as well (:425-457); decision and
  * avg_attn may both be NULL.
- * workspace: sp_attn_workspace_bytes(...) bytes of device scratch holding the key-major repack of V.
+ * workspace: sp_attn_workspace_bytes(...) bytes of device scratch (key-major repack of V, a work counter and
+ * the pivot heads' softmax row statistics).
  * sp_attn_repack_v_bf16 fills it; sp_block_sparse_attn_fwd_bf16 calls it first unless flags has
  * SP_ATTN_V_REPACKED (the caller already repacked this v into this workspace). */
 #define SP_ATTN_V_REPACKED 1u
-size_t sp_attn_workspace_bytes(int64_t n, int32_t hkv, int32_t d, int32_t bs);
+size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs);
 int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n, int64_t v_stride_h,
                           int32_t bs, void* workspace, size_t workspace_bytes, sp_stream_t stream);
 int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,

@@ -65,31 +65,58 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
   }
 }
 
-// ---- work-item -> (head, query block) mapping -------------------------------------------------------
-// Workgroups are handed to the 8 XCDs round-robin by linear id.  Each XCD (its own L2) is given the
-// query heads of one KV head at a time, heavy (late) rows first, the group's q heads interleaved, so
-// that workgroups running together read the same K / V^T tiles.
-__device__ static inline void at_map(int id, int hq, int hkv, int nb, int& h, int& r) {
-  const int group = hq / hkv;
-  int kvh, s;
-  if (hkv % 8 == 0) {
-    const int xcd = id & 7;
-    const int per = group * nb;  // items per kv head
-    s = id >> 3;
-    kvh = xcd + 8 * (s / per);
-    s = s % per;
-    h = kvh * group + (s % group);
-    r = nb - 1 - (s / group);
-  } else if (8 % hkv == 0 && nb % (8 / hkv) == 0) {
-    const int split = 8 / hkv;  // XCDs per kv head, rows dealt round-robin between them
-    const int xcd = id & 7;
-    s = id >> 3;
-    kvh = xcd / split;
-    h = kvh * group + (s % group);
-    r = nb - 1 - ((s / group) * split + (xcd % split));
-  } else {
-    h = id / nb;
-    r = nb - 1 - (id % nb);
+// ---- work distribution ----------------------------------------------------------------------------------
+// The kernel is persistent: 2 workgroups per CU pull items from an atomic counter.  Item order is
+// (kv head, query block descending, q head of the group), so at any moment the whole chip works on a few
+// hundred neighbouring rows of ONE kv head -- its K / V^T tiles stay hot in L2 / Infinity Cache -- and the
+// heavy (late) rows of a head are started first.  Dynamic pulling keeps the XCDs balanced although heads
+// differ widely in kept-block density.
+__device__ static inline void at_item(int id, int group, int nb, int& h, int& r) {
+  const int gi = id % group;
+  const int t = id / group;
+  r = nb - 1 - (t % nb);
+  h = (t / nb) * group + gi;
+}
+
+// ---- LDS staging -------------------------------------------------------------------------------------------
+// A block is processed as two sub-tiles of 64 keys.  One stage holds a K sub-tile [64 keys][16 chunks] and a
+// V^T sub-tile [128 channels][8 chunks] (chunk = 16 bytes = 8 bf16), 32 KiB; two stages are double-buffered.
+// Tiles are filled by direct global->LDS 128-bit loads: lane i of a wave writes LDS chunk (base + i), fetching
+// whichever global chunk belongs there.  Instead of row padding the chunk index is XOR-swizzled with the row,
+//   K  : chunk c of row r sits at r*16 + (c ^ (r & 15))
+//   V^T: chunk c of row r sits at r*8  + (c ^ ((r >> 1) & 7))
+// so the 16 lanes that read the same logical chunk of 16 consecutive rows hit 16 different bank groups.
+#define AT_SUB 64
+#define AT_KSTAGE_BYTES (AT_SUB * AT_D * 2)      // 16 KiB
+#define AT_VSTAGE_BYTES (AT_D * AT_SUB * 2)      // 16 KiB
+#define AT_STAGE_BYTES (AT_KSTAGE_BYTES + AT_VSTAGE_BYTES)
+
+typedef __attribute__((address_space(3))) void* at_lds_ptr;
+typedef const __attribute__((address_space(1))) void* at_gbl_ptr;
+
+__device__ static inline void at_issue_sub(const sp_bf16* __restrict__ kh, const sp_bf16* __restrict__ vth, int64_t n,
+                                           int64_t sk_n, int c, int half, char* stage, int wave, int lane) {
+  const int64_t key0 = (int64_t)c * AT_BS + half * AT_SUB;
+  const int64_t lim64 = n - 1 - key0;              // last valid row of this sub-tile (rows beyond are clamped)
+  const int lim = lim64 < 0 ? 0 : (lim64 > AT_SUB - 1 ? AT_SUB - 1 : (int)lim64);
+  const sp_bf16* kbase = kh + (lim64 < 0 ? (n - 1) : key0) * sk_n;
+  const sp_bf16* vbase = vth + (int64_t)c * AT_D * AT_BS + half * AT_SUB;
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int seg = it * 4 + wave;                 // 1 KiB segment of the tile handled by this wave-instruction
+    {
+      const int row = seg * 4 + (lane >> 4);
+      const int cl = (lane & 15) ^ (row & 15);
+      const int rowc = row < lim ? row : lim;
+      const sp_bf16* g = kbase + (uint32_t)(rowc * (int)sk_n + cl * 8);
+      __builtin_amdgcn_global_load_lds((at_gbl_ptr)g, (at_lds_ptr)(stage + seg * 1024), 16, 0, 0);
+    }
+    {
+      const int row = seg * 8 + (lane >> 3);
+      const int cl = (lane & 7) ^ ((row >> 1) & 7);
+      const sp_bf16* g = vbase + (uint32_t)(row * AT_BS + cl * 8);
+      __builtin_amdgcn_global_load_lds((at_gbl_ptr)g, (at_lds_ptr)(stage + AT_KSTAGE_BYTES + seg * 1024), 16, 0, 0);
+    }
   }
 }
 
@@ -100,214 +127,294 @@ __device__ static inline bf16x8 at_pack8(const floatx16& a, int base) {
   return __builtin_convertvector(f, bf16x8);
 }
 
+__device__ static inline bf16x8 at_lds128(const char* p) {
+  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+
+// iterator over the set bits (columns c <= r) of one mask row; uniform across the workgroup
+struct AtBlocks {
+  const uint64_t* row;
+  int r, w;
+  uint64_t word;
+  __device__ void init(const uint64_t* row_, int r_) {
+    row = row_;
+    r = r_;
+    w = 0;
+    word = fetch(0);
+  }
+  __device__ uint64_t fetch(int wi) const {
+    uint64_t x = row[wi];
+    if (wi == (r >> 6) && (r & 63) != 63) x &= (2ull << (r & 63)) - 1ull;
+    return x;
+  }
+  __device__ int next() {
+    while (word == 0) {
+      if (++w > (r >> 6)) return -1;
+      word = fetch(w);
+    }
+    const int c = w * 64 + __builtin_ctzll(word);
+    word &= word - 1;
+    return c;
+  }
+};
+
+#define AT_WAIT_VMCNT0() __builtin_amdgcn_s_waitcnt(0x0F70)  // vmcnt(0) only: the direct-to-LDS loads have landed
+
 __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ vt,
     const uint64_t* __restrict__ mask, const int32_t* __restrict__ decision, sp_bf16* __restrict__ out,
-    float* __restrict__ avg_attn, int64_t n, int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n,
-    int64_t sk_h, int nb, int nbw, float scale_log2) {
-  __shared__ sp_bf16 Ks[AT_BS * AT_PITCH];
-  __shared__ sp_bf16 Vs[AT_D * AT_PITCH];
-  __shared__ float wred[4];
+    float2* __restrict__ rowstat, int64_t n, int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n,
+    int64_t sk_h, int nb, int nbw, float scale_log2, int* __restrict__ work_counter, int total_items) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // 2 stages x 32 KiB
+  __shared__ int s_item;
 
-  int h, r;
-  at_map(blockIdx.x, hq, hkv, nb, h, r);
-  const int kvh = h / (hq / hkv);
+  const int group = hq / hkv;
   const int t = threadIdx.x;
   const int wave = t >> 6, lane = t & 63;
   const int lq = lane & 31, g = lane >> 5;
-  const int ld_row = t >> 4, ld_chunk = t & 15;
-
-  // Q^T operand: this lane's query, 8 k-steps of 8 channels
-  bf16x8 qb[8];
-  {
-    int64_t qrow = (int64_t)r * AT_BS + wave * 32 + lq;
-    if (qrow > n - 1) qrow = n - 1;
-    const sp_bf16* src = q + (int64_t)h * sq_h + qrow * sq_n + 8 * g;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qb[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 16 * ks));
-  }
-  const sp_bf16* kh = k + (int64_t)kvh * sk_h;
-  const sp_bf16* vth = vt + (int64_t)kvh * nb * AT_D * AT_BS;
-  const uint64_t* mrow = mask + ((int64_t)h * nb + r) * nbw;
-
-  floatx16 o[4];
-#pragma unroll
-  for (int dt = 0; dt < 4; ++dt) o[dt] = (floatx16){0};
-  float m_run = -INFINITY, l_run = 0.f;
   const int q_off = wave * 32 + lq;  // query offset inside the block
 
-  for (int w = 0; w <= (r >> 6); ++w) {
-    uint64_t word = mrow[w];
-    if (w == (r >> 6) && (r & 63) != 63) word &= (2ull << (r & 63)) - 1ull;  // only columns c <= r
-    while (word) {
-      const int c = w * 64 + __builtin_ctzll(word);
-      word &= word - 1;
-      // ---- stage K tile and V^T tile ----
+  // lane-constant LDS read offsets (bytes) inside a stage
+  int koff[8];  // K rows lq (+32 via immediate), logical chunk 2*ks + g
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) koff[ks] = lq * 256 + (((2 * ks + g) ^ (lq & 15)) << 4);
+  int voff[4];  // V^T rows lq (+32*dt via immediate), logical chunk 4*kt + 2*s + g, index kt*2+s
+#pragma unroll
+  for (int j = 0; j < 4; ++j) voff[j] = AT_KSTAGE_BYTES + lq * 128 + (((2 * j + g) ^ ((lq >> 1) & 7)) << 4);
+
+  for (;;) {
+    __syncthreads();  // previous item's LDS reads are done
+    if (t == 0) s_item = atomicAdd(work_counter, 1);
+    __syncthreads();
+    const int item = s_item;
+    if (item >= total_items) break;
+    int h, r;
+    at_item(item, group, nb, h, r);
+    const int kvh = h / group;
+    const sp_bf16* kh = k + (int64_t)kvh * sk_h;
+    const sp_bf16* vth = vt + (int64_t)kvh * nb * AT_D * AT_BS;
+    const uint64_t* mrow = mask + ((int64_t)h * nb + r) * nbw;
+
+    AtBlocks it;
+    it.init(mrow, r);
+    int c_cur = it.next();
+    int half = 0;
+    int buf = 0;
+    if (c_cur >= 0) at_issue_sub(kh, vth, n, sk_n, c_cur, 0, lds, wave, lane);
+
+    // Q^T operand: this lane's query, 8 k-steps of 8 channels
+    bf16x8 qb[8];
+    {
+      int64_t qrow = (int64_t)r * AT_BS + q_off;
+      if (qrow > n - 1) qrow = n - 1;
+      const sp_bf16* src = q + (int64_t)h * sq_h + qrow * sq_n + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks)
+        qb[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 16 * ks));
+    }
+
+    floatx16 o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) o[dt] = (floatx16){0};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    while (c_cur >= 0) {
+      // this sub-tile has landed (own loads), and every wave is past the previous sub-tile's compute
+      AT_WAIT_VMCNT0();
       __syncthreads();
-#pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int row = it * 16 + ld_row;
-        int64_t key = (int64_t)c * AT_BS + row;
-        if (key > n - 1) key = n - 1;
-        const uint4 kv = *reinterpret_cast<const uint4*>(kh + key * sk_n + ld_chunk * 8);
-        const uint4 vv = *reinterpret_cast<const uint4*>(vth + ((int64_t)c * AT_D + row) * AT_BS + ld_chunk * 8);
-        *reinterpret_cast<uint4*>(&Ks[row * AT_PITCH + ld_chunk * 8]) = kv;
-        *reinterpret_cast<uint4*>(&Vs[row * AT_PITCH + ld_chunk * 8]) = vv;
+      // ---- start fetching the next sub-tile into the other stage ----
+      int c_next = c_cur, half_next = 1;
+      if (half == 1) {
+        c_next = it.next();
+        half_next = 0;
       }
-      __syncthreads();
-      // ---- S^T = K . Q^T ----
-      floatx16 s[4];
+      if (c_next >= 0) at_issue_sub(kh, vth, n, sk_n, c_next, half_next, lds + (buf ^ 1) * AT_STAGE_BYTES, wave, lane);
+
+      const char* st = lds + buf * AT_STAGE_BYTES;
+      // ---- S^T = K . Q^T for 64 keys ----
+      floatx16 s[2];
+      s[0] = (floatx16){0};
+      s[1] = (floatx16){0};
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
-        floatx16 acc = (floatx16){0};
-        const sp_bf16* arow = &Ks[(kt * 32 + lq) * AT_PITCH + 8 * g];
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-          const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + 16 * ks));
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qb[ks], acc, 0, 0, 0);
-        }
-        s[kt] = acc;
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 x0 = at_lds128(st + koff[ks]);
+        const bf16x8 x1 = at_lds128(st + koff[ks] + 32 * 256);
+        s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x0, qb[ks], s[0], 0, 0, 0);
+        s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x1, qb[ks], s[1], 0, 0, 0);
       }
-      // ---- online softmax (base 2) ----
-      float mx = m_run;
-      if (c == r) {
+      // ---- online softmax (base 2): running max on raw logits, scale folded into the exponent ----
+      if (c_cur == r) {
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            const int key_off = kt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-            float v = s[kt][i] * scale_log2;
-            v = (key_off <= q_off) ? v : -INFINITY;
-            s[kt][i] = v;
-            mx = fmaxf(mx, v);
-          }
-      } else {
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const float v = s[kt][i] * scale_log2;
-            s[kt][i] = v;
-            mx = fmaxf(mx, v);
+            const int key_off = half * AT_SUB + kt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+            s[kt][i] = (key_off <= q_off) ? s[kt][i] : -INFINITY;
           }
       }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, SP_WAVE));
-      const float alpha = __builtin_amdgcn_exp2f(m_run - mx);
-      m_run = mx;
+      const float m_new = fmaxf(m_run, mx * scale_log2);
+      if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {  // some row's max moved: rescale
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        l_run *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+        m_run = m_new;
+      }
+      // a row with nothing unmasked so far keeps m_run = -inf; exp2(-inf - (-inf)) must not be evaluated
+      const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
       float psum = 0.f;
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const float p = __builtin_amdgcn_exp2f(s[kt][i] - mx);
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], scale_log2, -m_use));
           s[kt][i] = p;
           psum += p;
         }
-      l_run = l_run * alpha + psum;
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+      l_run += psum;
       // ---- O^T += V^T . P^T ----
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
+      for (int kt = 0; kt < 2; ++kt) {
         const bf16x8 p0 = at_pack8(s[kt], 0);
         const bf16x8 p1 = at_pack8(s[kt], 8);
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) {
-          const sp_bf16* arow = &Vs[(dt * 32 + lq) * AT_PITCH + kt * 32 + 8 * g];
-          const bf16x8 a0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow));
-          const bf16x8 a1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + 16));
+          const bf16x8 a0 = at_lds128(st + voff[kt * 2 + 0] + dt * 32 * 128);
+          const bf16x8 a1 = at_lds128(st + voff[kt * 2 + 1] + dt * 32 * 128);
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, p0, o[dt], 0, 0, 0);
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, p1, o[dt], 0, 0, 0);
         }
       }
+      buf ^= 1;
+      c_cur = c_next;
+      half = half_next;
     }
-  }
-  const float l_tot = l_run + __shfl_xor(l_run, 32, SP_WAVE);
+    const float l_tot = l_run + __shfl_xor(l_run, 32, SP_WAVE);
 
-  // ---- pivot heads: block-averaged attention map (second pass over the same blocks) ----
-  if (decision != nullptr && decision[h] == SP_DEC_DENSE && avg_attn != nullptr) {
-    const int64_t rem = n - (int64_t)r * AT_BS;
-    const int valid_q = rem < AT_BS ? (int)rem : AT_BS;
-    const bool q_valid = q_off < valid_q;
-    const float inv_l = 1.0f / l_tot;
-    float* arow_out = avg_attn + ((int64_t)h * nb + r) * nb;
-    for (int w = 0; w <= (r >> 6); ++w) {
-      uint64_t word = mrow[w];
-      if (w == (r >> 6) && (r & 63) != 63) word &= (2ull << (r & 63)) - 1ull;
-      while (word) {
-        const int c = w * 64 + __builtin_ctzll(word);
-        word &= word - 1;
-        __syncthreads();
-#pragma unroll
-        for (int it = 0; it < 8; ++it) {
-          const int row = it * 16 + ld_row;
-          int64_t key = (int64_t)c * AT_BS + row;
-          if (key > n - 1) key = n - 1;
-          *reinterpret_cast<uint4*>(&Ks[row * AT_PITCH + ld_chunk * 8]) =
-              *reinterpret_cast<const uint4*>(kh + key * sk_n + ld_chunk * 8);
-        }
-        __syncthreads();
-        float part = 0.f;
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-          floatx16 acc = (floatx16){0};
-          const sp_bf16* arow = &Ks[(kt * 32 + lq) * AT_PITCH + 8 * g];
-#pragma unroll
-          for (int ks = 0; ks < 8; ++ks) {
-            const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + 16 * ks));
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qb[ks], acc, 0, 0, 0);
-          }
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int key_off = kt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-            const bool ok = q_valid && (c < r || key_off <= q_off) && ((int64_t)c * AT_BS + key_off < n);
-            part += ok ? __builtin_amdgcn_exp2f(acc[i] * scale_log2 - m_run) * inv_l : 0.f;
-          }
-        }
-        part = sp_wave_sum(part);
-        if (lane == 0) wred[wave] = part;
-        __syncthreads();
-        if (t == 0) arow_out[c] = ((wred[0] + wred[1]) + (wred[2] + wred[3])) / (float)valid_q;
-      }
+    // pivot heads: keep the softmax statistics of every query row for the block-average pass
+    if (rowstat != nullptr && decision != nullptr && decision[h] == SP_DEC_DENSE && g == 0) {
+      const int64_t qrow = (int64_t)r * AT_BS + q_off;
+      if (qrow < n) rowstat[(int64_t)h * n + qrow] = make_float2(m_run, l_tot);
     }
-  }
 
-  // ---- epilogue: normalise, transpose through LDS, coalesced bf16 store ----
-  __syncthreads();
-  {
-    const float inv_l = 1.0f / l_tot;
-    sp_bf16* orow = &Ks[q_off * AT_PITCH];
+    // ---- epilogue: normalise, transpose through LDS (padded rows), coalesced bf16 store ----
+    __syncthreads();
+    {
+      const float inv_l = 1.0f / l_tot;
+      sp_bf16* orow = reinterpret_cast<sp_bf16*>(lds) + q_off * AT_PITCH;
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+      for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        const int d0 = dt * 32 + 8 * i4 + 4 * g;
-        const uint32_t b0 = sp_f32_to_bf16(o[dt][4 * i4 + 0] * inv_l);
-        const uint32_t b1 = sp_f32_to_bf16(o[dt][4 * i4 + 1] * inv_l);
-        const uint32_t b2 = sp_f32_to_bf16(o[dt][4 * i4 + 2] * inv_l);
-        const uint32_t b3 = sp_f32_to_bf16(o[dt][4 * i4 + 3] * inv_l);
-        *reinterpret_cast<uint2*>(orow + d0) = make_uint2(b0 | (b1 << 16), b2 | (b3 << 16));
+        for (int i4 = 0; i4 < 4; ++i4) {
+          const int d0 = dt * 32 + 8 * i4 + 4 * g;
+          const uint32_t b0 = sp_f32_to_bf16(o[dt][4 * i4 + 0] * inv_l);
+          const uint32_t b1 = sp_f32_to_bf16(o[dt][4 * i4 + 1] * inv_l);
+          const uint32_t b2 = sp_f32_to_bf16(o[dt][4 * i4 + 2] * inv_l);
+          const uint32_t b3 = sp_f32_to_bf16(o[dt][4 * i4 + 3] * inv_l);
+          *reinterpret_cast<uint2*>(orow + d0) = make_uint2(b0 | (b1 << 16), b2 | (b3 << 16));
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i8 = 0; i8 < 8; ++i8) {
+      const int row = i8 * 16 + (t >> 4);
+      const int64_t qrow = (int64_t)r * AT_BS + row;
+      if (qrow < n) {
+        *reinterpret_cast<uint4*>(out + (qrow * hq + h) * AT_D + (t & 15) * 8) =
+            *reinterpret_cast<const uint4*>(reinterpret_cast<sp_bf16*>(lds) + row * AT_PITCH + (t & 15) * 8);
       }
-  }
-  __syncthreads();
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int row = it * 16 + ld_row;
-    const int64_t qrow = (int64_t)r * AT_BS + row;
-    if (qrow < n) {
-      *reinterpret_cast<uint4*>(out + (qrow * hq + h) * AT_D + ld_chunk * 8) =
-          *reinterpret_cast<const uint4*>(&Ks[row * AT_PITCH + ld_chunk * 8]);
     }
   }
 }
 
+__global__ void sp_zero_i32_kernel(int* p) { *p = 0; }
+
+// ---- pivot heads: block-averaged attention map (shareprefill_attn.py:425-457) ---------------------------
+// avg[h][r][c] = mean over the valid queries of block r of the softmax mass that falls into key block c,
+// recomputed from the row statistics the forward kernel left behind.  One workgroup per (query block, head);
+// heads that are not pivots leave at once.
+__global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_kernel(
+    const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const uint64_t* __restrict__ mask,
+    const int32_t* __restrict__ decision, const float2* __restrict__ rowstat, float* __restrict__ avg_attn, int64_t n,
+    int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n, int64_t sk_h, int nb, int nbw, float scale_log2) {
+  __shared__ sp_bf16 Ks[AT_BS * AT_PITCH];
+  __shared__ float wred[4];
+  const int r = nb - 1 - blockIdx.x, h = blockIdx.y;
+  if (decision[h] != SP_DEC_DENSE) return;
+  const int kvh = h / (hq / hkv);
+  const int t = threadIdx.x;
+  const int wave = t >> 6, lane = t & 63;
+  const int lq = lane & 31, g = lane >> 5;
+  const int q_off = wave * 32 + lq;
+  const int64_t rem = n - (int64_t)r * AT_BS;
+  const int valid_q = rem < AT_BS ? (int)rem : AT_BS;
+  const bool q_valid = q_off < valid_q;
+  int64_t qrow = (int64_t)r * AT_BS + q_off;
+  if (qrow > n - 1) qrow = n - 1;
+  bf16x8 qb[8];
+  {
+    const sp_bf16* src = q + (int64_t)h * sq_h + qrow * sq_n + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qb[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 16 * ks));
+  }
+  const float2 st = rowstat[(int64_t)h * n + qrow];
+  const float m_row = st.x, inv_l = 1.0f / st.y;
+  const sp_bf16* kh = k + (int64_t)kvh * sk_h;
+  float* arow_out = avg_attn + ((int64_t)h * nb + r) * nb;
+  AtBlocks it;
+  it.init(mask + ((int64_t)h * nb + r) * nbw, r);
+  for (int c = it.next(); c >= 0; c = it.next()) {
+    __syncthreads();
+#pragma unroll
+    for (int i8 = 0; i8 < 8; ++i8) {
+      const int row = i8 * 16 + (t >> 4);
+      int64_t key = (int64_t)c * AT_BS + row;
+      if (key > n - 1) key = n - 1;
+      *reinterpret_cast<uint4*>(&Ks[row * AT_PITCH + (t & 15) * 8]) =
+          *reinterpret_cast<const uint4*>(kh + key * sk_n + (t & 15) * 8);
+    }
+    __syncthreads();
+    float part = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      floatx16 acc = (floatx16){0};
+      const sp_bf16* arow = &Ks[(kt * 32 + lq) * AT_PITCH + 8 * g];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + 16 * ks));
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qb[ks], acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key_off = kt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+        const bool ok = q_valid && (c < r || key_off <= q_off) && ((int64_t)c * AT_BS + key_off < n);
+        part += ok ? __builtin_amdgcn_exp2f(__builtin_fmaf(acc[i], scale_log2, -m_row)) * inv_l : 0.f;
+      }
+    }
+    part = sp_wave_sum(part);
+    if (lane == 0) wred[wave] = part;
+    __syncthreads();
+    if (t == 0) arow_out[c] = ((wred[0] + wred[1]) + (wred[2] + wred[3])) / (float)valid_q;
+  }
+}
+
 // ---- host ---------------------------------------------------------------------------------------------
-extern "C" size_t sp_attn_workspace_bytes(int64_t n, int32_t hkv, int32_t d, int32_t bs) {
-  if (n <= 0 || hkv <= 0 || d <= 0 || bs <= 0) return 0;
-  const int64_t nb = sp_ceil_div(n, bs);
-  return (size_t)hkv * nb * bs * d * sizeof(sp_bf16);
+// workspace layout: [ repacked V^T : hkv*nb*128*128 bf16 | work counter : 256 B | row statistics : hq*n float2 ]
+static size_t at_vt_bytes(int64_t n, int32_t hkv, int32_t d, int32_t bs) {
+  return (size_t)hkv * (size_t)sp_ceil_div(n, bs) * bs * d * sizeof(sp_bf16);
+}
+
+extern "C" size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs) {
+  if (n <= 0 || hq <= 0 || hkv <= 0 || d <= 0 || bs <= 0) return 0;
+  return at_vt_bytes(n, hkv, d, bs) + 256 + (size_t)hq * (size_t)n * sizeof(float2);
 }
 
 extern "C" int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n,
@@ -320,7 +427,7 @@ extern "C" int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int3
   SP_REQUIRE(v_stride_n % 8 == 0 && v_stride_h % 8 == 0 && ((uintptr_t)v % 16) == 0 &&
                  ((uintptr_t)workspace % 16) == 0,
              SP_ERR_UNSUPPORTED, "sp_attn_repack_v_bf16: v must be 16-byte aligned, strides multiple of 8");
-  SP_REQUIRE(workspace_bytes >= sp_attn_workspace_bytes(n, hkv, d, bs), SP_ERR_WORKSPACE,
+  SP_REQUIRE(workspace_bytes >= at_vt_bytes(n, hkv, d, bs), SP_ERR_WORKSPACE,
              "sp_attn_repack_v_bf16: workspace too small");
   const int64_t nb = sp_ceil_div(n, bs);
   hipLaunchKernelGGL(sp_repack_v_kernel, dim3((unsigned)nb, hkv), dim3(AT_THREADS), 0, (hipStream_t)stream,
@@ -340,13 +447,16 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
              "sp_block_sparse_attn_fwd_bf16: null pointer");
   SP_REQUIRE(n > 0 && hq > 0 && hkv > 0 && hq % hkv == 0, SP_ERR_INVALID_ARGUMENT,
              "sp_block_sparse_attn_fwd_bf16: bad shape n=%lld hq=%d hkv=%d", (long long)n, hq, hkv);
+  SP_REQUIRE(softmax_scale > 0.f, SP_ERR_INVALID_ARGUMENT, "sp_block_sparse_attn_fwd_bf16: softmax_scale must be > 0");
   SP_REQUIRE(bs == AT_BS, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: block size %d unsupported (only 128)",
              bs);
   SP_REQUIRE(d == AT_D, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: head_dim %d unsupported (only 128)", d);
   SP_REQUIRE(q_stride_n % 8 == 0 && q_stride_h % 8 == 0 && k_stride_n % 8 == 0 && k_stride_h % 8 == 0 &&
                  ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)out % 16) == 0,
              SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: tensors must be 16-byte aligned, strides multiple of 8");
-  SP_REQUIRE(workspace_bytes >= sp_attn_workspace_bytes(n, hkv, d, bs), SP_ERR_WORKSPACE,
+  SP_REQUIRE((int64_t)AT_BS * k_stride_n < (1ll << 31), SP_ERR_UNSUPPORTED,
+             "sp_block_sparse_attn_fwd_bf16: key token stride %lld too large", (long long)k_stride_n);
+  SP_REQUIRE(workspace_bytes >= sp_attn_workspace_bytes(n, hq, hkv, d, bs), SP_ERR_WORKSPACE,
              "sp_block_sparse_attn_fwd_bf16: workspace too small");
   const int64_t nb = sp_ceil_div(n, bs);
   SP_REQUIRE(nb * hq < (1ll << 31), SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: grid too large");
@@ -355,10 +465,36 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
     if (rc != SP_OK) return rc;
   }
   const float scale_log2 = softmax_scale * 1.4426950408889634f;
-  hipLaunchKernelGGL(sp_attn_fwd_kernel, dim3((unsigned)(nb * hq)), dim3(AT_THREADS), 0, (hipStream_t)stream,
-                     (const sp_bf16*)q, (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out,
-                     avg_attn, n, hq, hkv, q_stride_n, q_stride_h, k_stride_n, k_stride_h, (int)nb,
-                     (int)((nb + 63) / 64), scale_log2);
+  char* ws = (char*)workspace;
+  int* counter = reinterpret_cast<int*>(ws + at_vt_bytes(n, hkv, d, bs));
+  float2* rowstat = reinterpret_cast<float2*>(ws + at_vt_bytes(n, hkv, d, bs) + 256);
+  const bool want_avg = decision != nullptr && avg_attn != nullptr;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(sp_zero_i32_kernel, dim3(1), dim3(1), 0, s, counter);
   SP_LAUNCH_CHECK();
+  const size_t lds_bytes = 2 * AT_STAGE_BYTES;
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    SP_HIP(hipGetDevice(&dev));
+    SP_HIP(hipGetDeviceProperties(&prop, dev));
+    SP_HIP(hipFuncSetAttribute((const void*)sp_attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)lds_bytes));
+    n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }
+  const int64_t total = nb * hq;
+  const int grid = (int)(total < 2ll * n_cu ? total : 2ll * n_cu);
+  hipLaunchKernelGGL(sp_attn_fwd_kernel, dim3(grid), dim3(AT_THREADS), lds_bytes, s, (const sp_bf16*)q,
+                     (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out,
+                     want_avg ? rowstat : (float2*)nullptr, n, hq, hkv, q_stride_n, q_stride_h, k_stride_n,
+                     k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, counter, (int)total);
+  SP_LAUNCH_CHECK();
+  if (want_avg) {
+    hipLaunchKernelGGL(sp_attn_avg_kernel, dim3((unsigned)nb, hq), dim3(AT_THREADS), 0, s, (const sp_bf16*)q,
+                       (const sp_bf16*)k, mask, decision, rowstat, avg_attn, n, hq, hkv, q_stride_n, q_stride_h,
+                       k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2);
+    SP_LAUNCH_CHECK();
+  }
   return SP_OK;
 }

@@ -234,7 +234,7 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
     assert mask.is_contiguous() and mask.dtype == torch.int64
     dev = q.device
     out = torch.empty(n, hq, d, dtype=torch.bfloat16, device=dev)
-    need = lib.sp_attn_workspace_bytes(n, hkv, d, block_size)
+    need = lib.sp_attn_workspace_bytes(n, hq, hkv, d, block_size)
     ws = _workspace("attn_vt", need, dev)
     st = lib.sp_attn_repack_v_bf16(_ptr(v), n, hkv, d, v.stride(1), v.stride(0), block_size, _ptr(ws), ws.numel(),
                                    _stream())
