@@ -9,7 +9,9 @@ from __future__ import annotations
 import ctypes as C
 import os
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libshareprefill_hip.so")
+# SHAREPREFILL_HIP_LIB overrides the in-tree library path (e.g. to try an experimental build)
+LIB_PATH = os.environ.get("SHAREPREFILL_HIP_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc",
+                                                                  "libshareprefill_hip.so")
 
 SP_DEC_VS, SP_DEC_DENSE, SP_DEC_SHARE, SP_DEC_QA = 0, 1, 2, 3
 SP_FLAG_LOGITS_BF16 = 1

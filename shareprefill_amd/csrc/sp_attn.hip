@@ -231,16 +231,27 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
       if (c_next >= 0) at_issue_sub(kh, vth, n, sk_n, c_next, half_next, lds + (buf ^ 1) * AT_STAGE_BYTES, wave, lane);
 
       const char* st = lds + buf * AT_STAGE_BYTES;
-      // ---- S^T = K . Q^T for 64 keys ----
+      // ---- S^T = K . Q^T for 64 keys; LDS operands are fetched two k-steps ahead of their MFMAs ----
       floatx16 s[2];
       s[0] = (floatx16){0};
       s[1] = (floatx16){0};
+      {
+        bf16x8 xa[3][2];
+        xa[0][0] = at_lds128(st + koff[0]);
+        xa[0][1] = at_lds128(st + koff[0] + 32 * 256);
+        xa[1][0] = at_lds128(st + koff[1]);
+        xa[1][1] = at_lds128(st + koff[1] + 32 * 256);
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const bf16x8 x0 = at_lds128(st + koff[ks]);
-        const bf16x8 x1 = at_lds128(st + koff[ks] + 32 * 256);
-        s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x0, qb[ks], s[0], 0, 0, 0);
-        s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x1, qb[ks], s[1], 0, 0, 0);
+        for (int ks = 0; ks < 8; ++ks) {
+          if (ks + 2 < 8) {
+            xa[(ks + 2) % 3][0] = at_lds128(st + koff[ks + 2]);
+            xa[(ks + 2) % 3][1] = at_lds128(st + koff[ks + 2] + 32 * 256);
+          }
+          s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[ks % 3][0], qb[ks], s[0], 0, 0, 0);
+          s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[ks % 3][1], qb[ks], s[1], 0, 0, 0);
+        }
+        __builtin_amdgcn_s_setprio(0);
       }
       // ---- online softmax (base 2): running max on raw logits, scale folded into the exponent ----
       if (c_cur == r) {
@@ -280,18 +291,29 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
           psum += p;
         }
       l_run += psum;
-      // ---- O^T += V^T . P^T ----
+      // ---- O^T += V^T . P^T; V^T operands fetched one (kt, dt) step ahead ----
+      {
+        bf16x8 pb[2][2];
+        pb[0][0] = at_pack8(s[0], 0);
+        pb[0][1] = at_pack8(s[0], 8);
+        pb[1][0] = at_pack8(s[1], 0);
+        pb[1][1] = at_pack8(s[1], 8);
+        bf16x8 va[2][2];
+        va[0][0] = at_lds128(st + voff[0]);
+        va[0][1] = at_lds128(st + voff[1]);
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-        const bf16x8 p0 = at_pack8(s[kt], 0);
-        const bf16x8 p1 = at_pack8(s[kt], 8);
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-          const bf16x8 a0 = at_lds128(st + voff[kt * 2 + 0] + dt * 32 * 128);
-          const bf16x8 a1 = at_lds128(st + voff[kt * 2 + 1] + dt * 32 * 128);
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, p0, o[dt], 0, 0, 0);
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, p1, o[dt], 0, 0, 0);
+        for (int step = 0; step < 8; ++step) {  // step = kt*4 + dt
+          const int kt = step >> 2, dt = step & 3;
+          if (step + 1 < 8) {
+            const int kt1 = (step + 1) >> 2, dt1 = (step + 1) & 3;
+            va[(step + 1) & 1][0] = at_lds128(st + voff[kt1 * 2 + 0] + dt1 * 32 * 128);
+            va[(step + 1) & 1][1] = at_lds128(st + voff[kt1 * 2 + 1] + dt1 * 32 * 128);
+          }
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[step & 1][0], pb[kt][0], o[dt], 0, 0, 0);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[step & 1][1], pb[kt][1], o[dt], 0, 0, 0);
         }
+        __builtin_amdgcn_s_setprio(0);
       }
       buf ^= 1;
       c_cur = c_next;

@@ -1,0 +1,65 @@
+"""GPU: SharePrefill(...)(model) on a small random-init Hugging Face Llama: the patched model runs prefill through
+the HIP path (no N x N mask is built), matches the eager model when the budgets keep every block, and can decode."""
+
+import json
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def small_llama(layers=2, hq=4, hkv=2):
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    cfg = LlamaConfig(hidden_size=hq * 128, intermediate_size=1024, num_hidden_layers=layers, num_attention_heads=hq,
+                      num_key_value_heads=hkv, head_dim=128, vocab_size=512, max_position_embeddings=8192)
+    torch.manual_seed(0)
+    return LlamaForCausalLM(cfg)
+
+
+def table(tmp_path, layers, hq):
+    t = {"clusters": {"0": [[l, h] for l in range(layers) for h in range(hq // 2)],
+                      "1": [[l, h] for l in range(layers) for h in range(hq // 2, hq)]}, "shared_clusters": ["0", "1"]}
+    p = tmp_path / "table.json"
+    p.write_text(json.dumps(t))
+    return str(p)
+
+
+def test_patched_model_matches_eager_when_every_block_is_kept(gpu_device, tmp_path):
+    from shareprefill_amd import SharePrefill
+
+    n = 1024
+    ids = torch.randint(0, 512, (1, n), generator=torch.Generator().manual_seed(1)).to(gpu_device)
+    ref_model = small_llama().to(gpu_device, torch.bfloat16)
+    ref_model.config._attn_implementation = "eager"
+    with torch.no_grad():
+        ref = ref_model(ids).logits.float()
+    model = SharePrefill(sharing_lookup_path=table(tmp_path, 2, 4), min_budget=8192)(
+        small_llama().to(gpu_device, torch.bfloat16))
+    with torch.no_grad():
+        out = model(ids, use_cache=False).logits.float()
+    assert out.shape == ref.shape
+    assert (out - ref).abs().max().item() < 0.15 and ((out - ref).abs().mean() / ref.abs().mean()).item() < 2e-2
+    hist = model.attention_sharing.decision_histogram()
+    assert sum(hist.values()) == 8 and hist["dense_pivot"] <= 2  # 2 layers x 4 heads, at most one pivot per cluster
+    # a second forward resets the sharing state and gives the same result
+    with torch.no_grad():
+        out2 = model(ids, use_cache=False).logits.float()
+    assert torch.equal(out, out2)
+
+
+def test_patched_model_sparse_prefill_and_generate(gpu_device, tmp_path):
+    from shareprefill_amd import SharePrefill
+
+    model = SharePrefill(sharing_lookup_path=table(tmp_path, 2, 4), pattern_threshold=0.9, min_budget=256)(
+        small_llama().to(gpu_device, torch.bfloat16))
+    ids = torch.randint(0, 512, (1, 2048), generator=torch.Generator().manual_seed(2)).to(gpu_device)
+    with torch.no_grad():
+        logits = model(ids, use_cache=False, logits_to_keep=1).logits
+    assert logits.shape == (1, 1, 512) and torch.isfinite(logits).all()
+    dens = [p.density().cpu() for p in model.attention_sharing.plans]
+    assert len(dens) == 2 and all((d > 0).all() and (d <= 1).all() for d in dens)
+    with torch.no_grad():
+        gen = model.generate(ids[:, :300], max_new_tokens=4, do_sample=False)
+    assert gen.shape == (1, 304)

@@ -1,0 +1,220 @@
+"""CPU-only checks: the C-ABI library loads and exports every symbol the header declares, the ctypes
+signatures cover the header, host-side configuration / table loading / patching behave like the reference's
+(shareprefill/shareprefill_patch.py, shareprefill_configurations.py, attn/attention_sharing.py:368-384)."""
+
+import ctypes
+import json
+import os
+import re
+import types
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "shareprefill_hip.h")
+
+
+def header_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sp_[a-z0-9_]+)\s*\(", text)) - {"sp_cluster_state"})
+
+
+def test_library_exports_every_declared_symbol():
+    from shareprefill_amd import _lib
+
+    assert os.path.exists(_lib.LIB_PATH), "build the library first: python -m shareprefill_amd.build"
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    names = header_functions()
+    assert len(names) >= 19
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == names, "ctypes signature table and header disagree"
+
+
+def test_library_identity_and_error_string():
+    from shareprefill_amd import _lib
+
+    lib = _lib.load()
+    assert lib.sp_version() >= 1
+    assert lib.sp_arch() == b"gfx950"
+    # argument validation happens on the host before any GPU call: usable without a GPU
+    st = lib.sp_pool_avg_bf16(None, None, 128, 1, 128, 128, 128, 128, 0, None, None)
+    assert st == -1 and b"null" in lib.sp_last_error()
+    with pytest.raises(ValueError):
+        _lib.check(st, "sp_pool_avg_bf16")
+    assert lib.sp_lastq_scores_workspace_bytes(131072, 32, 128) == (32 * 128 * 128 + 32 * 128) * 8
+    assert lib.sp_attn_workspace_bytes(131072, 32, 8, 128, 128) == 8 * 131072 * 128 * 2 + 256 + 32 * 131072 * 8
+
+
+def test_cluster_state_struct_matches_header_layout():
+    from shareprefill_amd._lib import ClusterStateStruct
+
+    assert ctypes.sizeof(ClusterStateStruct) == 16 + 8 * 8
+    assert [f[0] for f in ClusterStateStruct._fields_][4:] == ["info", "ratio", "vert", "slash", "cols", "dists",
+                                                              "pattern", "accum"]
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    from shareprefill_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    with pytest.raises(_lib.SharePrefillLibraryError, match="no CPU fallback"):
+        _lib.load(str(tmp_path / "missing.so"))
+    monkeypatch.setattr(_lib, "_lib", None)
+
+
+def test_cpu_tensors_are_rejected_not_silently_computed():
+    from shareprefill_amd import ops
+
+    x = torch.zeros(2, 256, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="GPU"):
+        ops.pool_avg(x, 128)
+
+
+# ---- configuration ---------------------------------------------------------------------------------
+def test_config_defaults_and_registry():
+    from shareprefill_amd import SharePrefillConfig
+
+    c = SharePrefillConfig(model_name="meta-llama/Llama-3.1-8B-Instruct")
+    assert (c.pattern_threshold, c.similarity_threshold, c.fallback_threshold, c.queryaware_threshold) == (
+        0.9, 0.5, 0.9, 0.1)
+    assert (c.block_size, c.min_budget, c.max_budget) == (128, 1024, None)
+    assert c.sharing_lookup_path.endswith("Llama-3.1-8B-Instruct_code_debug_hiera-40.0-2.json")
+    assert os.path.exists(c.sharing_lookup_path)
+    with pytest.raises(AssertionError):
+        SharePrefillConfig(model_name="org/unknown-model")
+    with pytest.raises(AssertionError):
+        SharePrefillConfig(attn_type="other", model_name="x")
+    with pytest.raises(AssertionError):
+        SharePrefillConfig()
+    assert SharePrefillConfig(sharing_lookup_path="/x/y.json").sharing_lookup_path == "/x/y.json"
+
+
+def test_shipped_table_properties():
+    from shareprefill_amd import AttentionSharing, SharePrefillConfig
+
+    path = SharePrefillConfig(model_name="Llama-3.1-8B-Instruct").sharing_lookup_path
+    clusters, shared = AttentionSharing.load_clusters(path)
+    pairs = [tuple(p) for v in clusters.values() for p in v]
+    assert len(clusters) == 44 and len(pairs) == 1024 and len(set(pairs)) == 1024
+    assert shared == {"9"} and len(clusters["9"]) == 42
+    assert {l for l, _ in clusters["9"]} <= set(range(14, 31))
+    sh = AttentionSharing(path)
+    for cid, v in clusters.items():
+        for layer, head in v[:3]:
+            assert sh.find_cluster_id(layer, head) == cid
+    assert sh.find_cluster_id(99, 0) is None
+
+
+def test_table_loader_errors(tmp_path):
+    from shareprefill_amd import AttentionSharing
+
+    with pytest.raises(FileNotFoundError):
+        AttentionSharing(str(tmp_path / "nope.json"))
+    bad = tmp_path / "bad.json"
+    bad.write_text(json.dumps({"clusters": {}}))
+    with pytest.raises(ValueError):
+        AttentionSharing(str(bad))
+
+
+def test_budget_conversion():
+    from shareprefill_amd.attention_sharing import budget_blocks
+
+    assert budget_blocks(1024, None, 128) == (8, (2 ** 31 - 1 + 127) // 128)
+    assert budget_blocks(None, 1000, 128) == (1, 8)
+    assert budget_blocks(129, 4096, 128) == (2, 32)
+
+
+# ---- patching a Hugging Face model -------------------------------------------------------------------
+def tiny_llama():
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    cfg = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
+                      num_key_value_heads=1, head_dim=128, vocab_size=128, max_position_embeddings=4096)
+    torch.manual_seed(0)
+    return LlamaForCausalLM(cfg)
+
+
+def tiny_table(tmp_path):
+    t = {"clusters": {"0": [[0, 0], [1, 0]], "1": [[0, 1], [1, 1]]}, "shared_clusters": ["0"]}
+    p = tmp_path / "table.json"
+    p.write_text(json.dumps(t))
+    return str(p)
+
+
+def test_patch_installs_reference_hooks(tmp_path):
+    from shareprefill_amd import AttentionSharing, SharePrefill, shareprefill_attention_forward
+    from transformers.models.llama import modeling_llama
+
+    model = tiny_llama()
+    patched = SharePrefill(sharing_lookup_path=tiny_table(tmp_path), pattern_threshold=0.95, min_budget=256)(model)
+    assert patched is model
+    assert model.config._attn_implementation == "shareprefill"
+    assert modeling_llama.ALL_ATTENTION_FUNCTIONS["shareprefill"] is shareprefill_attention_forward
+    assert isinstance(model.attention_sharing, AttentionSharing)
+    assert callable(model.reset_attention_sharing) and callable(model._init_attention_sharing)
+    # thresholds are pushed onto the shared HF config, every attention module sees the same state object
+    assert model.config.pattern_threshold == 0.95 and model.config.min_budget == 256 and model.config.block_size == 128
+    for layer in model.model.layers:
+        assert layer.self_attn.attention_sharing is model.attention_sharing
+        assert layer.self_attn.config is model.config
+
+
+def test_patched_forward_resets_state_and_has_no_cpu_path(tmp_path):
+    from shareprefill_amd import SharePrefill
+
+    model = SharePrefill(sharing_lookup_path=tiny_table(tmp_path))(tiny_llama()).to(torch.bfloat16)
+    calls = []
+    orig = model.attention_sharing.reset_state
+    model.attention_sharing.reset_state = lambda: (calls.append(1), orig())[1]
+    ids = torch.randint(0, 128, (1, 256))
+    # the attention function reaches the HIP ops, which refuse CPU tensors: no silent fallback
+    with pytest.raises(ValueError, match="GPU"):
+        model(ids)
+    assert len(calls) == 1
+
+
+def test_patch_rejects_unsupported_models_and_types(tmp_path):
+    from shareprefill_amd import SharePrefill
+
+    with pytest.raises(TypeError):
+        SharePrefill(sharing_lookup_path=tiny_table(tmp_path))(torch.nn.Linear(2, 2))
+    sp = SharePrefill(sharing_lookup_path=tiny_table(tmp_path))
+    sp.config.attn_type = "flash"
+    with pytest.raises(ValueError):
+        sp(tiny_llama())
+
+
+def test_attention_forward_argument_errors(tmp_path):
+    from shareprefill_amd import AttentionSharing, shareprefill_attention_forward
+
+    cfg = types.SimpleNamespace(block_size=128, min_budget=1024, max_budget=None, pattern_threshold=0.9,
+                                similarity_threshold=0.5, fallback_threshold=0.9, queryaware_threshold=0.1)
+    mod = types.SimpleNamespace(config=cfg, attention_sharing=AttentionSharing(tiny_table(tmp_path)), layer_idx=0,
+                                scaling=0.1)
+    q = torch.zeros(1, 2, 256, 128, dtype=torch.bfloat16)
+    k = torch.zeros(1, 1, 256, 128, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        shareprefill_attention_forward(mod, q, k, k, None, scaling=0.1, sliding_window=128)
+    with pytest.raises(NotImplementedError):
+        shareprefill_attention_forward(mod, q, k, k, None, scaling=0.1, gqa_interleave=True)
+    with pytest.raises(ValueError):
+        shareprefill_attention_forward(mod, q.expand(2, -1, -1, -1), k.expand(2, -1, -1, -1), k.expand(2, -1, -1, -1),
+                                       None, scaling=0.1)
+    with pytest.raises(AssertionError):
+        shareprefill_attention_forward(mod, q.float(), k.float(), k.float(), None, scaling=0.1)
+    with pytest.raises(AssertionError):
+        shareprefill_attention_forward(mod, q, k[:, :, :128], k[:, :, :128], None, scaling=0.1)
+
+
+def test_synthetic_tables_and_generator_are_seeded():
+    from shareprefill_amd import synthetic
+
+    a = synthetic.random_cluster_table(32, 8, 2, 5)
+    assert a == synthetic.random_cluster_table(32, 8, 2, 5)
+    assert sorted(h for c in a["clusters"].values() for l, h in c if l == 0) == list(range(32))
+    q1, k1, v1 = synthetic.planted_qkv(4, 2, 512, 128, 3)
+    q2, _, _ = synthetic.planted_qkv(4, 2, 512, 128, 3)
+    assert torch.equal(q1, q2) and q1.shape == (1, 4, 512, 128) and q1.stride(3) == 1 and q1.stride(1) == 128
