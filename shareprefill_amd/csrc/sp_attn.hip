@@ -66,16 +66,36 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 }
 
 // ---- work distribution ----------------------------------------------------------------------------------
-// The kernel is persistent: 2 workgroups per CU pull items from an atomic counter.  Item order is
-// (kv head, query block descending, q head of the group), so at any moment the whole chip works on a few
-// hundred neighbouring rows of ONE kv head -- its K / V^T tiles stay hot in L2 / Infinity Cache -- and the
-// heavy (late) rows of a head are started first.  Dynamic pulling keeps the XCDs balanced although heads
-// differ widely in kept-block density.
-__device__ static inline void at_item(int id, int group, int nb, int& h, int& r) {
-  const int gi = id % group;
-  const int t = id / group;
-  r = nb - 1 - (t % nb);
-  h = (t / nb) * group + gi;
+// The kernel is persistent, 2 workgroups per CU.  Work items are (head, query block) rows, grouped in gangs of
+// AT_GANG consecutive query blocks of ONE head.  Gangs are dealt statically to the 8 XCDs (queue x = gang
+// position % 8; workgroup b serves queue b % 8 first -- workgroups are placed on XCDs round-robin), so the
+// 64 workgroups of an XCD start a gang together at column 0 and sweep the key blocks nearly in lock-step:
+// every K / V^T tile one of them pulls into the XCD's L2 is hit by the others.  The head order inside a kv
+// group is rotated from chunk to chunk so that every queue sees every head, heavy (late) rows go first, and a
+// workgroup whose queue is empty steals from the other queues.  Pulling is by atomic tickets only: nobody
+// ever waits for anybody, and every workgroup leaves once all eight queues are exhausted.
+#define AT_GANG 64
+
+struct AtGeom {
+  int group, nb, n_chunks, n_gangs;
+};
+
+__device__ static inline int at_queue_items(const AtGeom& gm, int xq) {
+  const int gangs = gm.n_gangs > xq ? (gm.n_gangs - xq + 7) / 8 : 0;
+  return gangs * AT_GANG;
+}
+
+// ticket of queue xq -> (head, query block); false for the padding slots of the last row chunk
+__device__ static inline bool at_item(const AtGeom& gm, int xq, int ticket, int& h, int& r) {
+  const int pos = (ticket / AT_GANG) * 8 + xq;  // gang position
+  const int slot = ticket % AT_GANG;
+  const int i = pos % gm.group;
+  const int rest = pos / gm.group;
+  const int j = rest % gm.n_chunks;  // row chunk, 0 = the last (heaviest) rows
+  const int kvh = rest / gm.n_chunks;
+  h = kvh * gm.group + (i + j) % gm.group;
+  r = gm.nb - 1 - (j * AT_GANG + slot);
+  return r >= 0;
 }
 
 // ---- LDS staging -------------------------------------------------------------------------------------------
@@ -94,28 +114,50 @@ __device__ static inline void at_item(int id, int group, int nb, int& h, int& r)
 typedef __attribute__((address_space(3))) void* at_lds_ptr;
 typedef const __attribute__((address_space(1))) void* at_gbl_ptr;
 
-__device__ static inline void at_issue_sub(const sp_bf16* __restrict__ kh, const sp_bf16* __restrict__ vth, int64_t n,
-                                           int64_t sk_n, int c, int half, char* stage, int wave, int lane) {
-  const int64_t key0 = (int64_t)c * AT_BS + half * AT_SUB;
-  const int64_t lim64 = n - 1 - key0;              // last valid row of this sub-tile (rows beyond are clamped)
-  const int lim = lim64 < 0 ? 0 : (lim64 > AT_SUB - 1 ? AT_SUB - 1 : (int)lim64);
-  const sp_bf16* kbase = kh + (lim64 < 0 ? (n - 1) : key0) * sk_n;
-  const sp_bf16* vbase = vth + (int64_t)c * AT_D * AT_BS + half * AT_SUB;
+// lane-constant byte offsets of the four K and four V^T chunks a lane fetches per sub-tile
+struct AtLoadOffsets {
+  uint32_t k[4], v[4];
+};
+
+__device__ static inline void at_load_offsets(AtLoadOffsets& lo, int64_t sk_n, int wave, int lane) {
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
-    const int seg = it * 4 + wave;                 // 1 KiB segment of the tile handled by this wave-instruction
-    {
+    const int seg = it * 4 + wave;  // 1 KiB segment of the tile handled by this wave-instruction
+    const int krow = seg * 4 + (lane >> 4);
+    lo.k[it] = (uint32_t)(krow * (int)sk_n + (((lane & 15) ^ (krow & 15)) * 8)) * 2u;
+    const int vrow = seg * 8 + (lane >> 3);
+    lo.v[it] = (uint32_t)(vrow * AT_BS + (((lane & 7) ^ ((vrow >> 1) & 7)) * 8)) * 2u;
+  }
+}
+
+__device__ static inline void at_issue_sub(const AtLoadOffsets& lo, const sp_bf16* __restrict__ kh,
+                                           const sp_bf16* __restrict__ vth, int64_t n, int64_t sk_n, int c, int half,
+                                           char* stage, int wave, int lane) {
+  const int64_t key0 = (int64_t)c * AT_BS + half * AT_SUB;
+  const char* vbase = reinterpret_cast<const char*>(vth + (int64_t)c * AT_D * AT_BS + half * AT_SUB);
+  if (key0 + AT_SUB <= n) {  // every key row exists: uniform base + lane-constant offset
+    const char* kbase = reinterpret_cast<const char*>(kh + key0 * sk_n);
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int seg = it * 4 + wave;
+      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(kbase + lo.k[it]), (at_lds_ptr)(stage + seg * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(vbase + lo.v[it]),
+                                       (at_lds_ptr)(stage + AT_KSTAGE_BYTES + seg * 1024), 16, 0, 0);
+    }
+  } else {  // ragged tail of the sequence: rows beyond the last key are clamped onto it
+    const int64_t lim64 = n - 1 - key0;
+    const int lim = lim64 < 0 ? 0 : (int)lim64;
+    const sp_bf16* kbase = kh + (lim64 < 0 ? (n - 1) : key0) * sk_n;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int seg = it * 4 + wave;
       const int row = seg * 4 + (lane >> 4);
       const int cl = (lane & 15) ^ (row & 15);
       const int rowc = row < lim ? row : lim;
       const sp_bf16* g = kbase + (uint32_t)(rowc * (int)sk_n + cl * 8);
       __builtin_amdgcn_global_load_lds((at_gbl_ptr)g, (at_lds_ptr)(stage + seg * 1024), 16, 0, 0);
-    }
-    {
-      const int row = seg * 8 + (lane >> 3);
-      const int cl = (lane & 7) ^ ((row >> 1) & 7);
-      const sp_bf16* g = vbase + (uint32_t)(row * AT_BS + cl * 8);
-      __builtin_amdgcn_global_load_lds((at_gbl_ptr)g, (at_lds_ptr)(stage + AT_KSTAGE_BYTES + seg * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(vbase + lo.v[it]),
+                                       (at_lds_ptr)(stage + AT_KSTAGE_BYTES + seg * 1024), 16, 0, 0);
     }
   }
 }
@@ -164,11 +206,17 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ vt,
     const uint64_t* __restrict__ mask, const int32_t* __restrict__ decision, sp_bf16* __restrict__ out,
     float2* __restrict__ rowstat, int64_t n, int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n,
-    int64_t sk_h, int nb, int nbw, float scale_log2, int* __restrict__ work_counter, int total_items) {
+    int64_t sk_h, int nb, int nbw, float scale_log2, int* __restrict__ sched) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // 2 stages x 32 KiB
-  __shared__ int s_item;
+  __shared__ int s_queue, s_ticket;
 
-  const int group = hq / hkv;
+  AtGeom gm;
+  gm.group = hq / hkv;
+  gm.nb = nb;
+  gm.n_chunks = (nb + AT_GANG - 1) / AT_GANG;
+  gm.n_gangs = hq * gm.n_chunks;
+  const int xcd = blockIdx.x & 7;
+  int first_try = 0;  // queues before this offset are known to be empty (used by thread 0 only)
   const int t = threadIdx.x;
   const int wave = t >> 6, lane = t & 63;
   const int lq = lane & 31, g = lane >> 5;
@@ -181,16 +229,32 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
   int voff[4];  // V^T rows lq (+32*dt via immediate), logical chunk 4*kt + 2*s + g, index kt*2+s
 #pragma unroll
   for (int j = 0; j < 4; ++j) voff[j] = AT_KSTAGE_BYTES + lq * 128 + (((2 * j + g) ^ ((lq >> 1) & 7)) << 4);
+  AtLoadOffsets lo;
+  at_load_offsets(lo, sk_n, wave, lane);
+
+  const bf16x8 ones = __builtin_bit_cast(bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
 
   for (;;) {
     __syncthreads();  // previous item's LDS reads are done
-    if (t == 0) s_item = atomicAdd(work_counter, 1);
+    if (t == 0) {
+      int found = -1, tk = 0;
+      for (int a = first_try; a < 8; ++a) {
+        const int xq = (xcd + a) & 7;
+        tk = atomicAdd(&sched[xq * 16], 1);
+        if (tk < at_queue_items(gm, xq)) {
+          found = xq;
+          first_try = a;
+          break;
+        }
+      }
+      s_queue = found;
+      s_ticket = tk;
+    }
     __syncthreads();
-    const int item = s_item;
-    if (item >= total_items) break;
+    if (s_queue < 0) break;
     int h, r;
-    at_item(item, group, nb, h, r);
-    const int kvh = h / group;
+    if (!at_item(gm, s_queue, s_ticket, h, r)) continue;
+    const int kvh = h / gm.group;
     const sp_bf16* kh = k + (int64_t)kvh * sk_h;
     const sp_bf16* vth = vt + (int64_t)kvh * nb * AT_D * AT_BS;
     const uint64_t* mrow = mask + ((int64_t)h * nb + r) * nbw;
@@ -200,7 +264,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
     int c_cur = it.next();
     int half = 0;
     int buf = 0;
-    if (c_cur >= 0) at_issue_sub(kh, vth, n, sk_n, c_cur, 0, lds, wave, lane);
+    if (c_cur >= 0) at_issue_sub(lo, kh, vth, n, sk_n, c_cur, 0, lds, wave, lane);
 
     // Q^T operand: this lane's query, 8 k-steps of 8 channels
     bf16x8 qb[8];
@@ -228,7 +292,8 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
         c_next = it.next();
         half_next = 0;
       }
-      if (c_next >= 0) at_issue_sub(kh, vth, n, sk_n, c_next, half_next, lds + (buf ^ 1) * AT_STAGE_BYTES, wave, lane);
+      if (c_next >= 0)
+        at_issue_sub(lo, kh, vth, n, sk_n, c_next, half_next, lds + (buf ^ 1) * AT_STAGE_BYTES, wave, lane);
 
       const char* st = lds + buf * AT_STAGE_BYTES;
       // ---- S^T = K . Q^T for 64 keys; LDS operands are fetched two k-steps ahead of their MFMAs ----
@@ -281,16 +346,11 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
       }
       // a row with nothing unmasked so far keeps m_run = -inf; exp2(-inf - (-inf)) must not be evaluated
       const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
-      float psum = 0.f;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], scale_log2, -m_use));
-          s[kt][i] = p;
-          psum += p;
-        }
-      l_run += psum;
+        for (int i = 0; i < 16; ++i)
+          s[kt][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], scale_log2, -m_use));
       // ---- O^T += V^T . P^T; V^T operands fetched one (kt, dt) step ahead ----
       {
         bf16x8 pb[2][2];
@@ -302,6 +362,10 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
         va[0][0] = at_lds128(st + voff[0]);
         va[0][1] = at_lds128(st + voff[1]);
         __builtin_amdgcn_s_setprio(1);
+        // row sums of the bf16 probabilities on the matrix core: ones(32x16) . P^T puts sum_k P[k][q] of the
+        // lane's query into every accumulator row (this replaces 32 dependent vector adds per sub-tile)
+        floatx16 rs = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[0][0], (floatx16){0}, 0, 0, 0);
+        rs = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[0][1], rs, 0, 0, 0);
 #pragma unroll
         for (int step = 0; step < 8; ++step) {  // step = kt*4 + dt
           const int kt = step >> 2, dt = step & 3;
@@ -312,14 +376,19 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
           }
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[step & 1][0], pb[kt][0], o[dt], 0, 0, 0);
           o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[step & 1][1], pb[kt][1], o[dt], 0, 0, 0);
+          if (step == 3) {
+            rs = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[1][0], rs, 0, 0, 0);
+            rs = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[1][1], rs, 0, 0, 0);
+          }
         }
         __builtin_amdgcn_s_setprio(0);
+        l_run += rs[0];  // the MFMA contracts over both lane halves: all 64 keys of the sub-tile for this query
       }
       buf ^= 1;
       c_cur = c_next;
       half = half_next;
     }
-    const float l_tot = l_run + __shfl_xor(l_run, 32, SP_WAVE);
+    const float l_tot = l_run;
 
     // pivot heads: keep the softmax statistics of every query row for the block-average pass
     if (rowstat != nullptr && decision != nullptr && decision[h] == SP_DEC_DENSE && g == 0) {
@@ -357,7 +426,9 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
   }
 }
 
-__global__ void sp_zero_i32_kernel(int* p) { *p = 0; }
+__global__ void sp_zero_i32_kernel(int* p, int count) {
+  for (int i = threadIdx.x; i < count; i += blockDim.x) p[i] = 0;
+}
 
 // ---- pivot heads: block-averaged attention map (shareprefill_attn.py:425-457) ---------------------------
 // avg[h][r][c] = mean over the valid queries of block r of the softmax mass that falls into key block c,
@@ -429,14 +500,14 @@ __global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_kernel(
 }
 
 // ---- host ---------------------------------------------------------------------------------------------
-// workspace layout: [ repacked V^T : hkv*nb*128*128 bf16 | work counter : 256 B | row statistics : hq*n float2 ]
+// workspace layout: [ repacked V^T : hkv*nb*128*128 bf16 | 8 queue tickets : 1 KiB | row statistics : hq*n float2 ]
 static size_t at_vt_bytes(int64_t n, int32_t hkv, int32_t d, int32_t bs) {
   return (size_t)hkv * (size_t)sp_ceil_div(n, bs) * bs * d * sizeof(sp_bf16);
 }
 
 extern "C" size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs) {
   if (n <= 0 || hq <= 0 || hkv <= 0 || d <= 0 || bs <= 0) return 0;
-  return at_vt_bytes(n, hkv, d, bs) + 256 + (size_t)hq * (size_t)n * sizeof(float2);
+  return at_vt_bytes(n, hkv, d, bs) + 1024 + (size_t)hq * (size_t)n * sizeof(float2);
 }
 
 extern "C" int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n,
@@ -489,10 +560,10 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   const float scale_log2 = softmax_scale * 1.4426950408889634f;
   char* ws = (char*)workspace;
   int* counter = reinterpret_cast<int*>(ws + at_vt_bytes(n, hkv, d, bs));
-  float2* rowstat = reinterpret_cast<float2*>(ws + at_vt_bytes(n, hkv, d, bs) + 256);
+  float2* rowstat = reinterpret_cast<float2*>(ws + at_vt_bytes(n, hkv, d, bs) + 1024);
   const bool want_avg = decision != nullptr && avg_attn != nullptr;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_zero_i32_kernel, dim3(1), dim3(1), 0, s, counter);
+  hipLaunchKernelGGL(sp_zero_i32_kernel, dim3(1), dim3(128), 0, s, counter, 8 * 16);
   SP_LAUNCH_CHECK();
   const size_t lds_bytes = 2 * AT_STAGE_BYTES;
   static int n_cu = 0;
@@ -506,11 +577,11 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
     n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
   const int64_t total = nb * hq;
-  const int grid = (int)(total < 2ll * n_cu ? total : 2ll * n_cu);
+  const int grid = (int)(total < 2ll * n_cu ? ((total + 7) / 8) * 8 : 2ll * n_cu);
   hipLaunchKernelGGL(sp_attn_fwd_kernel, dim3(grid), dim3(AT_THREADS), lds_bytes, s, (const sp_bf16*)q,
                      (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out,
                      want_avg ? rowstat : (float2*)nullptr, n, hq, hkv, q_stride_n, q_stride_h, k_stride_n,
-                     k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, counter, (int)total);
+                     k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, counter);
   SP_LAUNCH_CHECK();
   if (want_avg) {
     hipLaunchKernelGGL(sp_attn_avg_kernel, dim3((unsigned)nb, hq), dim3(AT_THREADS), 0, s, (const sp_bf16*)q,

@@ -45,7 +45,7 @@ def test_library_identity_and_error_string():
     with pytest.raises(ValueError):
         _lib.check(st, "sp_pool_avg_bf16")
     assert lib.sp_lastq_scores_workspace_bytes(131072, 32, 128) == (32 * 128 * 128 + 32 * 128) * 8
-    assert lib.sp_attn_workspace_bytes(131072, 32, 8, 128, 128) == 8 * 131072 * 128 * 2 + 256 + 32 * 131072 * 8
+    assert lib.sp_attn_workspace_bytes(131072, 32, 8, 128, 128) == 8 * 131072 * 128 * 2 + 1024 + 32 * 131072 * 8
 
 
 def test_cluster_state_struct_matches_header_layout():
