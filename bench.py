@@ -34,7 +34,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C5"])
+    ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--seq-len", type=int, default=131072, help="C4 only: prompt length")
     ap.add_argument("--pattern-threshold", type=float, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the stage breakdown / dense baseline / sweep")
@@ -106,12 +107,79 @@ def cpu_baseline(w, q, k, v, mask_bool, decision, kept_blocks, pt):
                       f"scaled to {kept_blocks} kept blocks; extrapolated"}
 
 
+# HBM-side bytes of one steady-state sp_attn_fwd_kernel launch of the default workload (C3, pattern_threshold
+# 0.95), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the V-repack kernel's known 256 MiB
+# (profiles/attention_layer_C3_hbm_traffic.txt): 329 GiB fetched + 1 GiB written.
+MEASURED_ATTN_TRAFFIC_BYTES = {("C3", 0.95): int((329.0 + 1.0) * 2 ** 30)}
+
+
+def run_c4(args):
+    """TTFT of the full Llama-3.1-8B architecture (random-init bf16, 32 layers, hidden 4096, Hq32 Hkv8, RoPE theta
+    5e5, vocab 128256) on uniform-random token ids, SharePrefill patched into every layer with the shipped
+    Llama-3.1-8B-Instruct table; one prefill forward with last-token logits only."""
+    import torch
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from shareprefill_amd import SharePrefill
+
+    dev = torch.device("cuda:0")
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, vocab_size=128256, max_position_embeddings=131072,
+                      rope_parameters={"rope_type": "default", "rope_theta": 500000.0}, rms_norm_eps=1e-5,
+                      tie_word_embeddings=False)
+    torch.manual_seed(1238)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    with torch.device(dev):
+        model = LlamaForCausalLM(cfg)
+    torch.set_default_dtype(old)
+    model.eval()
+    model = SharePrefill(model_name="meta-llama/Llama-3.1-8B-Instruct", pattern_threshold=0.95, similarity_threshold=0.5,
+                         fallback_threshold=0.95, block_size=128, min_budget=1024)(model)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1238)
+    ids = torch.randint(0, cfg.vocab_size, (1, args.seq_len), generator=gen, device=dev)
+
+    def fwd():
+        with torch.no_grad():
+            return model(ids, use_cache=False, logits_to_keep=1).logits
+
+    for _ in range(max(args.warmup, 1)):
+        fwd()
+    torch.cuda.synchronize()
+    steps = max(1, min(args.steps, 3))
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = fwd()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / steps
+    sharing = model.attention_sharing
+    dens = torch.stack([p.density() for p in sharing.plans]).mean().item()
+    line = {"metric": "ttft_s_llama31_8b_arch_prefill", "value": round(sec, 3), "unit": "s", "n_gpus": 1,
+            "steps": steps, "warmup": max(args.warmup, 1), "ms_per_step": round(sec * 1e3, 1),
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"C4: Llama-3.1-8B architecture, random-init bf16, {args.seq_len} uniform-random token "
+                                   "ids, SharePrefill in all 32 layers (shipped Llama-3.1-8B-Instruct table, "
+                                   "pattern 0.95, similarity 0.5, fallback 0.95, min_budget 1024), logits_to_keep=1"},
+            "tokens_per_s": round(args.seq_len / sec, 1), "mean_block_density": round(dens, 4),
+            "decisions": sharing.decision_histogram(), "finite_logits": bool(torch.isfinite(out).all())}
+    print(json.dumps(line))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only (the SharePrefill layer has no multi-GPU path); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "C4":
+        import torch
+
+        if not torch.cuda.is_available():
+            print("bench.py: no GPU visible", file=sys.stderr)
+            sys.exit(2)
+        run_c4(args)
+        return
 
     import torch
 
@@ -205,7 +273,8 @@ def main():
                    "density": round(kept0 / tri, 4)},
         "roofline": {"bound": "mfma", "kernel": "sp_attn_fwd_kernel", "achieved": round(attn_tflops, 1),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
-                     "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms), "traffic": None},
+                     "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms),
+                     "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get((args.workload, pt))},
     }
 
     if not args.no_extras:

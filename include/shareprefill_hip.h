@@ -141,12 +141,17 @@ int sp_build_mask(const sp_cluster_state* state /* host */, const int32_t* head_
  * qbar: bf16 [nb][hq][d] (sp_pool_avg_bf16 of q), kbar: bf16 [nb][hkv][d]. */
 int sp_queryaware_select_bf16(const void* qbar, const void* kbar, const int32_t* decision, int32_t hq,
                               int32_t hkv, int32_t d, int32_t nb, uint32_t flags, float pattern_threshold,
-                              float* probs, uint64_t* mask, sp_stream_t stream);
+                              float* probs, uint64_t* mask, void* workspace, size_t workspace_bytes,
+                              sp_stream_t stream);
 
 /* the selection alone, on caller-supplied probabilities: mask[v] |= kept entries of x[v] ([nb][nb] each),
- * restricted to the lower triangle; vectors with enable[v] == 0 are skipped (enable may be NULL). */
+ * restricted to the lower triangle (entries above the diagonal are ignored; they are exactly zero in the
+ * reference's maps); vectors with enable[v] == 0 are skipped (enable may be NULL).
+ * workspace: sp_cover_select_workspace_bytes(n_vec) bytes of device scratch, 8-byte aligned (also needed by
+ * sp_queryaware_select_bf16, with n_vec = hq). */
+size_t sp_cover_select_workspace_bytes(int32_t n_vec);
 int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec, int32_t nb, float score,
-                           uint64_t* mask, sp_stream_t stream);
+                           uint64_t* mask, void* workspace, size_t workspace_bytes, sp_stream_t stream);
 
 /* ---- GQA causal block-sparse flash attention ------------------------------------------------
  * Replaces triton_block_wise_prefill_attention / block_wise_prefill_attention_kernel /

@@ -47,8 +47,9 @@ SIGNATURES = {
                                        _P]),
     "sp_share_decide": (_I32, [_ST, _P, _I32, _I32, _P, _P, _P, _P, _P, _I32, _F, _D, _P, _P, _P, _P, _P, _P]),
     "sp_build_mask": (_I32, [_ST, _P, _P, _P, _P, _P, _P, _I32, _I32, _P, _P]),
-    "sp_queryaware_select_bf16": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _U32, _F, _P, _P, _P]),
-    "sp_cover_select_global": (_I32, [_P, _P, _I32, _I32, _F, _P, _P]),
+    "sp_queryaware_select_bf16": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _U32, _F, _P, _P, _P, _SZ, _P]),
+    "sp_cover_select_workspace_bytes": (_SZ, [_I32]),
+    "sp_cover_select_global": (_I32, [_P, _P, _I32, _I32, _F, _P, _P, _SZ, _P]),
     "sp_attn_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _I32]),
     "sp_attn_repack_v_bf16": (_I32, [_P, _I64, _I32, _I32, _I64, _I64, _I32, _P, _SZ, _P]),
     "sp_block_sparse_attn_fwd_bf16": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I64, _I64,

@@ -195,73 +195,268 @@ extern "C" int sp_cover_budgets(const float* vert_tok, const float* slash_tok, i
 }
 
 // ---- score_cover_idx (attn/utils.py:53-57) on [nb][nb] maps, written into bit masks -----------------
-__global__ __launch_bounds__(SEL_THREADS) void sp_cover_select_global_kernel(
-    const float* __restrict__ x, const int32_t* __restrict__ enable, int enable_match, int nb, int nbw,
-    long long t_le, uint64_t* __restrict__ mask) {
+// Multi-workgroup radix mass descent over the LOWER TRIANGLE of each map (entries above the diagonal are
+// exactly zero in the reference's maps and cannot be selected; they are ignored here).  Per level: many
+// workgroups per vector build LDS histograms of their rows and merge them into a global (count, mass)
+// histogram with integer atomics; one workgroup per vector then picks the bin in which the running mass
+// crosses the budget.  A row-parallel kernel writes the mask bits.  Only when the boundary falls inside a
+// group of equal values that is taken partially (lowest indices first) a sequential kernel ranks them.
+#define GSEL_SPLIT 64     // workgroups per vector in the histogram / emit kernels
+#define GSEL_THREADS 256
+
+struct GselState {
+  unsigned long long rem;   // budget left after the bins / groups above the current prefix
+  uint32_t prefix;          // key bits fixed so far
+  uint32_t above;           // elements with key above the cut
+  uint32_t n_equal, n_take; // boundary group
+  int32_t all;              // 1: the whole vector is kept
+  int32_t enabled;
+  uint32_t pad[8];
+};
+
+__device__ static inline bool gsel_enabled(const int32_t* enable, int enable_match, int v) {
+  if (!enable) return true;
+  const int e = enable[v];
+  return enable_match < 0 ? (e != 0) : (e == enable_match);
+}
+
+__global__ void sp_gsel_init_kernel(GselState* st, uint32_t* cnt, unsigned long long* sum, const int32_t* enable,
+                                    int enable_match, int n_vec, long long t_le, uint64_t* mask, int nb, int nbw) {
+  const int v = blockIdx.x;
+  for (int i = threadIdx.x; i < SEL_BINS; i += blockDim.x) {
+    cnt[(int64_t)v * SEL_BINS + i] = 0;
+    sum[(int64_t)v * SEL_BINS + i] = 0;
+  }
+  if (threadIdx.x == 0) {
+    GselState s;
+    s.rem = t_le < 0 ? 0ull : (unsigned long long)t_le;
+    s.prefix = 0;
+    s.above = 0;
+    s.n_equal = 0;
+    s.n_take = 0;
+    s.all = 0;
+    s.enabled = (gsel_enabled(enable, enable_match, v) && t_le >= 0) ? 1 : 0;
+    for (int i = 0; i < 8; ++i) s.pad[i] = 0;
+    st[v] = s;
+    if (gsel_enabled(enable, enable_match, v))  // block (0,0): the padding id of the reference
+      atomicOr(reinterpret_cast<uint32_t*>(mask + (int64_t)v * nb * nbw), 1u);
+  }
+}
+
+template <int LEVEL>
+__global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_hist_kernel(const float* __restrict__ x, int nb,
+                                                                    const GselState* __restrict__ st,
+                                                                    uint32_t* __restrict__ gcnt,
+                                                                    unsigned long long* __restrict__ gsum) {
+  __shared__ unsigned long long lsum[SEL_BINS];
+  __shared__ uint32_t lcnt[SEL_BINS];
+  const int v = blockIdx.y;
+  const GselState s = st[v];
+  if (!s.enabled || s.all) return;
+  constexpr int shift = LEVEL == 0 ? 21 : (LEVEL == 1 ? 10 : 0);
+  constexpr int width = LEVEL == 2 ? 10 : 11;
+  constexpr int pshift = LEVEL == 0 ? 32 : (LEVEL == 1 ? 21 : 10);
+  for (int i = threadIdx.x; i < SEL_BINS; i += GSEL_THREADS) {
+    lsum[i] = 0;
+    lcnt[i] = 0;
+  }
+  __syncthreads();
+  const float* xv = x + (int64_t)v * nb * nb;
+  for (int r = blockIdx.x; r < nb; r += GSEL_SPLIT) {
+    const float* row = xv + (int64_t)r * nb;
+    for (int c = threadIdx.x; c <= r; c += GSEL_THREADS) {
+      const float val = row[c];
+      const uint32_t key = sp_sort_key(val);
+      if (pshift < 32 && (key >> (pshift & 31)) != s.prefix) continue;
+      const uint32_t b = (key >> shift) & ((1u << width) - 1u);
+      atomicAdd(&lcnt[b], 1u);
+      const unsigned long long fx = sp_to_fixed(val);
+      if (fx) atomicAdd(&lsum[b], fx);
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < (1 << width); i += GSEL_THREADS) {
+    if (lcnt[i]) atomicAdd(&gcnt[(int64_t)v * SEL_BINS + i], lcnt[i]);
+    if (lsum[i]) atomicAdd(&gsum[(int64_t)v * SEL_BINS + i], lsum[i]);
+  }
+}
+
+template <int LEVEL>
+__global__ __launch_bounds__(SEL_THREADS) void sp_gsel_pick_kernel(GselState* __restrict__ st,
+                                                                   uint32_t* __restrict__ gcnt,
+                                                                   unsigned long long* __restrict__ gsum) {
   __shared__ SelShared sh;
+  const int v = blockIdx.x, t = threadIdx.x;
+  GselState s = st[v];
+  if (!s.enabled || s.all) return;
+  constexpr int width = LEVEL == 2 ? 10 : 11;
+  const int nbins = 1 << width;
+  uint32_t* gc = gcnt + (int64_t)v * SEL_BINS;
+  unsigned long long* gs = gsum + (int64_t)v * SEL_BINS;
+  sh.sum[t] = gs[t];
+  sh.sum[t + SEL_THREADS] = gs[t + SEL_THREADS];
+  sh.cnt[t] = gc[t];
+  sh.cnt[t + SEL_THREADS] = gc[t + SEL_THREADS];
+  gs[t] = 0;  // ready for the next level
+  gs[t + SEL_THREADS] = 0;
+  gc[t] = 0;
+  gc[t + SEL_THREADS] = 0;
+  if (t == 0) {
+    sh.bin = -1;
+    sh.cnt_above = 0;
+  }
+  __syncthreads();
+  const unsigned long long own0 = sh.sum[t], own1 = sh.sum[t + SEL_THREADS];
+  __syncthreads();
+  sel_suffix_scan(sh);
+#pragma unroll
+  for (int rep = 0; rep < 2; ++rep) {
+    const int b = t + rep * SEL_THREADS;
+    if (b < nbins) {
+      const unsigned long long incl = sh.sum[b];
+      const unsigned long long excl = (b + 1 < SEL_BINS) ? sh.sum[b + 1] : 0ull;
+      if (incl > s.rem && excl <= s.rem) {
+        sh.bin = b;
+        sh.sum_above = excl;
+        sh.bin_sum = rep ? own1 : own0;
+        sh.bin_cnt = sh.cnt[b];
+      }
+    }
+  }
+  __syncthreads();
+  const int bin = sh.bin;
+  if (bin < 0) {  // the running mass never exceeds the budget (top level only): keep everything
+    if (t == 0) {
+      s.all = 1;
+      st[v] = s;
+    }
+    return;
+  }
+  uint32_t c = 0;
+#pragma unroll
+  for (int rep = 0; rep < 2; ++rep) {
+    const int b = t + rep * SEL_THREADS;
+    if (b < nbins && b > bin) c += sh.cnt[b];
+  }
+  if (c) atomicAdd(&sh.cnt_above, c);
+  __syncthreads();
+  if (t == 0) {
+    s.prefix = (s.prefix << width) | (uint32_t)bin;
+    s.above += sh.cnt_above;
+    s.rem -= sh.sum_above;
+    if (LEVEL == 2) {
+      s.n_equal = sh.bin_cnt;
+      const unsigned long long each = sh.bin_sum / (sh.bin_cnt ? sh.bin_cnt : 1u);
+      unsigned long long take = each ? s.rem / each : (unsigned long long)s.n_equal;
+      if (take > s.n_equal) take = s.n_equal;
+      s.n_take = (uint32_t)take;
+    }
+    st[v] = s;
+  }
+}
+
+__global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_emit_kernel(const float* __restrict__ x, int nb, int nbw,
+                                                                    const GselState* __restrict__ st,
+                                                                    uint64_t* __restrict__ mask) {
+  const int v = blockIdx.y;
+  const GselState s = st[v];
+  if (!s.enabled) return;
+  const bool take_all_equal = s.all || s.n_take >= s.n_equal;
+  const float* xv = x + (int64_t)v * nb * nb;
+  uint64_t* mv = mask + (int64_t)v * nb * nbw;
+  for (int r = blockIdx.x; r < nb; r += GSEL_SPLIT) {
+    const float* row = xv + (int64_t)r * nb;
+    for (int c0 = 0; c0 <= r; c0 += GSEL_THREADS) {  // uniform trip count per workgroup: every lane votes
+      const int c = c0 + threadIdx.x;
+      bool sel = false;
+      if (c <= r) {
+        const uint32_t key = sp_sort_key(row[c]);
+        sel = s.all || key > s.prefix || (key == s.prefix && take_all_equal);
+      }
+      const unsigned long long bal = __ballot(sel);
+      if ((threadIdx.x & 63) == 0 && bal)
+        atomicOr(reinterpret_cast<unsigned long long*>(mv) + (int64_t)r * nbw + (c >> 6), bal);
+    }
+  }
+}
+
+// boundary group taken partially: the n_take lowest indices (row-major) of the equal-valued entries win
+__global__ __launch_bounds__(SEL_THREADS) void sp_gsel_emit_ranked_kernel(const float* __restrict__ x, int nb, int nbw,
+                                                                          const GselState* __restrict__ st,
+                                                                          uint64_t* __restrict__ mask) {
   __shared__ uint32_t wave_cnt[SEL_THREADS / SP_WAVE];
   __shared__ uint32_t running;
   const int v = blockIdx.x;
-  if (enable) {
-    const int e = enable[v];
-    if (enable_match < 0 ? (e == 0) : (e != enable_match)) return;
-  }
+  const GselState s = st[v];
+  if (!s.enabled || s.all || s.n_take == 0 || s.n_take >= s.n_equal) return;
   const int64_t len = (int64_t)nb * nb;
   const float* xv = x + (int64_t)v * len;
   uint32_t* mv = reinterpret_cast<uint32_t*>(mask + (int64_t)v * nb * nbw);
-  if (threadIdx.x == 0) atomicOr(&mv[0], 1u);  // block (0,0): the padding id of the reference
-  if (t_le < 0) return;
-  MassCut cut = sel_mass_cut(xv, len, (unsigned long long)t_le, sh);
-  const bool ranked = !cut.all && cut.n_take > 0 && cut.n_take < cut.n_equal;
   if (threadIdx.x == 0) running = 0;
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int64_t base = 0; base < len; base += SEL_THREADS) {
     const int64_t i = base + threadIdx.x;
-    bool sel = false;
     bool eq = false;
     int r = 0, c = 0;
     if (i < len) {
       r = (int)(i / nb);
       c = (int)(i - (int64_t)r * nb);
-      const uint32_t key = sp_sort_key(xv[i]);
-      if (cut.all || key > cut.key)
-        sel = true;
-      else if (key == cut.key) {
-        if (cut.n_take >= cut.n_equal)
-          sel = true;
-        else
-          eq = cut.n_take > 0;
-      }
+      eq = c <= r && sp_sort_key(xv[i]) == s.prefix;
     }
-    if (ranked) {  // ties at the boundary: the n_take lowest indices win
-      const unsigned long long bal = __ballot(eq);
-      const uint32_t before = __popcll(bal & ((1ull << lane) - 1ull));
-      if (lane == 0) wave_cnt[wave] = __popcll(bal);
-      __syncthreads();
-      uint32_t off = running;
-      for (int w = 0; w < wave; ++w) off += wave_cnt[w];
-      if (eq && off + before < cut.n_take) sel = true;
-      __syncthreads();
-      if (threadIdx.x == 0) {
-        uint32_t tot = 0;
-        for (int w = 0; w < SEL_THREADS / SP_WAVE; ++w) tot += wave_cnt[w];
-        running += tot;
-      }
-      __syncthreads();
+    const unsigned long long bal = __ballot(eq);
+    const uint32_t before = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_cnt[wave] = __popcll(bal);
+    __syncthreads();
+    uint32_t off = running;
+    for (int w = 0; w < wave; ++w) off += wave_cnt[w];
+    if (eq && off + before < s.n_take)
+      atomicOr(&mv[((int64_t)r * nbw + (c >> 6)) * 2 + ((c >> 5) & 1)], 1u << (c & 31));
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint32_t tot = 0;
+      for (int w = 0; w < SEL_THREADS / SP_WAVE; ++w) tot += wave_cnt[w];
+      running += tot;
     }
-    if (sel && c <= r) atomicOr(&mv[((int64_t)r * nbw + (c >> 6)) * 2 + ((c >> 5) & 1)], 1u << (c & 31));
+    __syncthreads();
+    if (running >= s.n_take) break;
   }
 }
 
-extern "C" int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec, int32_t nb, float score,
-                                      uint64_t* mask, sp_stream_t stream) {
-  SP_REQUIRE(x && mask && n_vec > 0 && nb > 0, SP_ERR_INVALID_ARGUMENT, "sp_cover_select_global: bad arguments");
+extern "C" size_t sp_cover_select_workspace_bytes(int32_t n_vec) {
+  if (n_vec <= 0) return 0;
+  return (size_t)n_vec * (sizeof(GselState) + SEL_BINS * (sizeof(uint32_t) + sizeof(unsigned long long)));
+}
+
+static int gsel_run(const float* x, const int32_t* enable, int enable_match, int n_vec, int nb, float score,
+                    uint64_t* mask, void* workspace, size_t workspace_bytes, hipStream_t s, const char* who) {
+  SP_REQUIRE(workspace && workspace_bytes >= sp_cover_select_workspace_bytes(n_vec) && ((uintptr_t)workspace % 8) == 0,
+             SP_ERR_WORKSPACE, "%s: workspace missing, misaligned or too small", who);
   const int nbw = (nb + 63) / 64;
-  hipLaunchKernelGGL(sp_cover_select_global_kernel, dim3(n_vec), dim3(SEL_THREADS), 0, (hipStream_t)stream, x, enable,
-                     -1, nb, nbw, (long long)sp_thr_le(score), mask);
+  GselState* st = reinterpret_cast<GselState*>(workspace);
+  unsigned long long* gsum = reinterpret_cast<unsigned long long*>(st + n_vec);
+  uint32_t* gcnt = reinterpret_cast<uint32_t*>(gsum + (size_t)n_vec * SEL_BINS);
+  hipLaunchKernelGGL(sp_gsel_init_kernel, dim3(n_vec), dim3(256), 0, s, st, gcnt, gsum, enable, enable_match, n_vec,
+                     (long long)sp_thr_le(score), mask, nb, nbw);
+  SP_LAUNCH_CHECK();
+  const dim3 hgrid(GSEL_SPLIT, n_vec);
+  hipLaunchKernelGGL(sp_gsel_hist_kernel<0>, hgrid, dim3(GSEL_THREADS), 0, s, x, nb, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_pick_kernel<0>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_hist_kernel<1>, hgrid, dim3(GSEL_THREADS), 0, s, x, nb, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_pick_kernel<1>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_hist_kernel<2>, hgrid, dim3(GSEL_THREADS), 0, s, x, nb, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_pick_kernel<2>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_emit_kernel, hgrid, dim3(GSEL_THREADS), 0, s, x, nb, nbw, st, mask);
+  hipLaunchKernelGGL(sp_gsel_emit_ranked_kernel, dim3(n_vec), dim3(SEL_THREADS), 0, s, x, nb, nbw, st, mask);
   SP_LAUNCH_CHECK();
   return SP_OK;
+}
+
+extern "C" int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec, int32_t nb, float score,
+                                      uint64_t* mask, void* workspace, size_t workspace_bytes, sp_stream_t stream) {
+  SP_REQUIRE(x && mask && n_vec > 0 && nb > 0, SP_ERR_INVALID_ARGUMENT, "sp_cover_select_global: bad arguments");
+  return gsel_run(x, enable, -1, n_vec, nb, score, mask, workspace, workspace_bytes, (hipStream_t)stream,
+                  "sp_cover_select_global");
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -719,7 +914,8 @@ __global__ __launch_bounds__(BP_THREADS) void sp_block_probs_kernel(
 
 extern "C" int sp_queryaware_select_bf16(const void* qbar, const void* kbar, const int32_t* decision, int32_t hq,
                                          int32_t hkv, int32_t d, int32_t nb, uint32_t flags, float pattern_threshold,
-                                         float* probs, uint64_t* mask, sp_stream_t stream) {
+                                         float* probs, uint64_t* mask, void* workspace, size_t workspace_bytes,
+                                         sp_stream_t stream) {
   SP_REQUIRE(qbar && kbar && decision && probs && mask, SP_ERR_INVALID_ARGUMENT,
              "sp_queryaware_select_bf16: null pointer");
   SP_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0 && d % 8 == 0 && nb > 0, SP_ERR_INVALID_ARGUMENT,
@@ -732,10 +928,8 @@ extern "C" int sp_queryaware_select_bf16(const void* qbar, const void* kbar, con
   SP_LAUNCH_CHECK();
   // score = pattern_threshold * nb evaluated in double, then taken to fp32 as a tensor comparison would
   const float score = (float)((double)pattern_threshold * (double)nb);
-  hipLaunchKernelGGL(sp_cover_select_global_kernel, dim3(hq), dim3(SEL_THREADS), 0, (hipStream_t)stream, probs,
-                     decision, SP_DEC_QA, nb, (nb + 63) / 64, (long long)sp_thr_le(score), mask);
-  SP_LAUNCH_CHECK();
-  return SP_OK;
+  return gsel_run(probs, decision, SP_DEC_QA, hq, nb, score, mask, workspace, workspace_bytes, (hipStream_t)stream,
+                  "sp_queryaware_select_bf16");
 }
 
 // ------------------------------------------------------------------------------------------------

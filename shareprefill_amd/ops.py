@@ -193,8 +193,9 @@ def queryaware_select(qbar, kbar, decision, mask, pattern_threshold, flags=_lib.
     hkv = kbar.shape[1]
     if probs is None:
         probs = torch.empty(hq, nb, nb, dtype=torch.float32, device=qbar.device)
+    ws = _workspace("cover_select", lib.sp_cover_select_workspace_bytes(hq), qbar.device)
     st = lib.sp_queryaware_select_bf16(_ptr(qbar), _ptr(kbar), _ptr(decision), hq, hkv, d, nb, flags,
-                                       pattern_threshold, _ptr(probs), _ptr(mask), _stream())
+                                       pattern_threshold, _ptr(probs), _ptr(mask), _ptr(ws), ws.numel(), _stream())
     _lib.check(st, "sp_queryaware_select_bf16")
     return probs
 
@@ -204,7 +205,8 @@ def cover_select_global(x: torch.Tensor, score: float, mask: torch.Tensor, enabl
     lib = _lib.load()
     assert x.dtype == torch.float32 and x.is_contiguous() and mask.is_contiguous()
     v, nb, _ = x.shape
-    st = lib.sp_cover_select_global(_ptr(x), _ptr(enable), v, nb, score, _ptr(mask), _stream())
+    ws = _workspace("cover_select", lib.sp_cover_select_workspace_bytes(v), x.device)
+    st = lib.sp_cover_select_global(_ptr(x), _ptr(enable), v, nb, score, _ptr(mask), _ptr(ws), ws.numel(), _stream())
     _lib.check(st, "sp_cover_select_global")
     return mask
 
