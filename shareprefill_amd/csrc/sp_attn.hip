@@ -11,8 +11,12 @@
 //   O^T += V^T . P^T: the P^T operand is the S^T accumulator converted to bf16 in place (no LDS round
 //                     trip); the V^T operand comes from a key-major repack of V made once per call, whose
 //                     key order inside every group of 16 keys matches the accumulator's row order.
-// K and V^T tiles are staged through LDS with a 272-byte row pitch (conflict-free 128-bit reads).
+// K and V^T sub-tiles (64 keys) are staged through LDS by direct global->LDS loads, XOR-swizzled; every wave runs a
+// software pipeline over 32-key half-tiles in which the softmax of one half-tile is issued between the MFMAs of
+// its neighbours (see "the software pipeline of one wave" below).
 #include "sp_common.h"
+
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx8 __attribute__((ext_vector_type(8)));
@@ -99,74 +103,70 @@ __device__ static inline bool at_item(const AtGeom& gm, int xq, int ticket, int&
 }
 
 // ---- LDS staging -------------------------------------------------------------------------------------------
-// A block is processed as two sub-tiles of 64 keys.  One stage holds a K sub-tile [64 keys][16 chunks] and a
-// V^T sub-tile [128 channels][8 chunks] (chunk = 16 bytes = 8 bf16), 32 KiB; two stages are double-buffered.
-// Tiles are filled by direct global->LDS 128-bit loads: lane i of a wave writes LDS chunk (base + i), fetching
-// whichever global chunk belongs there.  Instead of row padding the chunk index is XOR-swizzled with the row,
+// A block is processed as two sub-tiles of 64 keys.  LDS holds two K sub-tile buffers [64 keys][16 chunks] and
+// two V^T sub-tile buffers [128 channels][8 chunks] (chunk = 16 bytes = 8 bf16), 16 KiB each.  Tiles are filled
+// by direct global->LDS 128-bit loads: lane i of a wave writes LDS chunk (base + i), fetching whichever global
+// chunk belongs there.  Instead of row padding the chunk index is XOR-swizzled with the row,
 //   K  : chunk c of row r sits at r*16 + (c ^ (r & 15))
 //   V^T: chunk c of row r sits at r*8  + (c ^ ((r >> 1) & 7))
 // so the 16 lanes that read the same logical chunk of 16 consecutive rows hit 16 different bank groups.
 #define AT_SUB 64
-#define AT_KSTAGE_BYTES (AT_SUB * AT_D * 2)      // 16 KiB
-#define AT_VSTAGE_BYTES (AT_D * AT_SUB * 2)      // 16 KiB
-#define AT_STAGE_BYTES (AT_KSTAGE_BYTES + AT_VSTAGE_BYTES)
+#define AT_KBUF_BYTES (AT_SUB * AT_D * 2)  // 16 KiB
+#define AT_VBUF_BYTES (AT_D * AT_SUB * 2)  // 16 KiB
+#define AT_LDS_BYTES (2 * AT_KBUF_BYTES + 2 * AT_VBUF_BYTES)
 
 typedef __attribute__((address_space(3))) void* at_lds_ptr;
 typedef const __attribute__((address_space(1))) void* at_gbl_ptr;
 
-// lane-constant byte offsets of the four K and four V^T chunks a lane fetches per sub-tile
+// Lane-constant byte offsets of the first K and V^T chunk a lane fetches per sub-tile.  A wave-instruction fills
+// one 1 KiB segment (seg = it*4 + wave): 4 K rows or 8 V^T rows.  Row and swizzle of a lane do not depend on `it`
+// beyond a uniform step (16 K rows / 32 V^T rows), which goes into the scalar base address.
 struct AtLoadOffsets {
-  uint32_t k[4], v[4];
+  uint32_t k, v;
 };
 
 __device__ static inline void at_load_offsets(AtLoadOffsets& lo, int64_t sk_n, int wave, int lane) {
-#pragma unroll
-  for (int it = 0; it < 4; ++it) {
-    const int seg = it * 4 + wave;  // 1 KiB segment of the tile handled by this wave-instruction
-    const int krow = seg * 4 + (lane >> 4);
-    lo.k[it] = (uint32_t)(krow * (int)sk_n + (((lane & 15) ^ (krow & 15)) * 8)) * 2u;
-    const int vrow = seg * 8 + (lane >> 3);
-    lo.v[it] = (uint32_t)(vrow * AT_BS + (((lane & 7) ^ ((vrow >> 1) & 7)) * 8)) * 2u;
-  }
+  const int krow = wave * 4 + (lane >> 4);
+  lo.k = (uint32_t)(krow * (int)sk_n + (((lane & 15) ^ (krow & 15)) * 8)) * 2u;
+  const int vrow = wave * 8 + (lane >> 3);
+  lo.v = (uint32_t)(vrow * AT_BS + (((lane & 7) ^ ((vrow >> 1) & 7)) * 8)) * 2u;
 }
 
-__device__ static inline void at_issue_sub(const AtLoadOffsets& lo, const sp_bf16* __restrict__ kh,
-                                           const sp_bf16* __restrict__ vth, int64_t n, int64_t sk_n, int c, int half,
-                                           char* stage, int wave, int lane) {
+__device__ static inline void at_issue_k(const AtLoadOffsets& lo, const sp_bf16* __restrict__ kh, int64_t n,
+                                         int64_t sk_n, int c, int half, char* kbuf, int wave, int t) {
   const int64_t key0 = (int64_t)c * AT_BS + half * AT_SUB;
-  const char* vbase = reinterpret_cast<const char*>(vth + (int64_t)c * AT_D * AT_BS + half * AT_SUB);
   if (key0 + AT_SUB <= n) {  // every key row exists: uniform base + lane-constant offset
     const char* kbase = reinterpret_cast<const char*>(kh + key0 * sk_n);
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int seg = it * 4 + wave;
-      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(kbase + lo.k[it]), (at_lds_ptr)(stage + seg * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(vbase + lo.v[it]),
-                                       (at_lds_ptr)(stage + AT_KSTAGE_BYTES + seg * 1024), 16, 0, 0);
-    }
+    for (int it = 0; it < 4; ++it)
+      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(kbase + (int64_t)it * 32 * sk_n + lo.k),
+                                       (at_lds_ptr)(kbuf + (it * 4 + wave) * 1024), 16, 0, 0);
   } else {  // ragged tail of the sequence: rows beyond the last key are clamped onto it
     const int64_t lim64 = n - 1 - key0;
     const int lim = lim64 < 0 ? 0 : (int)lim64;
     const sp_bf16* kbase = kh + (lim64 < 0 ? (n - 1) : key0) * sk_n;
+    int ln = t & 63;
+    asm volatile("" : "+v"(ln));  // keeps this rare path's lane arithmetic from being hoisted out of the key loop
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
       const int seg = it * 4 + wave;
-      const int row = seg * 4 + (lane >> 4);
-      const int cl = (lane & 15) ^ (row & 15);
+      const int row = seg * 4 + (ln >> 4);
+      const int cl = (ln & 15) ^ (row & 15);
       const int rowc = row < lim ? row : lim;
       const sp_bf16* g = kbase + (uint32_t)(rowc * (int)sk_n + cl * 8);
-      __builtin_amdgcn_global_load_lds((at_gbl_ptr)g, (at_lds_ptr)(stage + seg * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(vbase + lo.v[it]),
-                                       (at_lds_ptr)(stage + AT_KSTAGE_BYTES + seg * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((at_gbl_ptr)g, (at_lds_ptr)(kbuf + seg * 1024), 16, 0, 0);
     }
   }
 }
 
-__device__ static inline bf16x8 at_pack8(const floatx16& a, int base) {
-  floatx8 f;
+// the repacked V^T is zero-filled beyond the last key, so no tail case
+__device__ static inline void at_issue_v(const AtLoadOffsets& lo, const sp_bf16* __restrict__ vth, int c, int half,
+                                         char* vbuf, int wave) {
+  const char* vbase = reinterpret_cast<const char*>(vth + (int64_t)c * AT_D * AT_BS + half * AT_SUB);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) f[j] = a[base + j];
-  return __builtin_convertvector(f, bf16x8);
+  for (int it = 0; it < 4; ++it)
+    __builtin_amdgcn_global_load_lds((at_gbl_ptr)(vbase + it * 32 * AT_BS * 2 + lo.v),
+                                     (at_lds_ptr)(vbuf + (it * 4 + wave) * 1024), 16, 0, 0);
 }
 
 __device__ static inline bf16x8 at_lds128(const char* p) {
@@ -201,13 +201,222 @@ struct AtBlocks {
 };
 
 #define AT_WAIT_VMCNT0() __builtin_amdgcn_s_waitcnt(0x0F70)  // vmcnt(0) only: the direct-to-LDS loads have landed
+#define AT_PIN() __builtin_amdgcn_sched_barrier(0)            // nothing is scheduled across this point
+// lane-derived values from an opaque copy of the thread index (not loop invariant as far as the compiler knows)
+#define AT_LANE_VIEW(tv)                         \
+  int tv##_o = (tv);                             \
+  asm volatile("" : "+v"(tv##_o));               \
+  const int lq = tv##_o & 31, g = (tv##_o >> 5) & 1; \
+  const int q_off = (tv##_o >> 6) * 32 + lq
+
+// ---- the software pipeline of one wave ------------------------------------------------------------------------
+// Keys are consumed in half-tiles of 32 (one 32x32 accumulator of S^T per wave).  For half-tile j the wave issues,
+// in ONE instruction stream,
+//     S(j+1) = K(j+1) . Q^T        8 MFMAs   (matrix core)
+//     O     += V^T(j-1) . P(j-1)   8 MFMAs   (matrix core)
+//     P(j)   = exp2(S(j)*scale - m), row sums, bf16 packing     ~56 vector instructions
+// interleaved one MFMA : one LDS operand read : three or four vector instructions.  A wave issues in order but
+// an MFMA executes for 32 cycles after it is issued, so the vector work of half-tile j runs in the shadow of the
+// matrix work of its neighbours; scheduling barriers pin that order.  The running max is taken before the fused
+// stage; when it moves (rare after the first tiles) the pending P(j-1) is flushed into O first, O and the row
+// sums are rescaled, and the stage runs without its P.V part.
+struct AtPipe {
+  const int* koff;  // [8] lane-constant byte offsets of the K operand chunks (k-step ks), swizzle applied
+  const int* voff;  // [4] same for V^T, index kt*2 + s
+};
+
+typedef uint32_t at_u32x4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t at_pack2(float a, float b) {
+  floatx2 f;
+  f[0] = a;
+  f[1] = b;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
+// KH: which 32-key half of the K buffer S_out is computed from; KT: which half of the V^T buffer P_prev belongs to
+// compile-time loop: f(std::integral_constant<int, K>) for K = 0 .. N-1
+template <int K, int N, typename F>
+__device__ __forceinline__ void at_static_for(F&& f) {
+  if constexpr (K < N) {
+    f(std::integral_constant<int, K>{});
+    at_static_for<K + 1, N>(f);
+  }
+}
+
+// LDS operand fetch the compiler does not track: it returns at once and the register is valid only after an
+// explicit AT_WAIT_LGKM(n) (n = younger fetches allowed to be still in flight; LDS reads return in order).
+// Reason: while direct-to-LDS tile loads are in flight the compiler waits for ALL outstanding LDS reads before
+// every use of any of them, which exposes the full LDS latency in front of each MFMA.
+template <int IMM>
+__device__ __forceinline__ bf16x8 at_lds128_async(uint32_t addr) {
+  at_u32x4 r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(IMM));
+  return __builtin_bit_cast(bf16x8, r);
+}
+#define AT_WAIT_LGKM(n) __builtin_amdgcn_s_waitcnt(0xC07F | ((n) << 8))
+
+__device__ __forceinline__ uint32_t at_lds_addr(const char* p) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
+}
+
+// KH: which 32-key half of the K buffer S_out is computed from; KT: which half of the V^T buffer P_prev belongs to
+template <bool DO_QK, bool DO_PV, int KH, int KT>
+__device__ __forceinline__ void at_fused(const char* kb, const char* vb, int koff, int voff,
+                                         const bf16x8 (&qb)[8], floatx16& s_out, const floatx16& s_in,
+                                         const bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2], floatx16 (&o)[4], float sc,
+                                         float neg_m, float& l_lane) {
+  constexpr int NM = (DO_QK ? 8 : 0) + (DO_PV ? 8 : 0);
+  static_assert(NM == 8 || NM == 16, "a fused stage has 8 or 16 MFMAs");
+  constexpr int EPS = 16 / NM;  // softmax elements handled per MFMA slot
+  constexpr int AHEAD = 2;      // LDS operands are fetched this many slots before their MFMA
+  bf16x8 opnd[NM];
+  float x[16], e[16];
+  uint32_t pk[8];
+  const uint32_t ka = at_lds_addr(kb) + (uint32_t)koff;  // buffers are 256-byte aligned: the XOR stays inside
+  const uint32_t va = at_lds_addr(vb) + (uint32_t)voff;
+  // slot k -> its MFMA: both kinds alternate (S, O, S, O, ...) so that dependent MFMAs are never adjacent
+  auto fetch = [&](auto kc) {
+    constexpr int k = decltype(kc)::value;
+    constexpr bool qk = DO_QK && (!DO_PV || (k & 1) == 0);
+    constexpr int i = (DO_QK && DO_PV) ? (k >> 1) : k;
+    if constexpr (qk)
+      opnd[k] = at_lds128_async<KH * 32 * 256>(ka ^ (uint32_t)(i << 5));
+    else
+      opnd[k] = at_lds128_async<(i & 3) * 32 * 128>(va ^ (uint32_t)((KT * 2 + (i >> 2)) << 5));
+  };
+  at_static_for<0, AHEAD>(fetch);
+  AT_PIN();
+  at_static_for<0, NM>([&](auto kc) {
+    constexpr int k = decltype(kc)::value;
+    constexpr bool qk = DO_QK && (!DO_PV || (k & 1) == 0);
+    constexpr int i = (DO_QK && DO_PV) ? (k >> 1) : k;
+    constexpr int in_flight_after = (NM - 1 - k) < (AHEAD - 1) ? (NM - 1 - k) : (AHEAD - 1);
+    AT_WAIT_LGKM(in_flight_after);  // operand k has landed
+    AT_PIN();
+    if constexpr (qk) {
+      if constexpr (i == 0)
+        s_out = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[k], qb[0], (floatx16){0}, 0, 0, 0);
+      else
+        s_out = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[k], qb[i], s_out, 0, 0, 0);
+    } else {
+      o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[k], p_prev[i >> 2], o[i & 3], 0, 0, 0);
+    }
+    if constexpr (k + AHEAD < NM) fetch(std::integral_constant<int, k + AHEAD>{});
+#pragma unroll
+    for (int u = 0; u < EPS; ++u) {
+      const int idx = k * EPS + u;
+      x[idx] = __builtin_fmaf(s_in[idx], sc, neg_m);
+      if (idx >= 1) e[idx - 1] = __builtin_amdgcn_exp2f(x[idx - 1]);
+      if (idx >= 2) l_lane += e[idx - 2];
+      if (idx >= 3 && ((idx - 3) & 1) == 0) pk[(idx - 3) >> 1] = at_pack2(e[idx - 3], e[idx - 2]);
+    }
+    AT_PIN();
+  });
+  e[15] = __builtin_amdgcn_exp2f(x[15]);
+  l_lane += e[14];
+  l_lane += e[15];
+  pk[7] = at_pack2(e[14], e[15]);
+  at_u32x4 w0, w1;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    w0[j] = pk[j];
+    w1[j] = pk[4 + j];
+  }
+  p_out[0] = __builtin_bit_cast(bf16x8, w0);
+  p_out[1] = __builtin_bit_cast(bf16x8, w1);
+}
+
+// MFMA-only stages (no vector work to hide): first S of a row, flush of a pending P, last P.V of a row
+template <int KH>
+__device__ __forceinline__ void at_qk_only(const char* kb, int koff, const bf16x8 (&qb)[8], floatx16& s_out) {
+  bf16x8 a[8];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) a[ks] = at_lds128(kb + (koff ^ (ks << 5)) + KH * 32 * 256);
+  AT_PIN();
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    if (ks + 4 < 8) a[ks + 4] = at_lds128(kb + (koff ^ ((ks + 4) << 5)) + KH * 32 * 256);
+    if (ks == 0)
+      s_out = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qb[0], (floatx16){0}, 0, 0, 0);
+    else
+      s_out = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], qb[ks], s_out, 0, 0, 0);
+    AT_PIN();
+  }
+}
+
+template <int KT>
+__device__ __forceinline__ void at_pv_only(const char* vb, int voff, const bf16x8 (&p)[2], floatx16 (&o)[4]) {
+  bf16x8 a[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a[i] = at_lds128(vb + (voff ^ ((KT * 2 + (i >> 2)) << 5)) + (i & 3) * 32 * 128);
+  AT_PIN();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if (i + 4 < 8) a[i + 4] = at_lds128(vb + (voff ^ ((KT * 2 + ((i + 4) >> 2)) << 5)) + ((i + 4) & 3) * 32 * 128);
+    o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], p[i >> 2], o[i & 3], 0, 0, 0);
+    AT_PIN();
+  }
+}
+
+// causal predicate inside the diagonal block; key_base = offset of the half-tile's first key inside the block
+__device__ __forceinline__ void at_causal(floatx16& s, int key_base, int t) {
+  AT_LANE_VIEW(t);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int key_off = key_base + 8 * (i >> 2) + 4 * g + (i & 3);
+    s[i] = (key_off <= q_off) ? s[i] : -INFINITY;
+  }
+}
+
+// max over the lane's 16 keys and over the partner lane (lane ^ 32) that holds the other 16 keys of the query
+__device__ __forceinline__ float at_rowmax(const floatx16& s) {
+  float mx = s[0];
+#pragma unroll
+  for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
+  const uint32_t u = __builtin_bit_cast(uint32_t, mx);
+  const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // (lower half's value, upper half's value)
+  return fmaxf(__builtin_bit_cast(float, (uint32_t)sw[0]), __builtin_bit_cast(float, (uint32_t)sw[1]));
+}
+
+// One pipeline step.  s_in = S(j) (complete), p_prev = P(j-1) not yet applied to O (HAVE_PREV).
+// When some query's running max moves, the pending P(j-1) -- computed against the old max -- is flushed into O
+// first, O and the row sums are rescaled, and P(j-1) is cleared so that the fused stage's P.V part adds nothing.
+// The fused stage itself exists once per step: O never lives in two register sets that would have to be merged.
+template <bool DO_QK, bool HAVE_PREV, int KH, int KT>
+__device__ __forceinline__ void at_step(const char* kb, const char* vb, int koff, int voff, const bf16x8 (&qb)[8],
+                                        floatx16& s_out, floatx16& s_in, bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
+                                        floatx16 (&o)[4], float scale_log2, float& m_run, float& l_lane, bool diag,
+                                        int key_base, int t) {
+  if (diag) at_causal(s_in, key_base, t);
+  const float m_new = fmaxf(m_run, at_rowmax(s_in) * scale_log2);
+  if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {  // some row's max moved
+    if (HAVE_PREV) {
+      at_pv_only<KT>(vb, voff, p_prev, o);
+      p_prev[0] = __builtin_bit_cast(bf16x8, (at_u32x4){0, 0, 0, 0});
+      p_prev[1] = p_prev[0];
+    }
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_run = -inf on a row's first keys: alpha = 0
+    l_lane *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+    m_run = m_new;
+  }
+  // a query with nothing unmasked so far keeps m_run = -inf; exp2(-inf - (-inf)) must not be evaluated
+  const float neg_m = (m_run == -INFINITY) ? 0.f : -m_run;
+  at_fused<DO_QK, HAVE_PREV, KH, KT>(kb, vb, koff, voff, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, l_lane);
+}
 
 __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ vt,
     const uint64_t* __restrict__ mask, const int32_t* __restrict__ decision, sp_bf16* __restrict__ out,
     float2* __restrict__ rowstat, int64_t n, int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n,
     int64_t sk_h, int nb, int nbw, float scale_log2, int* __restrict__ sched) {
-  extern __shared__ __attribute__((aligned(1024))) char lds[];  // 2 stages x 32 KiB
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // K buffers 0,1 | V^T buffers 0,1
   __shared__ int s_queue, s_ticket;
 
   AtGeom gm;
@@ -218,21 +427,26 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
   const int xcd = blockIdx.x & 7;
   int first_try = 0;  // queues before this offset are known to be empty (used by thread 0 only)
   const int t = threadIdx.x;
-  const int wave = t >> 6, lane = t & 63;
-  const int lq = lane & 31, g = lane >> 5;
-  const int q_off = wave * 32 + lq;  // query offset inside the block
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
 
-  // lane-constant LDS read offsets (bytes) inside a stage
-  int koff[8];  // K rows lq (+32 via immediate), logical chunk 2*ks + g
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks) koff[ks] = lq * 256 + (((2 * ks + g) ^ (lq & 15)) << 4);
-  int voff[4];  // V^T rows lq (+32*dt via immediate), logical chunk 4*kt + 2*s + g, index kt*2+s
-#pragma unroll
-  for (int j = 0; j < 4; ++j) voff[j] = AT_KSTAGE_BYTES + lq * 128 + (((2 * j + g) ^ ((lq >> 1) & 7)) << 4);
+  // Lane-constant LDS read offsets (bytes) inside a buffer.  With lq = lane % 32 (the lane's row in a 32-row
+  // operand tile) and g = lane / 32, the XOR swizzle makes the operand of k-step ks (K) or of key group j (V^T)
+  // sit at (offset ^ (index << 5)):
+  //   K  : row lq (+32 via immediate), logical chunk 2*ks + g      -> lq*256 + (((2*ks + g) ^ (lq & 15)) << 4)
+  //   V^T: row lq (+32*dt via immediate), logical chunk 2*j + g    -> lq*128 + (((2*j + g) ^ ((lq >> 1) & 7)) << 4)
+  // Only these, the two global load offsets and t stay in registers across the key loop; everything else that
+  // depends on the lane is recomputed where it is needed from an opaque copy of t (AT_LANE_VIEW), so that the
+  // compiler does not carry a dozen precomputed lane constants through the loop.
+  int koff, voff;
   AtLoadOffsets lo;
-  at_load_offsets(lo, sk_n, wave, lane);
-
-  const bf16x8 ones = __builtin_bit_cast(bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
+  {
+    const int lane = t & 63, lq = lane & 31, g = lane >> 5;
+    koff = lq * 256 + ((g ^ (lq & 15)) << 4);
+    voff = lq * 128 + ((g ^ ((lq >> 1) & 7)) << 4);
+    at_load_offsets(lo, sk_n, wave, lane);
+  }
+  char* const kbuf0 = lds;
+  char* const vbuf0 = lds + 2 * AT_KBUF_BYTES;
 
   for (;;) {
     __syncthreads();  // previous item's LDS reads are done
@@ -262,13 +476,12 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
     AtBlocks it;
     it.init(mrow, r);
     int c_cur = it.next();
-    int half = 0;
-    int buf = 0;
-    if (c_cur >= 0) at_issue_sub(lo, kh, vth, n, sk_n, c_cur, 0, lds, wave, lane);
+    if (c_cur >= 0) at_issue_k(lo, kh, n, sk_n, c_cur, 0, kbuf0, wave, t);
 
     // Q^T operand: this lane's query, 8 k-steps of 8 channels
     bf16x8 qb[8];
     {
+      AT_LANE_VIEW(t);
       int64_t qrow = (int64_t)r * AT_BS + q_off;
       if (qrow > n - 1) qrow = n - 1;
       const sp_bf16* src = q + (int64_t)h * sq_h + qrow * sq_n + 8 * g;
@@ -280,115 +493,66 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
     floatx16 o[4];
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) o[dt] = (floatx16){0};
-    float m_run = -INFINITY, l_run = 0.f;
+    float m_run = -INFINITY, l_lane = 0.f;
 
-    while (c_cur >= 0) {
-      // this sub-tile has landed (own loads), and every wave is past the previous sub-tile's compute
+    if (c_cur >= 0) {
+      floatx16 sa, sb;
+      bf16x8 pa[2], pb[2];
+      // ---- sub-tile 0: nothing to overlap with yet ----
       AT_WAIT_VMCNT0();
       __syncthreads();
-      // ---- start fetching the next sub-tile into the other stage ----
-      int c_next = c_cur, half_next = 1;
-      if (half == 1) {
-        c_next = it.next();
-        half_next = 0;
-      }
-      if (c_next >= 0)
-        at_issue_sub(lo, kh, vth, n, sk_n, c_next, half_next, lds + (buf ^ 1) * AT_STAGE_BYTES, wave, lane);
-
-      const char* st = lds + buf * AT_STAGE_BYTES;
-      // ---- S^T = K . Q^T for 64 keys; LDS operands are fetched two k-steps ahead of their MFMAs ----
-      floatx16 s[2];
-      s[0] = (floatx16){0};
-      s[1] = (floatx16){0};
-      {
-        bf16x8 xa[3][2];
-        xa[0][0] = at_lds128(st + koff[0]);
-        xa[0][1] = at_lds128(st + koff[0] + 32 * 256);
-        xa[1][0] = at_lds128(st + koff[1]);
-        xa[1][1] = at_lds128(st + koff[1] + 32 * 256);
-        __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-          if (ks + 2 < 8) {
-            xa[(ks + 2) % 3][0] = at_lds128(st + koff[ks + 2]);
-            xa[(ks + 2) % 3][1] = at_lds128(st + koff[ks + 2] + 32 * 256);
-          }
-          s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[ks % 3][0], qb[ks], s[0], 0, 0, 0);
-          s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[ks % 3][1], qb[ks], s[1], 0, 0, 0);
+      at_issue_k(lo, kh, n, sk_n, c_cur, 1, kbuf0 + AT_KBUF_BYTES, wave, t);
+      at_issue_v(lo, vth, c_cur, 0, vbuf0, wave);
+      at_qk_only<0>(kbuf0, koff, qb, sa);
+      at_step<true, false, 1, 0>(kbuf0, vbuf0, koff, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane,
+                                 c_cur == r, 0, t);
+      // ---- steady state: sub-tile ti supplies K, sub-tile ti-1 supplies V^T ----
+      int c_prev = c_cur, half_prev = 0;
+      int half = 1;
+      int ti = 1;
+      for (;;) {
+        AT_WAIT_VMCNT0();
+        __syncthreads();  // K(ti) and V^T(ti-1) have landed; every wave is past sub-tile ti-1's K and ti-2's V^T
+        // (hidden loop invariance, as for koff/voff below: no precomputed 64-bit copies that could be spilled --
+        // a scratch reload here would wait for the tile loads just issued)
+        asm volatile("" : "+v"(lo.k), "+v"(lo.v));
+        int c_next = c_cur, half_next = 1;
+        if (half == 1) {
+          c_next = it.next();
+          half_next = 0;
         }
-        __builtin_amdgcn_s_setprio(0);
+        if (c_next >= 0)
+          at_issue_k(lo, kh, n, sk_n, c_next, half_next, kbuf0 + ((ti + 1) & 1) * AT_KBUF_BYTES, wave, t);
+        at_issue_v(lo, vth, c_cur, half, vbuf0 + (ti & 1) * AT_VBUF_BYTES, wave);
+        const char* kb = kbuf0 + (ti & 1) * AT_KBUF_BYTES;
+        const char* vb = vbuf0 + ((ti - 1) & 1) * AT_VBUF_BYTES;
+        // the operand addresses are one XOR away from these two registers; hiding their loop invariance keeps
+        // the compiler from precomputing (and spilling) all twelve of them
+        asm volatile("" : "+v"(koff), "+v"(voff));
+        // S(sub-tile ti-1, keys 32..63) -> P;  S(ti, keys 0..31) on the matrix core;  O += V^T(ti-1, keys 0..31) . P
+        at_step<true, true, 0, 0>(kb, vb, koff, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, c_prev == r,
+                                  half_prev * AT_SUB + 32, t);
+        at_step<true, true, 1, 1>(kb, vb, koff, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, c_cur == r,
+                                  half * AT_SUB, t);
+        c_prev = c_cur;
+        half_prev = half;
+        c_cur = c_next;
+        half = half_next;
+        ++ti;
+        if (c_cur < 0) break;
       }
-      // ---- online softmax (base 2): running max on raw logits, scale folded into the exponent ----
-      if (c_cur == r) {
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int key_off = half * AT_SUB + kt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-            s[kt][i] = (key_off <= q_off) ? s[kt][i] : -INFINITY;
-          }
-      }
-      float mx = -INFINITY;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, SP_WAVE));
-      const float m_new = fmaxf(m_run, mx * scale_log2);
-      if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {  // some row's max moved: rescale
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        l_run *= alpha;
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
-        m_run = m_new;
-      }
-      // a row with nothing unmasked so far keeps m_run = -inf; exp2(-inf - (-inf)) must not be evaluated
-      const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-          s[kt][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], scale_log2, -m_use));
-      // ---- O^T += V^T . P^T; V^T operands fetched one (kt, dt) step ahead ----
+      // ---- drain: the last sub-tile's second half and its P.V ----
+      AT_WAIT_VMCNT0();
+      __syncthreads();
       {
-        bf16x8 pb[2][2];
-        pb[0][0] = at_pack8(s[0], 0);
-        pb[0][1] = at_pack8(s[0], 8);
-        pb[1][0] = at_pack8(s[1], 0);
-        pb[1][1] = at_pack8(s[1], 8);
-        bf16x8 va[2][2];
-        va[0][0] = at_lds128(st + voff[0]);
-        va[0][1] = at_lds128(st + voff[1]);
-        __builtin_amdgcn_s_setprio(1);
-        // row sums of the bf16 probabilities on the matrix core: ones(32x16) . P^T puts sum_k P[k][q] of the
-        // lane's query into every accumulator row (this replaces 32 dependent vector adds per sub-tile)
-        floatx16 rs = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[0][0], (floatx16){0}, 0, 0, 0);
-        rs = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[0][1], rs, 0, 0, 0);
-#pragma unroll
-        for (int step = 0; step < 8; ++step) {  // step = kt*4 + dt
-          const int kt = step >> 2, dt = step & 3;
-          if (step + 1 < 8) {
-            const int kt1 = (step + 1) >> 2, dt1 = (step + 1) & 3;
-            va[(step + 1) & 1][0] = at_lds128(st + voff[kt1 * 2 + 0] + dt1 * 32 * 128);
-            va[(step + 1) & 1][1] = at_lds128(st + voff[kt1 * 2 + 1] + dt1 * 32 * 128);
-          }
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[step & 1][0], pb[kt][0], o[dt], 0, 0, 0);
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[step & 1][1], pb[kt][1], o[dt], 0, 0, 0);
-          if (step == 3) {
-            rs = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[1][0], rs, 0, 0, 0);
-            rs = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[1][1], rs, 0, 0, 0);
-          }
-        }
-        __builtin_amdgcn_s_setprio(0);
-        l_run += rs[0];  // the MFMA contracts over both lane halves: all 64 keys of the sub-tile for this query
+        const char* vb = vbuf0 + ((ti - 1) & 1) * AT_VBUF_BYTES;
+        at_step<false, true, 0, 0>(kbuf0, vb, koff, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane,
+                                   c_prev == r, half_prev * AT_SUB + 32, t);
+        at_pv_only<1>(vb, voff, pb, o);
       }
-      buf ^= 1;
-      c_cur = c_next;
-      half = half_next;
     }
-    const float l_tot = l_run;
+    const float l_tot = l_lane + __shfl_xor(l_lane, 32, SP_WAVE);
+    AT_LANE_VIEW(t);
 
     // pivot heads: keep the softmax statistics of every query row for the block-average pass
     if (rowstat != nullptr && decision != nullptr && decision[h] == SP_DEC_DENSE && g == 0) {
@@ -416,11 +580,11 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
     __syncthreads();
 #pragma unroll
     for (int i8 = 0; i8 < 8; ++i8) {
-      const int row = i8 * 16 + (t >> 4);
+      const int row = i8 * 16 + (t_o >> 4);
       const int64_t qrow = (int64_t)r * AT_BS + row;
       if (qrow < n) {
-        *reinterpret_cast<uint4*>(out + (qrow * hq + h) * AT_D + (t & 15) * 8) =
-            *reinterpret_cast<const uint4*>(reinterpret_cast<sp_bf16*>(lds) + row * AT_PITCH + (t & 15) * 8);
+        *reinterpret_cast<uint4*>(out + (qrow * hq + h) * AT_D + (t_o & 15) * 8) =
+            *reinterpret_cast<const uint4*>(reinterpret_cast<sp_bf16*>(lds) + row * AT_PITCH + (t_o & 15) * 8);
       }
     }
   }
@@ -565,7 +729,7 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(sp_zero_i32_kernel, dim3(1), dim3(128), 0, s, counter, 8 * 16);
   SP_LAUNCH_CHECK();
-  const size_t lds_bytes = 2 * AT_STAGE_BYTES;
+  const size_t lds_bytes = AT_LDS_BYTES;
   static int n_cu = 0;
   if (n_cu == 0) {
     int dev = 0;
