@@ -70,18 +70,22 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 }
 
 // ---- work distribution ----------------------------------------------------------------------------------
-// The kernel is persistent, 2 workgroups per CU.  Work items are (head, query block) rows, grouped in gangs of
-// AT_GANG consecutive query blocks of ONE head.  Gangs are dealt statically to the 8 XCDs (queue x = gang
-// position % 8; workgroup b serves queue b % 8 first -- workgroups are placed on XCDs round-robin), so the
-// 64 workgroups of an XCD start a gang together at column 0 and sweep the key blocks nearly in lock-step:
-// every K / V^T tile one of them pulls into the XCD's L2 is hit by the others.  The head order inside a kv
-// group is rotated from chunk to chunk so that every queue sees every head, heavy (late) rows go first, and a
-// workgroup whose queue is empty steals from the other queues.  Pulling is by atomic tickets only: nobody
-// ever waits for anybody, and every workgroup leaves once all eight queues are exhausted.
-#define AT_GANG 64
+// The kernel is persistent, one workgroup of 8 waves per CU.  A work item is a PAIR of adjacent query blocks
+// (rows 2p, 2p+1) of one head: waves 0-3 own the even row, waves 4-7 the odd row, and both consume the same
+// K / V^T tiles from LDS (the union of the two rows' masks), which halves the L2->LDS traffic wherever
+// neighbouring rows keep the same columns.  Items are grouped in gangs of AT_GANG consecutive pairs of ONE
+// head.  Gangs are dealt statically to the 8 XCDs (queue x = gang position % 8; workgroup b serves queue b % 8
+// first -- workgroups are placed on XCDs round-robin), so the 32 workgroups of an XCD start a gang together at
+// column 0 and sweep the key blocks nearly in lock-step: every K / V^T tile one of them pulls into the XCD's
+// L2 is hit by the others.  The head order inside a kv group is rotated from chunk to chunk so that every
+// queue sees every head, heavy (late) rows go first, and a workgroup whose queue is empty steals from the
+// other queues.  Pulling is by atomic tickets only: nobody ever waits for anybody, and every workgroup leaves
+// once all eight queues are exhausted.
+#define AT_GANG 32
+#define AT_FWD_THREADS 512
 
 struct AtGeom {
-  int group, nb, n_chunks, n_gangs;
+  int group, n_pairs, n_chunks, n_gangs;
 };
 
 __device__ static inline int at_queue_items(const AtGeom& gm, int xq) {
@@ -89,38 +93,41 @@ __device__ static inline int at_queue_items(const AtGeom& gm, int xq) {
   return gangs * AT_GANG;
 }
 
-// ticket of queue xq -> (head, query block); false for the padding slots of the last row chunk
-__device__ static inline bool at_item(const AtGeom& gm, int xq, int ticket, int& h, int& r) {
+// ticket of queue xq -> (head, row pair); false for the padding slots of the last chunk
+__device__ static inline bool at_item(const AtGeom& gm, int xq, int ticket, int& h, int& pair) {
   const int pos = (ticket / AT_GANG) * 8 + xq;  // gang position
   const int slot = ticket % AT_GANG;
   const int i = pos % gm.group;
   const int rest = pos / gm.group;
-  const int j = rest % gm.n_chunks;  // row chunk, 0 = the last (heaviest) rows
+  const int j = rest % gm.n_chunks;  // chunk of pairs, 0 = the last (heaviest) rows
   const int kvh = rest / gm.n_chunks;
   h = kvh * gm.group + (i + j) % gm.group;
-  r = gm.nb - 1 - (j * AT_GANG + slot);
-  return r >= 0;
+  pair = gm.n_pairs - 1 - (j * AT_GANG + slot);
+  return pair >= 0;
 }
 
 // ---- LDS staging -------------------------------------------------------------------------------------------
-// A block is processed as two sub-tiles of 64 keys.  LDS holds two K sub-tile buffers [64 keys][16 chunks] and
-// two V^T sub-tile buffers [128 channels][8 chunks] (chunk = 16 bytes = 8 bf16), 16 KiB each.  Tiles are filled
-// by direct global->LDS 128-bit loads: lane i of a wave writes LDS chunk (base + i), fetching whichever global
-// chunk belongs there.  Instead of row padding the chunk index is XOR-swizzled with the row,
+// A block is processed as two sub-tiles of 64 keys.  LDS holds a ring of four K sub-tile buffers
+// [64 keys][16 chunks] and a ring of four V^T sub-tile buffers [128 channels][8 chunks] (chunk = 16 bytes =
+// 8 bf16), 16 KiB each.  While sub-tile u is computed on (K of u, V^T of u-1: the P.V product trails by one
+// sub-tile), K of u+1..u+3 and V^T of u..u+2 are in flight.  Tiles are filled by direct global->LDS 128-bit
+// loads: lane i of a wave writes LDS chunk (base + i), fetching whichever global chunk belongs there.  Instead
+// of row padding the chunk index is XOR-swizzled with the row,
 //   K  : chunk c of row r sits at r*16 + (c ^ (r & 15))
 //   V^T: chunk c of row r sits at r*8  + (c ^ ((r >> 1) & 7))
 // so the 16 lanes that read the same logical chunk of 16 consecutive rows hit 16 different bank groups.
 #define AT_SUB 64
+#define AT_RING 4
 #define AT_KBUF_BYTES (AT_SUB * AT_D * 2)  // 16 KiB
 #define AT_VBUF_BYTES (AT_D * AT_SUB * 2)  // 16 KiB
-#define AT_LDS_BYTES (2 * AT_KBUF_BYTES + 2 * AT_VBUF_BYTES)
+#define AT_LDS_BYTES (AT_RING * (AT_KBUF_BYTES + AT_VBUF_BYTES))
 
 typedef __attribute__((address_space(3))) void* at_lds_ptr;
 typedef const __attribute__((address_space(1))) void* at_gbl_ptr;
 
 // Lane-constant byte offsets of the first K and V^T chunk a lane fetches per sub-tile.  A wave-instruction fills
-// one 1 KiB segment (seg = it*4 + wave): 4 K rows or 8 V^T rows.  Row and swizzle of a lane do not depend on `it`
-// beyond a uniform step (16 K rows / 32 V^T rows), which goes into the scalar base address.
+// one 1 KiB segment (seg = it*8 + wave, wave = 0..7): 4 K rows or 8 V^T rows.  Row and swizzle of a lane do not
+// depend on `it` beyond a uniform step (32 K rows / 64 V^T rows), which goes into the scalar base address.
 struct AtLoadOffsets {
   uint32_t k, v;
 };
@@ -132,15 +139,16 @@ __device__ static inline void at_load_offsets(AtLoadOffsets& lo, int64_t sk_n, i
   lo.v = (uint32_t)(vrow * AT_BS + (((lane & 7) ^ ((vrow >> 1) & 7)) * 8)) * 2u;
 }
 
+// two wave-instructions per wave and sub-tile
 __device__ static inline void at_issue_k(const AtLoadOffsets& lo, const sp_bf16* __restrict__ kh, int64_t n,
                                          int64_t sk_n, int c, int half, char* kbuf, int wave, int t) {
   const int64_t key0 = (int64_t)c * AT_BS + half * AT_SUB;
   if (key0 + AT_SUB <= n) {  // every key row exists: uniform base + lane-constant offset
     const char* kbase = reinterpret_cast<const char*>(kh + key0 * sk_n);
 #pragma unroll
-    for (int it = 0; it < 4; ++it)
-      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(kbase + (int64_t)it * 32 * sk_n + lo.k),
-                                       (at_lds_ptr)(kbuf + (it * 4 + wave) * 1024), 16, 0, 0);
+    for (int it = 0; it < 2; ++it)
+      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(kbase + (int64_t)it * 64 * sk_n + lo.k),
+                                       (at_lds_ptr)(kbuf + (it * 8 + wave) * 1024), 16, 0, 0);
   } else {  // ragged tail of the sequence: rows beyond the last key are clamped onto it
     const int64_t lim64 = n - 1 - key0;
     const int lim = lim64 < 0 ? 0 : (int)lim64;
@@ -148,8 +156,8 @@ __device__ static inline void at_issue_k(const AtLoadOffsets& lo, const sp_bf16*
     int ln = t & 63;
     asm volatile("" : "+v"(ln));  // keeps this rare path's lane arithmetic from being hoisted out of the key loop
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int seg = it * 4 + wave;
+    for (int it = 0; it < 2; ++it) {
+      const int seg = it * 8 + wave;
       const int row = seg * 4 + (ln >> 4);
       const int cl = (ln & 15) ^ (row & 15);
       const int rowc = row < lim ? row : lim;
@@ -164,9 +172,9 @@ __device__ static inline void at_issue_v(const AtLoadOffsets& lo, const sp_bf16*
                                          char* vbuf, int wave) {
   const char* vbase = reinterpret_cast<const char*>(vth + (int64_t)c * AT_D * AT_BS + half * AT_SUB);
 #pragma unroll
-  for (int it = 0; it < 4; ++it)
-    __builtin_amdgcn_global_load_lds((at_gbl_ptr)(vbase + it * 32 * AT_BS * 2 + lo.v),
-                                     (at_lds_ptr)(vbuf + (it * 4 + wave) * 1024), 16, 0, 0);
+  for (int it = 0; it < 2; ++it)
+    __builtin_amdgcn_global_load_lds((at_gbl_ptr)(vbase + it * 64 * AT_BS * 2 + lo.v),
+                                     (at_lds_ptr)(vbuf + (it * 8 + wave) * 1024), 16, 0, 0);
 }
 
 __device__ static inline bf16x8 at_lds128(const char* p) {
@@ -200,7 +208,47 @@ struct AtBlocks {
   }
 };
 
+// Iterator over the union of two adjacent mask rows (row ra: columns <= r0, row rb: columns <= r0 + 1; rb may be
+// absent).  wa / wb keep the causally trimmed words of the current 64-column group, so membership of the column
+// returned last is a bit test.  Everything here is uniform across the workgroup.
+struct AtUnion {
+  const uint64_t *ra, *rb;
+  int r0, wmax, w;
+  bool has_b;
+  uint64_t wa, wb, wu;
+  __device__ static uint64_t trim(uint64_t x, int wi, int r) {
+    if (wi > (r >> 6)) return 0ull;
+    if (wi == (r >> 6) && (r & 63) != 63) x &= (2ull << (r & 63)) - 1ull;
+    return x;
+  }
+  __device__ void load(int wi) {
+    wa = trim(ra[wi], wi, r0);
+    wb = has_b ? trim(rb[wi], wi, r0 + 1) : 0ull;
+    wu = wa | wb;
+  }
+  __device__ void init(const uint64_t* ra_, const uint64_t* rb_, int r0_, bool has_b_) {
+    ra = ra_;
+    rb = rb_;
+    r0 = r0_;
+    has_b = has_b_;
+    wmax = (has_b ? r0 + 1 : r0) >> 6;
+    w = 0;
+    load(0);
+  }
+  __device__ int next() {
+    while (wu == 0) {
+      if (++w > wmax) return -1;
+      load(w);
+    }
+    const int c = w * 64 + __builtin_ctzll(wu);
+    wu &= wu - 1;
+    return c;
+  }
+  __device__ bool in_row(int c, int which) const { return (((which ? wb : wa) >> (c & 63)) & 1ull) != 0ull; }
+};
+
 #define AT_WAIT_VMCNT0() __builtin_amdgcn_s_waitcnt(0x0F70)  // vmcnt(0) only: the direct-to-LDS loads have landed
+#define AT_WAIT_VMCNT8() __builtin_amdgcn_s_waitcnt(0x0F78)  // all but the 8 youngest vector-memory operations are done
 #define AT_PIN() __builtin_amdgcn_sched_barrier(0)            // nothing is scheduled across this point
 // lane-derived values from an opaque copy of the thread index (not loop invariant as far as the compiler knows)
 #define AT_LANE_VIEW(tv)                         \
@@ -411,31 +459,33 @@ __device__ __forceinline__ void at_step(const char* kb, const char* vb, int koff
   at_fused<DO_QK, HAVE_PREV, KH, KT>(kb, vb, koff, voff, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, l_lane);
 }
 
-__global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
+__global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ vt,
     const uint64_t* __restrict__ mask, const int32_t* __restrict__ decision, sp_bf16* __restrict__ out,
     float2* __restrict__ rowstat, int64_t n, int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n,
     int64_t sk_h, int nb, int nbw, float scale_log2, int* __restrict__ sched) {
-  extern __shared__ __attribute__((aligned(1024))) char lds[];  // K buffers 0,1 | V^T buffers 0,1
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // K ring (4 x 16 KiB) | V^T ring (4 x 16 KiB)
   __shared__ int s_queue, s_ticket;
 
   AtGeom gm;
   gm.group = hq / hkv;
-  gm.nb = nb;
-  gm.n_chunks = (nb + AT_GANG - 1) / AT_GANG;
+  gm.n_pairs = (nb + 1) / 2;
+  gm.n_chunks = (gm.n_pairs + AT_GANG - 1) / AT_GANG;
   gm.n_gangs = hq * gm.n_chunks;
   const int xcd = blockIdx.x & 7;
   int first_try = 0;  // queues before this offset are known to be empty (used by thread 0 only)
   const int t = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // 0..7
+  const int grp = wave >> 2;                                 // which row of the pair this wave works on
+  const int tq = t & 255;                                    // thread index inside the row's four waves
 
   // Lane-constant LDS read offsets (bytes) inside a buffer.  With lq = lane % 32 (the lane's row in a 32-row
   // operand tile) and g = lane / 32, the XOR swizzle makes the operand of k-step ks (K) or of key group j (V^T)
   // sit at (offset ^ (index << 5)):
   //   K  : row lq (+32 via immediate), logical chunk 2*ks + g      -> lq*256 + (((2*ks + g) ^ (lq & 15)) << 4)
   //   V^T: row lq (+32*dt via immediate), logical chunk 2*j + g    -> lq*128 + (((2*j + g) ^ ((lq >> 1) & 7)) << 4)
-  // Only these, the two global load offsets and t stay in registers across the key loop; everything else that
-  // depends on the lane is recomputed where it is needed from an opaque copy of t (AT_LANE_VIEW), so that the
+  // Only these, the two global load offsets and tq stay in registers across the key loop; everything else that
+  // depends on the lane is recomputed where it is needed from an opaque copy of tq (AT_LANE_VIEW), so that the
   // compiler does not carry a dozen precomputed lane constants through the loop.
   int koff, voff;
   AtLoadOffsets lo;
@@ -445,8 +495,8 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
     voff = lq * 128 + ((g ^ ((lq >> 1) & 7)) << 4);
     at_load_offsets(lo, sk_n, wave, lane);
   }
-  char* const kbuf0 = lds;
-  char* const vbuf0 = lds + 2 * AT_KBUF_BYTES;
+  char* const kring = lds;
+  char* const vring = lds + AT_RING * AT_KBUF_BYTES;
 
   for (;;) {
     __syncthreads();  // previous item's LDS reads are done
@@ -465,23 +515,24 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
       s_ticket = tk;
     }
     __syncthreads();
-    if (s_queue < 0) break;
-    int h, r;
-    if (!at_item(gm, s_queue, s_ticket, h, r)) continue;
+    const int queue = __builtin_amdgcn_readfirstlane(s_queue);
+    if (queue < 0) break;
+    const int ticket = __builtin_amdgcn_readfirstlane(s_ticket);
+    int h, pair;
+    if (!at_item(gm, queue, ticket, h, pair)) continue;
+    const int r0 = 2 * pair;
+    const bool has_b = r0 + 1 < nb;
+    const int r = r0 + grp;             // this wave's row
+    const bool row_ok = grp == 0 || has_b;
     const int kvh = h / gm.group;
     const sp_bf16* kh = k + (int64_t)kvh * sk_h;
     const sp_bf16* vth = vt + (int64_t)kvh * nb * AT_D * AT_BS;
-    const uint64_t* mrow = mask + ((int64_t)h * nb + r) * nbw;
-
-    AtBlocks it;
-    it.init(mrow, r);
-    int c_cur = it.next();
-    if (c_cur >= 0) at_issue_k(lo, kh, n, sk_n, c_cur, 0, kbuf0, wave, t);
+    const uint64_t* mrow = mask + ((int64_t)h * nb + r0) * nbw;
 
     // Q^T operand: this lane's query, 8 k-steps of 8 channels
     bf16x8 qb[8];
     {
-      AT_LANE_VIEW(t);
+      AT_LANE_VIEW(tq);
       int64_t qrow = (int64_t)r * AT_BS + q_off;
       if (qrow > n - 1) qrow = n - 1;
       const sp_bf16* src = q + (int64_t)h * sq_h + qrow * sq_n + 8 * g;
@@ -495,76 +546,130 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
     for (int dt = 0; dt < 4; ++dt) o[dt] = (floatx16){0};
     float m_run = -INFINITY, l_lane = 0.f;
 
-    if (c_cur >= 0) {
-      floatx16 sa, sb;
-      bf16x8 pa[2], pb[2];
-      // ---- sub-tile 0: nothing to overlap with yet ----
-      AT_WAIT_VMCNT0();
-      __syncthreads();
-      at_issue_k(lo, kh, n, sk_n, c_cur, 1, kbuf0 + AT_KBUF_BYTES, wave, t);
-      at_issue_v(lo, vth, c_cur, 0, vbuf0, wave);
-      at_qk_only<0>(kbuf0, koff, qb, sa);
-      at_step<true, false, 1, 0>(kbuf0, vbuf0, koff, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane,
-                                 c_cur == r, 0, t);
-      // ---- steady state: sub-tile ti supplies K, sub-tile ti-1 supplies V^T ----
-      int c_prev = c_cur, half_prev = 0;
-      int half = 1;
-      int ti = 1;
-      for (;;) {
-        AT_WAIT_VMCNT0();
-        __syncthreads();  // K(ti) and V^T(ti-1) have landed; every wave is past sub-tile ti-1's K and ti-2's V^T
-        // (hidden loop invariance, as for koff/voff below: no precomputed 64-bit copies that could be spilled --
-        // a scratch reload here would wait for the tile loads just issued)
-        asm volatile("" : "+v"(lo.k), "+v"(lo.v));
-        int c_next = c_cur, half_next = 1;
-        if (half == 1) {
-          c_next = it.next();
-          half_next = 0;
+    // Two walks over the union of the pair's masks: `ld` runs three sub-tiles ahead and feeds the loads.
+    // Sub-tile u lives in ring slot u % 4.  Every step issues the same number of loads (the waits count
+    // instructions): K of sub-tile u+3 and V^T of sub-tile u+2 -- the sub-tile whose K went out one step earlier.
+    // Past the end the last sub-tile is fetched again into a slot nobody reads any more.
+    AtUnion ld, cp;
+    ld.init(mrow, mrow + nbw, r0, has_b);
+    cp = ld;
+    int lc = ld.next(), lhalf = 0;  // sub-tile whose K is loaded next
+    int vc = lc, vhalf = 0;         // sub-tile whose V^T is loaded next
+    auto advance = [&]() {
+      if (lhalf == 0) {
+        lhalf = 1;
+      } else {
+        const int nx = ld.next();
+        if (nx >= 0) {
+          lc = nx;
+          lhalf = 0;
         }
-        if (c_next >= 0)
-          at_issue_k(lo, kh, n, sk_n, c_next, half_next, kbuf0 + ((ti + 1) & 1) * AT_KBUF_BYTES, wave, t);
-        at_issue_v(lo, vth, c_cur, half, vbuf0 + (ti & 1) * AT_VBUF_BYTES, wave);
-        const char* kb = kbuf0 + (ti & 1) * AT_KBUF_BYTES;
-        const char* vb = vbuf0 + ((ti - 1) & 1) * AT_VBUF_BYTES;
-        // the operand addresses are one XOR away from these two registers; hiding their loop invariance keeps
-        // the compiler from precomputing (and spilling) all twelve of them
-        asm volatile("" : "+v"(koff), "+v"(voff));
-        // S(sub-tile ti-1, keys 32..63) -> P;  S(ti, keys 0..31) on the matrix core;  O += V^T(ti-1, keys 0..31) . P
-        at_step<true, true, 0, 0>(kb, vb, koff, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, c_prev == r,
-                                  half_prev * AT_SUB + 32, t);
-        at_step<true, true, 1, 1>(kb, vb, koff, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, c_cur == r,
-                                  half * AT_SUB, t);
-        c_prev = c_cur;
-        half_prev = half;
-        c_cur = c_next;
-        half = half_next;
-        ++ti;
-        if (c_cur < 0) break;
       }
-      // ---- drain: the last sub-tile's second half and its P.V ----
-      AT_WAIT_VMCNT0();
-      __syncthreads();
-      {
-        const char* vb = vbuf0 + ((ti - 1) & 1) * AT_VBUF_BYTES;
-        at_step<false, true, 0, 0>(kbuf0, vb, koff, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane,
-                                   c_prev == r, half_prev * AT_SUB + 32, t);
-        at_pv_only<1>(vb, voff, pb, o);
+    };
+    if (lc >= 0) {
+#pragma unroll
+      for (int i = 0; i < 3; ++i) {  // steps -3..-1: K(0..2), V^T(0 [unused copy], 0, 1)
+        at_issue_k(lo, kh, n, sk_n, lc, lhalf, kring + i * AT_KBUF_BYTES, wave, t);
+        at_issue_v(lo, vth, vc, vhalf, vring + ((i + 3) & 3) * AT_VBUF_BYTES, wave);
+        vc = lc;
+        vhalf = lhalf;
+        advance();
       }
     }
+
+    // The compute walk.  Per sub-tile u every wave passes `top` exactly once (wait, barrier, issue), whatever its
+    // row does with the sub-tile.  A row's own sub-tiles come in runs; a run is one straight-line pipeline:
+    // start (first S), steady steps while the next sub-tile is the row's too, drain on the sub-tile after the run
+    // (V^T(u-1) is still resident while sub-tile u is current) or after the walk.
+    int u = 0;
+    int c_cur = cp.next(), half = 0;
+    bool mine = c_cur >= 0 && row_ok && cp.in_row(c_cur, grp);
+    const char *kb = kring, *vb = vring;
+    auto top = [&]() {
+      AT_WAIT_VMCNT8();              // K(u) and V^T(u-1) have landed (own loads)
+      __builtin_amdgcn_s_barrier();  // ... everybody's; and every wave is past sub-tile u-1
+      // (hidden loop invariance: no precomputed copies of these lane constants that could be spilled -- a scratch
+      // reload would wait for the tile loads just issued)
+      asm volatile("" : "+v"(lo.k), "+v"(lo.v));
+      at_issue_k(lo, kh, n, sk_n, lc, lhalf, kring + ((u + 3) & 3) * AT_KBUF_BYTES, wave, t);
+      at_issue_v(lo, vth, vc, vhalf, vring + ((u + 2) & 3) * AT_VBUF_BYTES, wave);
+      vc = lc;
+      vhalf = lhalf;
+      advance();
+      kb = kring + (u & 3) * AT_KBUF_BYTES;
+      vb = vring + ((u + 3) & 3) * AT_VBUF_BYTES;  // V^T(u-1)
+      asm volatile("" : "+v"(koff), "+v"(voff));
+    };
+    auto step_walk = [&]() {
+      ++u;
+      if (half == 0) {
+        half = 1;
+      } else {
+        c_cur = cp.next();
+        half = 0;
+        mine = c_cur >= 0 && row_ok && cp.in_row(c_cur, grp);
+      }
+    };
+    bool finished = false;  // the final wait + barrier has been passed
+    while (c_cur >= 0) {
+      top();
+      if (!mine) {
+        step_walk();
+        continue;
+      }
+      floatx16 sa, sb;
+      bf16x8 pa[2], pb[2];
+      // ---- start of a run: S of the first half-tile, nothing to overlap with yet ----
+      at_qk_only<0>(kb, koff, qb, sa);
+      at_step<true, false, 1, 0>(kb, vb, koff, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, c_cur == r,
+                                 half * AT_SUB, tq);
+      int c_prev = c_cur, half_prev = half;
+      step_walk();
+      // ---- steady state: sub-tile u supplies K, sub-tile u-1 supplies V^T ----
+      while (mine) {  // (mine implies c_cur >= 0)
+        top();
+        // S(u-1, keys 32..63) -> P;  S(u, keys 0..31) on the matrix core;  O += V^T(u-1, keys 0..31) . P
+        at_step<true, true, 0, 0>(kb, vb, koff, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, c_prev == r,
+                                  half_prev * AT_SUB + 32, tq);
+        at_step<true, true, 1, 1>(kb, vb, koff, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, c_cur == r,
+                                  half * AT_SUB, tq);
+        c_prev = c_cur;
+        half_prev = half;
+        step_walk();
+      }
+      // ---- drain: the run's last second half and its P.V ----
+      if (c_cur >= 0) {
+        top();
+        step_walk();
+      } else {
+        AT_WAIT_VMCNT0();
+        __syncthreads();
+        finished = true;
+        vb = vring + ((u + 3) & 3) * AT_VBUF_BYTES;
+      }
+      at_step<false, true, 0, 0>(kb, vb, koff, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, c_prev == r,
+                                 half_prev * AT_SUB + 32, tq);
+      at_pv_only<1>(vb, voff, pb, o);
+    }
+    if (!finished) {
+      AT_WAIT_VMCNT0();
+      __syncthreads();
+    }
     const float l_tot = l_lane + __shfl_xor(l_lane, 32, SP_WAVE);
-    AT_LANE_VIEW(t);
+    AT_LANE_VIEW(tq);
 
     // pivot heads: keep the softmax statistics of every query row for the block-average pass
-    if (rowstat != nullptr && decision != nullptr && decision[h] == SP_DEC_DENSE && g == 0) {
+    if (row_ok && rowstat != nullptr && decision != nullptr && decision[h] == SP_DEC_DENSE && g == 0) {
       const int64_t qrow = (int64_t)r * AT_BS + q_off;
       if (qrow < n) rowstat[(int64_t)h * n + qrow] = make_float2(m_run, l_tot);
     }
 
-    // ---- epilogue: normalise, transpose through LDS (padded rows), coalesced bf16 store ----
+    // ---- epilogue: normalise, transpose through LDS (padded rows, one region per row), coalesced bf16 store ----
     __syncthreads();
+    sp_bf16* stage_out = reinterpret_cast<sp_bf16*>(lds) + grp * (AT_BS * AT_PITCH);
     {
       const float inv_l = 1.0f / l_tot;
-      sp_bf16* orow = reinterpret_cast<sp_bf16*>(lds) + q_off * AT_PITCH;
+      sp_bf16* orow = stage_out + q_off * AT_PITCH;
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -578,13 +683,15 @@ __global__ __launch_bounds__(AT_THREADS, 2) void sp_attn_fwd_kernel(
         }
     }
     __syncthreads();
+    if (row_ok) {
 #pragma unroll
-    for (int i8 = 0; i8 < 8; ++i8) {
-      const int row = i8 * 16 + (t_o >> 4);
-      const int64_t qrow = (int64_t)r * AT_BS + row;
-      if (qrow < n) {
-        *reinterpret_cast<uint4*>(out + (qrow * hq + h) * AT_D + (t_o & 15) * 8) =
-            *reinterpret_cast<const uint4*>(reinterpret_cast<sp_bf16*>(lds) + row * AT_PITCH + (t_o & 15) * 8);
+      for (int i8 = 0; i8 < 8; ++i8) {
+        const int row = i8 * 16 + (tq_o >> 4);
+        const int64_t qrow = (int64_t)r * AT_BS + row;
+        if (qrow < n) {
+          *reinterpret_cast<uint4*>(out + (qrow * hq + h) * AT_D + (tq_o & 15) * 8) =
+              *reinterpret_cast<const uint4*>(stage_out + row * AT_PITCH + (tq_o & 15) * 8);
+        }
       }
     }
   }
@@ -740,9 +847,9 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
                                (int)lds_bytes));
     n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
-  const int64_t total = nb * hq;
-  const int grid = (int)(total < 2ll * n_cu ? ((total + 7) / 8) * 8 : 2ll * n_cu);
-  hipLaunchKernelGGL(sp_attn_fwd_kernel, dim3(grid), dim3(AT_THREADS), lds_bytes, s, (const sp_bf16*)q,
+  const int64_t total = ((nb + 1) / 2) * hq;  // row pairs
+  const int grid = (int)(total < (int64_t)n_cu ? ((total + 7) / 8) * 8 : (int64_t)n_cu);
+  hipLaunchKernelGGL(sp_attn_fwd_kernel, dim3(grid), dim3(AT_FWD_THREADS), lds_bytes, s, (const sp_bf16*)q,
                      (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out,
                      want_avg ? rowstat : (float2*)nullptr, n, hq, hkv, q_stride_n, q_stride_h, k_stride_n,
                      k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, counter);
