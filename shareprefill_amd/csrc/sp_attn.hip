@@ -19,6 +19,7 @@
 #include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
@@ -120,7 +121,9 @@ __device__ static inline bool at_item(const AtGeom& gm, int xq, int ticket, int&
 #define AT_RING 4
 #define AT_KBUF_BYTES (AT_SUB * AT_D * 2)  // 16 KiB
 #define AT_VBUF_BYTES (AT_D * AT_SUB * 2)  // 16 KiB
-#define AT_LDS_BYTES (AT_RING * (AT_KBUF_BYTES + AT_VBUF_BYTES))
+#define AT_LIST_MAX 4096                      // union blocks of a row pair (nb <= 4096)
+#define AT_LIST_BYTES (AT_LIST_MAX * 4)
+#define AT_LDS_BYTES (AT_RING * (AT_KBUF_BYTES + AT_VBUF_BYTES) + AT_LIST_BYTES)
 
 typedef __attribute__((address_space(3))) void* at_lds_ptr;
 typedef const __attribute__((address_space(1))) void* at_gbl_ptr;
@@ -139,38 +142,36 @@ __device__ static inline void at_load_offsets(AtLoadOffsets& lo, int64_t sk_n, i
   lo.v = (uint32_t)(vrow * AT_BS + (((lane & 7) ^ ((vrow >> 1) & 7)) * 8)) * 2u;
 }
 
-// two wave-instructions per wave and sub-tile
-__device__ static inline void at_issue_k(const AtLoadOffsets& lo, const sp_bf16* __restrict__ kh, int64_t n,
-                                         int64_t sk_n, int c, int half, char* kbuf, int wave, int t) {
-  const int64_t key0 = (int64_t)c * AT_BS + half * AT_SUB;
-  if (key0 + AT_SUB <= n) {  // every key row exists: uniform base + lane-constant offset
-    const char* kbase = reinterpret_cast<const char*>(kh + key0 * sk_n);
+// two wave-instructions per wave and sub-tile; kbase = address of the sub-tile's first key row
+__device__ static inline void at_issue_k(const AtLoadOffsets& lo, const char* kbase, int64_t sk_n, char* kbuf,
+                                         int wave) {
 #pragma unroll
-    for (int it = 0; it < 2; ++it)
-      __builtin_amdgcn_global_load_lds((at_gbl_ptr)(kbase + (int64_t)it * 64 * sk_n + lo.k),
-                                       (at_lds_ptr)(kbuf + (it * 8 + wave) * 1024), 16, 0, 0);
-  } else {  // ragged tail of the sequence: rows beyond the last key are clamped onto it
-    const int64_t lim64 = n - 1 - key0;
-    const int lim = lim64 < 0 ? 0 : (int)lim64;
-    const sp_bf16* kbase = kh + (lim64 < 0 ? (n - 1) : key0) * sk_n;
-    int ln = t & 63;
-    asm volatile("" : "+v"(ln));  // keeps this rare path's lane arithmetic from being hoisted out of the key loop
+  for (int it = 0; it < 2; ++it)
+    __builtin_amdgcn_global_load_lds((at_gbl_ptr)(kbase + (int64_t)it * 64 * sk_n + lo.k),
+                                     (at_lds_ptr)(kbuf + (it * 8 + wave) * 1024), 16, 0, 0);
+}
+
+// ragged tail of the sequence (last block only): rows beyond the last key are clamped onto it
+__device__ static inline void at_issue_k_tail(const sp_bf16* __restrict__ kh, int64_t n, int64_t sk_n, int64_t key0,
+                                              char* kbuf, int wave, int t) {
+  const int64_t lim64 = n - 1 - key0;
+  const int lim = lim64 < 0 ? 0 : (int)lim64;
+  const sp_bf16* kbase = kh + (lim64 < 0 ? (n - 1) : key0) * sk_n;
+  int lane = t & 63;
+  asm volatile("" : "+v"(lane));  // keeps this rare path's lane arithmetic from being hoisted out of the key loop
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int seg = it * 8 + wave;
-      const int row = seg * 4 + (ln >> 4);
-      const int cl = (ln & 15) ^ (row & 15);
-      const int rowc = row < lim ? row : lim;
-      const sp_bf16* g = kbase + (uint32_t)(rowc * (int)sk_n + cl * 8);
-      __builtin_amdgcn_global_load_lds((at_gbl_ptr)g, (at_lds_ptr)(kbuf + seg * 1024), 16, 0, 0);
-    }
+  for (int it = 0; it < 2; ++it) {
+    const int seg = it * 8 + wave;
+    const int row = seg * 4 + (lane >> 4);
+    const int cl = (lane & 15) ^ (row & 15);
+    const int rowc = row < lim ? row : lim;
+    const sp_bf16* g = kbase + (uint32_t)(rowc * (int)sk_n + cl * 8);
+    __builtin_amdgcn_global_load_lds((at_gbl_ptr)g, (at_lds_ptr)(kbuf + seg * 1024), 16, 0, 0);
   }
 }
 
-// the repacked V^T is zero-filled beyond the last key, so no tail case
-__device__ static inline void at_issue_v(const AtLoadOffsets& lo, const sp_bf16* __restrict__ vth, int c, int half,
-                                         char* vbuf, int wave) {
-  const char* vbase = reinterpret_cast<const char*>(vth + (int64_t)c * AT_D * AT_BS + half * AT_SUB);
+// the repacked V^T is zero-filled beyond the last key, so no tail case; vbase = first channel row of the sub-tile
+__device__ static inline void at_issue_v(const AtLoadOffsets& lo, const char* vbase, char* vbuf, int wave) {
 #pragma unroll
   for (int it = 0; it < 2; ++it)
     __builtin_amdgcn_global_load_lds((at_gbl_ptr)(vbase + it * 64 * AT_BS * 2 + lo.v),
@@ -208,47 +209,19 @@ struct AtBlocks {
   }
 };
 
-// Iterator over the union of two adjacent mask rows (row ra: columns <= r0, row rb: columns <= r0 + 1; rb may be
-// absent).  wa / wb keep the causally trimmed words of the current 64-column group, so membership of the column
-// returned last is a bit test.  Everything here is uniform across the workgroup.
-struct AtUnion {
-  const uint64_t *ra, *rb;
-  int r0, wmax, w;
-  bool has_b;
-  uint64_t wa, wb, wu;
-  __device__ static uint64_t trim(uint64_t x, int wi, int r) {
-    if (wi > (r >> 6)) return 0ull;
-    if (wi == (r >> 6) && (r & 63) != 63) x &= (2ull << (r & 63)) - 1ull;
-    return x;
-  }
-  __device__ void load(int wi) {
-    wa = trim(ra[wi], wi, r0);
-    wb = has_b ? trim(rb[wi], wi, r0 + 1) : 0ull;
-    wu = wa | wb;
-  }
-  __device__ void init(const uint64_t* ra_, const uint64_t* rb_, int r0_, bool has_b_) {
-    ra = ra_;
-    rb = rb_;
-    r0 = r0_;
-    has_b = has_b_;
-    wmax = (has_b ? r0 + 1 : r0) >> 6;
-    w = 0;
-    load(0);
-  }
-  __device__ int next() {
-    while (wu == 0) {
-      if (++w > wmax) return -1;
-      load(w);
-    }
-    const int c = w * 64 + __builtin_ctzll(wu);
-    wu &= wu - 1;
-    return c;
-  }
-  __device__ bool in_row(int c, int which) const { return (((which ? wb : wa) >> (c & 63)) & 1ull) != 0ull; }
-};
+// causally trimmed 64-column word wi of the mask row of query block r
+__device__ static inline uint64_t at_trim(uint64_t x, int wi, int r) {
+  if (wi > (r >> 6)) return 0ull;
+  if (wi == (r >> 6) && (r & 63) != 63) x &= (2ull << (r & 63)) - 1ull;
+  return x;
+}
+
+// entry of the per-pair block list: column | row-membership flags
+#define AT_IN_A (1u << 30)
+#define AT_IN_B (1u << 31)
+#define AT_COL_MASK 0x00FFFFFFu
 
 #define AT_WAIT_VMCNT0() __builtin_amdgcn_s_waitcnt(0x0F70)  // vmcnt(0) only: the direct-to-LDS loads have landed
-#define AT_WAIT_VMCNT8() __builtin_amdgcn_s_waitcnt(0x0F78)  // all but the 8 youngest vector-memory operations are done
 #define AT_PIN() __builtin_amdgcn_sched_barrier(0)            // nothing is scheduled across this point
 // lane-derived values from an opaque copy of the thread index (not loop invariant as far as the compiler knows)
 #define AT_LANE_VIEW(tv)                         \
@@ -275,7 +248,6 @@ struct AtPipe {
 
 typedef uint32_t at_u32x4 __attribute__((ext_vector_type(4)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ uint32_t at_pack2(float a, float b) {
   floatx2 f;
@@ -284,7 +256,6 @@ __device__ __forceinline__ uint32_t at_pack2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
 
-// KH: which 32-key half of the K buffer S_out is computed from; KT: which half of the V^T buffer P_prev belongs to
 // compile-time loop: f(std::integral_constant<int, K>) for K = 0 .. N-1
 template <int K, int N, typename F>
 __device__ __forceinline__ void at_static_for(F&& f) {
@@ -310,37 +281,59 @@ __device__ __forceinline__ uint32_t at_lds_addr(const char* p) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
 }
 
-// KH: which 32-key half of the K buffer S_out is computed from; KT: which half of the V^T buffer P_prev belongs to
-template <bool DO_QK, bool DO_PV, int KH, int KT>
-__device__ __forceinline__ void at_fused(const char* kb, const char* vb, int koff, int voff,
-                                         const bf16x8 (&qb)[8], floatx16& s_out, const floatx16& s_in,
-                                         const bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2], floatx16 (&o)[4], float sc,
-                                         float neg_m, float& l_lane) {
+// LDS addresses of a block's operands, one XOR each, made once per block: K k-step ks of sub-tile 2b at ka[ks]
+// (second half of the sub-tile and sub-tile 2b+1 via immediate offsets), V^T key group j of sub-tile 2b-1 at
+// va[0][j] and of sub-tile 2b at va[1][j].
+struct AtAddr {
+  uint32_t ka[8];
+  uint32_t va[2][4];
+};
+
+__device__ __forceinline__ void at_block_addr(AtAddr& ad, const char* kb, const char* vb, const char* vb1, int koff,
+                                              int voff) {
+  const uint32_t k0 = at_lds_addr(kb) + (uint32_t)koff;  // buffers are 256-byte aligned: the XOR stays inside
+  const uint32_t v0 = at_lds_addr(vb) + (uint32_t)voff, v1 = at_lds_addr(vb1) + (uint32_t)voff;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ad.ka[i] = k0 ^ (uint32_t)(i << 5);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    ad.va[0][j] = v0 ^ (uint32_t)(j << 5);
+    ad.va[1][j] = v1 ^ (uint32_t)(j << 5);
+  }
+}
+
+// KQ: which 32-key quarter (0..3) of the block's two K buffers S_out is computed from; VB / KT: which V^T buffer
+// (0: sub-tile 2b-1, 1: sub-tile 2b) and which half of it P_prev belongs to.
+// Slot order: the 8 MFMAs of S_out first (one dependent chain), then the 8 of O, so that S_out is complete early
+// enough for its in-lane maximum (mx_out) to be taken in the shadow of the last slots.
+template <bool DO_QK, bool DO_PV, int KQ, int VB, int KT>
+__device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[8], floatx16& s_out,
+                                         const floatx16& s_in, const bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
+                                         floatx16 (&o)[4], float sc, float neg_m, float& l_lane, float& mx_out) {
   constexpr int NM = (DO_QK ? 8 : 0) + (DO_PV ? 8 : 0);
   static_assert(NM == 8 || NM == 16, "a fused stage has 8 or 16 MFMAs");
   constexpr int EPS = 16 / NM;  // softmax elements handled per MFMA slot
   constexpr int AHEAD = 2;      // LDS operands are fetched this many slots before their MFMA
+  constexpr int MX0 = 11;       // first slot that takes part in the maximum of S_out (16-slot stages)
   bf16x8 opnd[NM];
   float x[16], e[16];
   uint32_t pk[8];
-  const uint32_t ka = at_lds_addr(kb) + (uint32_t)koff;  // buffers are 256-byte aligned: the XOR stays inside
-  const uint32_t va = at_lds_addr(vb) + (uint32_t)voff;
-  // slot k -> its MFMA: both kinds alternate (S, O, S, O, ...) so that dependent MFMAs are never adjacent
+  float mx = -INFINITY;
   auto fetch = [&](auto kc) {
     constexpr int k = decltype(kc)::value;
-    constexpr bool qk = DO_QK && (!DO_PV || (k & 1) == 0);
-    constexpr int i = (DO_QK && DO_PV) ? (k >> 1) : k;
+    constexpr bool qk = DO_QK && k < 8;
+    constexpr int i = k & 7;
     if constexpr (qk)
-      opnd[k] = at_lds128_async<KH * 32 * 256>(ka ^ (uint32_t)(i << 5));
+      opnd[k] = at_lds128_async<(KQ >> 1) * AT_KBUF_BYTES + (KQ & 1) * 32 * 256>(ad.ka[i]);
     else
-      opnd[k] = at_lds128_async<(i & 3) * 32 * 128>(va ^ (uint32_t)((KT * 2 + (i >> 2)) << 5));
+      opnd[k] = at_lds128_async<(i & 3) * 32 * 128>(ad.va[VB][KT * 2 + (i >> 2)]);
   };
   at_static_for<0, AHEAD>(fetch);
   AT_PIN();
   at_static_for<0, NM>([&](auto kc) {
     constexpr int k = decltype(kc)::value;
-    constexpr bool qk = DO_QK && (!DO_PV || (k & 1) == 0);
-    constexpr int i = (DO_QK && DO_PV) ? (k >> 1) : k;
+    constexpr bool qk = DO_QK && k < 8;
+    constexpr int i = k & 7;
     constexpr int in_flight_after = (NM - 1 - k) < (AHEAD - 1) ? (NM - 1 - k) : (AHEAD - 1);
     AT_WAIT_LGKM(in_flight_after);  // operand k has landed
     AT_PIN();
@@ -356,17 +349,45 @@ __device__ __forceinline__ void at_fused(const char* kb, const char* vb, int kof
 #pragma unroll
     for (int u = 0; u < EPS; ++u) {
       const int idx = k * EPS + u;
-      x[idx] = __builtin_fmaf(s_in[idx], sc, neg_m);
+      // The softmax arithmetic depends only on values known before the stage starts, and the optimiser would
+      // otherwise move all of it in front of the stage (out of the MFMAs' shadow): the empty asm ties each
+      // element to its slot.
+      float sv = s_in[idx];
+      asm volatile("" : "+v"(sv));
+      x[idx] = __builtin_fmaf(sv, sc, neg_m);
       if (idx >= 1) e[idx - 1] = __builtin_amdgcn_exp2f(x[idx - 1]);
-      if (idx >= 2) l_lane += e[idx - 2];
-      if (idx >= 3 && ((idx - 3) & 1) == 0) pk[(idx - 3) >> 1] = at_pack2(e[idx - 3], e[idx - 2]);
+      if (idx >= 3 && ((idx - 3) & 1) == 0) {
+        const int m = (idx - 3) >> 1;
+        pk[m] = at_pack2(e[idx - 3], e[idx - 2]);
+        l_lane += e[idx - 3];
+        l_lane += e[idx - 2];
+      }
+      // ... and the results to the slot they were produced in (instruction selection lets pure arithmetic float)
+      asm volatile("" : "+v"(x[idx]));
+      if (idx >= 1) asm volatile("" : "+v"(e[idx - 1]));
+      if (idx >= 3 && ((idx - 3) & 1) == 0) asm volatile("" : "+v"(pk[(idx - 3) >> 1]), "+v"(l_lane));
+    }
+    if constexpr (DO_QK && DO_PV && k >= MX0) {  // three elements of S_out per slot; the last slot takes four
+      constexpr int j0 = (k - MX0) * 3;
+      mx = fmaxf(mx, fmaxf(s_out[j0], s_out[j0 + 1]));
+      mx = fmaxf(mx, s_out[j0 + 2]);
+      if constexpr (k == NM - 1) {
+        static_assert(j0 + 3 == 15, "the maximum must cover all 16 elements");
+        mx = fmaxf(mx, s_out[15]);
+      }
+      asm volatile("" : "+v"(mx));
     }
     AT_PIN();
   });
   e[15] = __builtin_amdgcn_exp2f(x[15]);
+  pk[7] = at_pack2(e[14], e[15]);
   l_lane += e[14];
   l_lane += e[15];
-  pk[7] = at_pack2(e[14], e[15]);
+  if constexpr (DO_QK && !DO_PV) {  // start of a run: nothing to hide the maximum behind
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_out[i]);
+  }
+  mx_out = mx;
   at_u32x4 w0, w1;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -419,30 +440,39 @@ __device__ __forceinline__ void at_causal(floatx16& s, int key_base, int t) {
   }
 }
 
-// max over the lane's 16 keys and over the partner lane (lane ^ 32) that holds the other 16 keys of the query
-__device__ __forceinline__ float at_rowmax(const floatx16& s) {
+// max over the lane's 16 keys
+__device__ __forceinline__ float at_lanemax(const floatx16& s) {
   float mx = s[0];
 #pragma unroll
   for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
+  return mx;
+}
+
+// ... and over the partner lane (lane ^ 32) that holds the other 16 keys of the query
+__device__ __forceinline__ float at_pairmax(float mx) {
   const uint32_t u = __builtin_bit_cast(uint32_t, mx);
   const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // (lower half's value, upper half's value)
   return fmaxf(__builtin_bit_cast(float, (uint32_t)sw[0]), __builtin_bit_cast(float, (uint32_t)sw[1]));
 }
 
-// One pipeline step.  s_in = S(j) (complete), p_prev = P(j-1) not yet applied to O (HAVE_PREV).
+// One pipeline step.  s_in = S(j) (complete) with in-lane maximum mx_carry, p_prev = P(j-1) not yet applied to O
+// (HAVE_PREV); on return mx_carry is the in-lane maximum of s_out.
 // When some query's running max moves, the pending P(j-1) -- computed against the old max -- is flushed into O
 // first, O and the row sums are rescaled, and P(j-1) is cleared so that the fused stage's P.V part adds nothing.
 // The fused stage itself exists once per step: O never lives in two register sets that would have to be merged.
-template <bool DO_QK, bool HAVE_PREV, int KH, int KT>
-__device__ __forceinline__ void at_step(const char* kb, const char* vb, int koff, int voff, const bf16x8 (&qb)[8],
+template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT>
+__device__ __forceinline__ void at_step(const AtAddr& ad, const char* vbuf, int voff, const bf16x8 (&qb)[8],
                                         floatx16& s_out, floatx16& s_in, bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
-                                        floatx16 (&o)[4], float scale_log2, float& m_run, float& l_lane, bool diag,
-                                        int key_base, int t) {
-  if (diag) at_causal(s_in, key_base, t);
-  const float m_new = fmaxf(m_run, at_rowmax(s_in) * scale_log2);
+                                        floatx16 (&o)[4], float scale_log2, float& m_run, float& l_lane,
+                                        float& mx_carry, bool diag, int key_base, int t) {
+  if (diag) {  // the causal predicate changes the maximum: take it again
+    at_causal(s_in, key_base, t);
+    mx_carry = at_lanemax(s_in);
+  }
+  const float m_new = fmaxf(m_run, at_pairmax(mx_carry) * scale_log2);
   if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {  // some row's max moved
     if (HAVE_PREV) {
-      at_pv_only<KT>(vb, voff, p_prev, o);
+      at_pv_only<KT>(vbuf, voff, p_prev, o);
       p_prev[0] = __builtin_bit_cast(bf16x8, (at_u32x4){0, 0, 0, 0});
       p_prev[1] = p_prev[0];
     }
@@ -456,7 +486,7 @@ __device__ __forceinline__ void at_step(const char* kb, const char* vb, int koff
   }
   // a query with nothing unmasked so far keeps m_run = -inf; exp2(-inf - (-inf)) must not be evaluated
   const float neg_m = (m_run == -INFINITY) ? 0.f : -m_run;
-  at_fused<DO_QK, HAVE_PREV, KH, KT>(kb, vb, koff, voff, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, l_lane);
+  at_fused<DO_QK, HAVE_PREV, KQ, VB, KT>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, l_lane, mx_carry);
 }
 
 __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
@@ -497,6 +527,8 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
   }
   char* const kring = lds;
   char* const vring = lds + AT_RING * AT_KBUF_BYTES;
+  uint32_t* const blist = reinterpret_cast<uint32_t*>(lds + AT_RING * (AT_KBUF_BYTES + AT_VBUF_BYTES));
+  const int c_ragged = (n % AT_BS) != 0 ? nb - 1 : -1;  // the only block whose K rows may run past the sequence
 
   for (;;) {
     __syncthreads();  // previous item's LDS reads are done
@@ -522,12 +554,33 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     if (!at_item(gm, queue, ticket, h, pair)) continue;
     const int r0 = 2 * pair;
     const bool has_b = r0 + 1 < nb;
-    const int r = r0 + grp;             // this wave's row
+    const int r = r0 + grp;  // this wave's row
     const bool row_ok = grp == 0 || has_b;
     const int kvh = h / gm.group;
     const sp_bf16* kh = k + (int64_t)kvh * sk_h;
-    const sp_bf16* vth = vt + (int64_t)kvh * nb * AT_D * AT_BS;
+    const char* vth = reinterpret_cast<const char*>(vt + (int64_t)kvh * nb * AT_D * AT_BS);
     const uint64_t* mrow = mask + ((int64_t)h * nb + r0) * nbw;
+
+    // ---- the pair's block list: every column kept by either row, ascending, with membership flags ----
+    // All waves walk the (uniform) mask words and keep a running count; wave w compacts words w, w+8, ...
+    int n_blk = 0;
+    {
+      const int wmax = (has_b ? r0 + 1 : r0) >> 6;
+      const int lane = t & 63;
+      for (int wi = 0; wi <= wmax; ++wi) {
+        const uint64_t wa = at_trim(mrow[wi], wi, r0);
+        const uint64_t wb = has_b ? at_trim(mrow[nbw + wi], wi, r0 + 1) : 0ull;
+        const uint64_t wu = wa | wb;
+        if ((wi & 7) == wave && ((wu >> lane) & 1ull)) {
+          const int pos = n_blk + __builtin_popcountll(wu & ((1ull << lane) - 1ull));
+          blist[pos] = (uint32_t)(wi * 64 + lane) | (((wa >> lane) & 1ull) ? AT_IN_A : 0u) |
+                       (((wb >> lane) & 1ull) ? AT_IN_B : 0u);
+        }
+        n_blk += __builtin_popcountll(wu);
+      }
+      n_blk = __builtin_amdgcn_readfirstlane(n_blk);
+    }
+    __syncthreads();
 
     // Q^T operand: this lane's query, 8 k-steps of 8 channels
     bf16x8 qb[8];
@@ -546,109 +599,142 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     for (int dt = 0; dt < 4; ++dt) o[dt] = (floatx16){0};
     float m_run = -INFINITY, l_lane = 0.f;
 
-    // Two walks over the union of the pair's masks: `ld` runs three sub-tiles ahead and feeds the loads.
-    // Sub-tile u lives in ring slot u % 4.  Every step issues the same number of loads (the waits count
-    // instructions): K of sub-tile u+3 and V^T of sub-tile u+2 -- the sub-tile whose K went out one step earlier.
-    // Past the end the last sub-tile is fetched again into a slot nobody reads any more.
-    AtUnion ld, cp;
-    ld.init(mrow, mrow + nbw, r0, has_b);
-    cp = ld;
-    int lc = ld.next(), lhalf = 0;  // sub-tile whose K is loaded next
-    int vc = lc, vhalf = 0;         // sub-tile whose V^T is loaded next
-    auto advance = [&]() {
-      if (lhalf == 0) {
-        lhalf = 1;
-      } else {
-        const int nx = ld.next();
-        if (nx >= 0) {
-          lc = nx;
-          lhalf = 0;
-        }
-      }
+    // Block b of the list is processed as sub-tiles 2b and 2b+1; sub-tile s lives in ring slot s % 4 (K and V^T
+    // rings alike).  One wait + barrier + issue per BLOCK: while block b is computed on (K of sub-tiles 2b, 2b+1
+    // and V^T of 2b-1, 2b -- the P.V product trails by one sub-tile), K of 2b+2, 2b+3 and V^T of 2b+1, 2b+2 are
+    // in flight.  Past the end the last block is fetched again into slots nobody reads any more.
+    auto entry = [&](int b) -> uint32_t {
+      const int bc = b < n_blk ? b : n_blk - 1;
+      return __builtin_amdgcn_readfirstlane(blist[bc]);
     };
-    if (lc >= 0) {
-#pragma unroll
-      for (int i = 0; i < 3; ++i) {  // steps -3..-1: K(0..2), V^T(0 [unused copy], 0, 1)
-        at_issue_k(lo, kh, n, sk_n, lc, lhalf, kring + i * AT_KBUF_BYTES, wave, t);
-        at_issue_v(lo, vth, vc, vhalf, vring + ((i + 3) & 3) * AT_VBUF_BYTES, wave);
-        vc = lc;
-        vhalf = lhalf;
-        advance();
-      }
+    auto issue_k = [&](int c, int hf, int sub) {  // K of sub-tile `sub` = (column c, half hf)
+      char* kbuf = kring + (sub & 3) * AT_KBUF_BYTES;
+      const int64_t key0 = (int64_t)c * AT_BS + hf * AT_SUB;
+      if (c != c_ragged)
+        at_issue_k(lo, reinterpret_cast<const char*>(kh + key0 * sk_n), sk_n, kbuf, wave);
+      else
+        at_issue_k_tail(kh, n, sk_n, key0, kbuf, wave, t);
+    };
+    auto issue_v = [&](int c, int hf, int sub) {  // V^T of sub-tile `sub` = (column c, half hf)
+      at_issue_v(lo, vth + (int64_t)c * (AT_D * AT_BS * 2) + hf * (AT_SUB * 2), vring + (sub & 3) * AT_VBUF_BYTES,
+                 wave);
+    };
+    int c_cur = -1;
+    bool mine = false;
+    const uint32_t my_flag = grp ? AT_IN_B : AT_IN_A;
+    if (n_blk > 0) {
+      const uint32_t e0 = entry(0);
+      c_cur = (int)(e0 & AT_COL_MASK);
+      mine = (e0 & my_flag) != 0u;
+      issue_k(c_cur, 0, 0);
+      issue_k(c_cur, 1, 1);
+      issue_v(c_cur, 0, 0);
     }
 
-    // The compute walk.  Per sub-tile u every wave passes `top` exactly once (wait, barrier, issue), whatever its
-    // row does with the sub-tile.  A row's own sub-tiles come in runs; a run is one straight-line pipeline:
-    // start (first S), steady steps while the next sub-tile is the row's too, drain on the sub-tile after the run
-    // (V^T(u-1) is still resident while sub-tile u is current) or after the walk.
-    int u = 0;
-    int c_cur = cp.next(), half = 0;
-    bool mine = c_cur >= 0 && row_ok && cp.in_row(c_cur, grp);
-    const char *kb = kring, *vb = vring;
+    // The compute walk.  Per block every wave passes `top` exactly once (wait, barrier, issue), whatever its row
+    // does with the block.  A row's own blocks come in runs; a run is one straight-line pipeline: start (first S),
+    // steady steps while the next block is the row's too, drain on the block after the run (V^T of the run's last
+    // sub-tile is resident by then) or after the walk.
+    int b = 0;
+    const char *kb = kring, *vb = vring;  // K(2b), V^T(2b-1); the second sub-tile's buffers follow in the rings
+    const char* vb1 = vring;              // V^T(2b)
+    int c_next = 0;  // column of block b+1 (clamped to the last block)
+    AtAddr ad;
     auto top = [&]() {
-      AT_WAIT_VMCNT8();              // K(u) and V^T(u-1) have landed (own loads)
-      __builtin_amdgcn_s_barrier();  // ... everybody's; and every wave is past sub-tile u-1
-      // (hidden loop invariance: no precomputed copies of these lane constants that could be spilled -- a scratch
-      // reload would wait for the tile loads just issued)
+      AT_WAIT_VMCNT0();              // K(2b), K(2b+1), V^T(2b-1), V^T(2b) have landed (own loads)
+      __builtin_amdgcn_s_barrier();  // ... everybody's; and every wave is past block b-1
+      // (hidden loop invariance: no precomputed copies of these lane constants that could be spilled)
       asm volatile("" : "+v"(lo.k), "+v"(lo.v));
-      at_issue_k(lo, kh, n, sk_n, lc, lhalf, kring + ((u + 3) & 3) * AT_KBUF_BYTES, wave, t);
-      at_issue_v(lo, vth, vc, vhalf, vring + ((u + 2) & 3) * AT_VBUF_BYTES, wave);
-      vc = lc;
-      vhalf = lhalf;
-      advance();
-      kb = kring + (u & 3) * AT_KBUF_BYTES;
-      vb = vring + ((u + 3) & 3) * AT_VBUF_BYTES;  // V^T(u-1)
+      c_next = (int)(entry(b + 1) & AT_COL_MASK);
+      kb = kring + ((2 * b) & 3) * AT_KBUF_BYTES;
+      vb = vring + ((2 * b + 3) & 3) * AT_VBUF_BYTES;
+      vb1 = vring + ((2 * b) & 3) * AT_VBUF_BYTES;
       asm volatile("" : "+v"(koff), "+v"(voff));
+      at_block_addr(ad, kb, vb, vb1, koff, voff);
+    };
+    // The next block's loads go out in four parts spread over the block's steps: issued in one burst, the eight
+    // waves' 64 KiB would queue up in front of the CU's vector-memory path and stall everybody for its duration.
+    auto feed = [&](int part) {
+      if (part == 0) issue_k(c_next, 0, 2 * b + 2);
+      if (part == 1) issue_k(c_next, 1, 2 * b + 3);
+      if (part == 2) issue_v(c_cur, 1, 2 * b + 1);
+      if (part == 3) issue_v(c_next, 0, 2 * b + 2);
+    };
+    auto feed_all = [&]() {
+      feed(0);
+      feed(1);
+      feed(2);
+      feed(3);
     };
     auto step_walk = [&]() {
-      ++u;
-      if (half == 0) {
-        half = 1;
+      ++b;
+      if (b < n_blk) {
+        const uint32_t e = entry(b);
+        c_cur = (int)(e & AT_COL_MASK);
+        mine = (e & my_flag) != 0u;
       } else {
-        c_cur = cp.next();
-        half = 0;
-        mine = c_cur >= 0 && row_ok && cp.in_row(c_cur, grp);
+        c_cur = -1;
+        mine = false;
       }
     };
     bool finished = false;  // the final wait + barrier has been passed
     while (c_cur >= 0) {
       top();
       if (!mine) {
+        feed_all();
         step_walk();
         continue;
       }
       floatx16 sa, sb;
       bf16x8 pa[2], pb[2];
       // ---- start of a run: S of the first half-tile, nothing to overlap with yet ----
+      feed(0);
       at_qk_only<0>(kb, koff, qb, sa);
-      at_step<true, false, 1, 0>(kb, vb, koff, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, c_cur == r,
-                                 half * AT_SUB, tq);
-      int c_prev = c_cur, half_prev = half;
+      float mx_carry = at_lanemax(sa);
+      feed(1);
+      at_step<true, false, 1, 0, 0>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+                                    c_cur == r, 0, tq);
+      feed(2);
+      at_step<true, true, 2, 1, 0>(ad, vb1, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+                                   c_cur == r, 32, tq);
+      feed(3);
+      at_step<true, true, 3, 1, 1>(ad, vb1, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+                                   c_cur == r, AT_SUB, tq);
+      int c_prev = c_cur;
       step_walk();
-      // ---- steady state: sub-tile u supplies K, sub-tile u-1 supplies V^T ----
+      // ---- steady state: four half-tile steps per block ----
       while (mine) {  // (mine implies c_cur >= 0)
         top();
-        // S(u-1, keys 32..63) -> P;  S(u, keys 0..31) on the matrix core;  O += V^T(u-1, keys 0..31) . P
-        at_step<true, true, 0, 0>(kb, vb, koff, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, c_prev == r,
-                                  half_prev * AT_SUB + 32, tq);
-        at_step<true, true, 1, 1>(kb, vb, koff, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, c_cur == r,
-                                  half * AT_SUB, tq);
+        feed(0);
+        // S(previous block, keys 96..127) -> P;  S(keys 0..31) on the matrix core;  O += V^T(2b-1, keys 0..31) . P
+        at_step<true, true, 0, 0, 0>(ad, vb, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+                                     c_prev == r, AT_SUB + 32, tq);
+        feed(1);
+        at_step<true, true, 1, 0, 1>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+                                     c_cur == r, 0, tq);
+        feed(2);
+        at_step<true, true, 2, 1, 0>(ad, vb1, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+                                     c_cur == r, 32, tq);
+        feed(3);
+        at_step<true, true, 3, 1, 1>(ad, vb1, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+                                     c_cur == r, AT_SUB, tq);
         c_prev = c_cur;
-        half_prev = half;
         step_walk();
       }
-      // ---- drain: the run's last second half and its P.V ----
+      // ---- drain: the run's last half-tile and its P.V (V^T of sub-tile 2b-1) ----
       if (c_cur >= 0) {
         top();
+        feed_all();
         step_walk();
       } else {
         AT_WAIT_VMCNT0();
         __syncthreads();
         finished = true;
-        vb = vring + ((u + 3) & 3) * AT_VBUF_BYTES;
+        vb = vring + ((2 * b + 3) & 3) * AT_VBUF_BYTES;
+        at_block_addr(ad, kb, vb, vb, koff, voff);
       }
-      at_step<false, true, 0, 0>(kb, vb, koff, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, c_prev == r,
-                                 half_prev * AT_SUB + 32, tq);
+      at_step<false, true, 0, 0, 0>(ad, vb, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+                                    c_prev == r, AT_SUB + 32, tq);
       at_pv_only<1>(vb, voff, pb, o);
     }
     if (!finished) {
@@ -824,6 +910,9 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
              "sp_block_sparse_attn_fwd_bf16: workspace too small");
   const int64_t nb = sp_ceil_div(n, bs);
   SP_REQUIRE(nb * hq < (1ll << 31), SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: grid too large");
+  SP_REQUIRE(nb <= AT_LIST_MAX, SP_ERR_UNSUPPORTED,
+             "sp_block_sparse_attn_fwd_bf16: %lld key blocks exceed the supported %d (sequence too long)", (long long)nb,
+             AT_LIST_MAX);
   if (!(flags & SP_ATTN_V_REPACKED)) {
     int rc = sp_attn_repack_v_bf16(v, n, hkv, d, v_stride_n, v_stride_h, bs, workspace, workspace_bytes, stream);
     if (rc != SP_OK) return rc;
