@@ -274,7 +274,8 @@ def main():
         "roofline": {"bound": "mfma", "kernel": "sp_attn_fwd_kernel", "achieved": round(attn_tflops, 1),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
                      "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms),
-                     "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get((args.workload, pt))},
+                     "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get((args.workload, pt)),
+                     "sclk_mhz": round(ops.attention_clock_mhz(w.seq_len, w.hkv, w.head_dim, w.block_size, dev))},
     }
 
     if not args.no_extras:
@@ -315,6 +316,10 @@ def main():
         line["dense_causal_baseline"] = {"ms": round(dms, 3), "blocks": tri,
                                          "tflops": round(tri * FLOP_PER_BLOCK / dms / 1e9, 1),
                                          "frac": round(tri * FLOP_PER_BLOCK / dms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+        # what back-to-back MFMAs alone sustain on this chip (power-managed clocks): the practical ceiling
+        line["mfma_sustained_tflops"] = {"random_operands": round(ops.mfma_probe_tflops(True), 1),
+                                         "constant_operands": round(ops.mfma_probe_tflops(False), 1),
+                                         "nominal_peak": PEAK_BF16_TFLOPS}
         if args.sweep:
             sweep = []
             for thr in (0.9, 0.95, 0.99):

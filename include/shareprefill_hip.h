@@ -71,6 +71,12 @@ typedef struct sp_cluster_state {
 int sp_version(void);
 const char* sp_arch(void);       /* "gfx950" */
 const char* sp_last_error(void); /* host string, valid until the next failing call on this thread */
+/* Measurement aid (no counterpart in the reference): runs `iters` x 4 back-to-back bf16 32x32x16 MFMAs per wave on
+ * every CU (8 waves per CU) with either random-valued (random_operands != 0) or constant operand registers.  The
+ * caller times it; flops = sp_diag_mfma_flops(iters).  Used to calibrate the sustained matrix-core rate, which
+ * depends on how much the operand bits toggle.  out: 512 floats of device scratch. */
+int sp_diag_mfma_bf16(int32_t iters, int32_t random_operands, float* out, sp_stream_t stream);
+double sp_diag_mfma_flops(int32_t iters);
 
 /* ---- (a) block average pooling --------------------------------------------------------------
  * Replaces triton_bnhd_pool / bnhd_pool_kernel (attn/utils.py:131-261, "avg" mode) and the torch
@@ -165,6 +171,12 @@ int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec,
  * SP_ATTN_V_REPACKED (the caller already repacked this v into this workspace). */
 #define SP_ATTN_V_REPACKED 1u
 size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs);
+/* Measurement aid (no counterpart in the reference): shader-clock cycles and 100 MHz wall ticks that workgroup 0
+ * of the LAST sp_block_sparse_attn_fwd_bf16 launch on this workspace spent in the kernel; cycles / (ticks / 100)
+ * is the average shader clock in MHz under that load.  Copies two int64 to host memory after synchronising the
+ * stream. */
+int sp_attn_last_launch_clocks(const void* workspace, int64_t n, int32_t hkv, int32_t d, int32_t bs,
+                               int64_t* cycles_and_ticks, sp_stream_t stream);
 int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n, int64_t v_stride_h,
                           int32_t bs, void* workspace, size_t workspace_bytes, sp_stream_t stream);
 int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,

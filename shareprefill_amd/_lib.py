@@ -37,6 +37,8 @@ SIGNATURES = {
     "sp_version": (_I32, []),
     "sp_arch": (C.c_char_p, []),
     "sp_last_error": (C.c_char_p, []),
+    "sp_diag_mfma_bf16": (_I32, [_I32, _I32, _P, _P]),
+    "sp_diag_mfma_flops": (_D, [_I32]),
     "sp_pool_avg_bf16": (_I32, [_P, _P, _I64, _I32, _I32, _I64, _I64, _I32, _I32, _P, _P]),
     "sp_lastq_scores_workspace_bytes": (_SZ, [_I64, _I32, _I32]),
     "sp_lastq_scores_bf16": (_I32, [_P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I32, _U32, _P, _SZ,
@@ -51,6 +53,7 @@ SIGNATURES = {
     "sp_cover_select_workspace_bytes": (_SZ, [_I32]),
     "sp_cover_select_global": (_I32, [_P, _P, _I32, _I32, _F, _P, _P, _SZ, _P]),
     "sp_attn_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _I32]),
+    "sp_attn_last_launch_clocks": (_I32, [_P, _I64, _I32, _I32, _I32, _P, _P]),
     "sp_attn_repack_v_bf16": (_I32, [_P, _I64, _I32, _I32, _I64, _I64, _I32, _P, _SZ, _P]),
     "sp_block_sparse_attn_fwd_bf16": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I64, _I64,
                                              _I32, _F, _P, _P, _P, _P, _P, _SZ, _U32, _P]),

@@ -83,6 +83,7 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 // other queues.  Pulling is by atomic tickets only: nobody ever waits for anybody, and every workgroup leaves
 // once all eight queues are exhausted.
 #define AT_GANG 32
+#define AT_CLOCK_SLOT 192  // int index inside the 1 KiB scheduler area: {shader cycles, 100 MHz ticks} of workgroup 0
 #define AT_FWD_THREADS 512
 
 struct AtGeom {
@@ -497,6 +498,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // K ring (4 x 16 KiB) | V^T ring (4 x 16 KiB)
   __shared__ int s_queue, s_ticket;
 
+  const long long clk0 = clock64(), tick0 = wall_clock64();  // see sp_attn_last_launch_clocks
   AtGeom gm;
   gm.group = hq / hkv;
   gm.n_pairs = (nb + 1) / 2;
@@ -548,7 +550,14 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     }
     __syncthreads();
     const int queue = __builtin_amdgcn_readfirstlane(s_queue);
-    if (queue < 0) break;
+    if (queue < 0) {
+      if (blockIdx.x == 0 && t == 0) {
+        long long* clk = reinterpret_cast<long long*>(sched + AT_CLOCK_SLOT);
+        clk[0] = clock64() - clk0;
+        clk[1] = wall_clock64() - tick0;
+      }
+      break;
+    }
     const int ticket = __builtin_amdgcn_readfirstlane(s_ticket);
     int h, pair;
     if (!at_item(gm, queue, ticket, h, pair)) continue;
@@ -865,6 +874,16 @@ static size_t at_vt_bytes(int64_t n, int32_t hkv, int32_t d, int32_t bs) {
 extern "C" size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs) {
   if (n <= 0 || hq <= 0 || hkv <= 0 || d <= 0 || bs <= 0) return 0;
   return at_vt_bytes(n, hkv, d, bs) + 1024 + (size_t)hq * (size_t)n * sizeof(float2);
+}
+
+extern "C" int sp_attn_last_launch_clocks(const void* workspace, int64_t n, int32_t hkv, int32_t d, int32_t bs,
+                                          int64_t* cycles_and_ticks, sp_stream_t stream) {
+  SP_REQUIRE(workspace && cycles_and_ticks && n > 0 && hkv > 0 && d > 0 && bs > 0, SP_ERR_INVALID_ARGUMENT,
+             "sp_attn_last_launch_clocks: bad arguments");
+  SP_HIP(hipStreamSynchronize((hipStream_t)stream));
+  SP_HIP(hipMemcpy(cycles_and_ticks, (const char*)workspace + at_vt_bytes(n, hkv, d, bs) + AT_CLOCK_SLOT * sizeof(int),
+                   2 * sizeof(int64_t), hipMemcpyDeviceToHost));
+  return SP_OK;
 }
 
 extern "C" int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n,

@@ -254,6 +254,36 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
     return out
 
 
+def attention_clock_mhz(n: int, hkv: int, d: int, block_size: int, device) -> float:
+    """Average shader clock (MHz) seen by workgroup 0 of the last block_sparse_attention launch on this device
+    (measurement aid; synchronises the current stream)."""
+    import ctypes
+    lib = _lib.load()
+    ws = _workspaces.get(("attn_vt", str(device)))
+    if ws is None:
+        raise RuntimeError("no attention launch on this device yet")
+    buf = (ctypes.c_int64 * 2)()
+    st = lib.sp_attn_last_launch_clocks(_ptr(ws), n, hkv, d, block_size, ctypes.cast(buf, ctypes.c_void_p), _stream())
+    _lib.check(st, "sp_attn_last_launch_clocks")
+    return float(buf[0]) / (float(buf[1]) / 100.0) if buf[1] > 0 else float("nan")
+
+
+def mfma_probe_tflops(random_operands: bool, iters: int = 1500000, reps: int = 2) -> float:
+    """Sustained bf16 MFMA rate of back-to-back 32x32x16 MFMAs on every CU (measurement aid).  The default runs
+    about 0.2 s per repetition, long enough for the clocks to settle under the load; the last repetition counts."""
+    lib = _lib.load()
+    out = torch.empty(512, dtype=torch.float32, device="cuda")
+    ms = 0.0
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(torch.cuda.current_stream())
+        _lib.check(lib.sp_diag_mfma_bf16(iters, 1 if random_operands else 0, _ptr(out), _stream()), "sp_diag_mfma_bf16")
+        b.record(torch.cuda.current_stream())
+        b.synchronize()
+        ms = a.elapsed_time(b)
+    return lib.sp_diag_mfma_flops(iters) / (ms * 1e-3) / 1e12
+
+
 class KernelTimer:
     """Brackets kernel launches with events on the stream they are launched on (torch's current stream).
     Set ops.kernel_timer to an instance to collect; durations are read after a synchronise."""
