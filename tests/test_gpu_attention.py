@@ -57,6 +57,47 @@ def test_block_sparse_attention_matches_oracle(gpu_device, hq, hkv, n):
     _check(out.transpose(0, 1), ref)
 
 
+def test_row_pairs_with_unequal_masks(gpu_device):
+    """The kernel walks the union of two adjacent rows' masks: rows that share runs of blocks, rows that share
+    nothing but the sink column, a row with only its diagonal block next to a dense one, an odd row count."""
+    from shareprefill_amd import ops
+
+    hq, hkv, n = 3, 1, 6144 + 128  # nb = 49: the last row has no partner
+    nb = n // 128
+    q, k, v = _qkv(hq, hkv, n, 77)
+    m = np.zeros((hq, nb, nb), dtype=bool)
+    r = np.arange(nb)
+    # head 0: vertical-slash (sink, two verticals, a band of three diagonals)
+    for d in (0, 1, 2, 9):
+        m[0, r[d:], r[d:] - d] = True
+    m[0, :, 0] = m[0, 7:, 7] = m[0, 20:, 20] = True
+    # head 1: even rows dense, odd rows diagonal only
+    m[1] = np.tril(np.ones((nb, nb), dtype=bool))
+    m[1, 1::2] = False
+    m[1, r, r] = True
+    # head 2: even rows keep even columns, odd rows odd columns (plus the diagonal)
+    m[2] = np.tril((r[:, None] + r[None, :]) % 2 == 0)
+    m[2, r, r] = True
+    m = np.tril(m)
+    scale = 1.0 / math.sqrt(128)
+    ref, _ = O.masked_attention(q, k, v, m, 128, scale)
+    mg = ops.bool_to_mask(torch.from_numpy(m)).to(gpu_device)
+    out = ops.block_sparse_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), mg, 128, scale).cpu()
+    _check(out.transpose(0, 1), ref)
+
+
+def test_measurement_aids(gpu_device):
+    from shareprefill_amd import ops
+
+    q, k, v = _qkv(2, 1, 1024, 5)
+    mg = ops.bool_to_mask(torch.tril(torch.ones(8, 8, dtype=torch.bool)).expand(2, 8, 8).contiguous()).to(gpu_device)
+    ops.block_sparse_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), mg, 128, 0.1)
+    mhz = ops.attention_clock_mhz(1024, 1, 128, 128, gpu_device)
+    assert 300.0 < mhz < 4000.0
+    rate = ops.mfma_probe_tflops(True, iters=20000, reps=1)
+    assert 100.0 < rate < 2600.0
+
+
 def test_full_mask_equals_sdpa_and_avg_map(gpu_device):
     from shareprefill_amd import ops
 
