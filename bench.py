@@ -113,6 +113,24 @@ def cpu_baseline(w, q, k, v, mask_bool, decision, kept_blocks, pt):
 MEASURED_ATTN_TRAFFIC_BYTES = {("C3", 0.95): int((105.1 + 1.0) * 2 ** 30)}
 
 
+def library_gemm_tflops(dev, n=8192, reps=10):
+    """bf16 GEMM rate of the vendor library (torch.matmul) on N(0,1) data: what a tuned dense kernel sustains on
+    this chip with operands that toggle -- a calibration point beside the nominal peak, nothing the path uses."""
+    import torch
+
+    g = torch.Generator(device=dev).manual_seed(1)
+    a = torch.randn(n, n, device=dev, dtype=torch.bfloat16, generator=g)
+    b = torch.randn(n, n, device=dev, dtype=torch.bfloat16, generator=g)
+    for _ in range(3):
+        a @ b
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        a @ b
+    torch.cuda.synchronize()
+    return 2.0 * n ** 3 * reps / (time.perf_counter() - t0) / 1e12
+
+
 def run_c4(args):
     """TTFT of the full Llama-3.1-8B architecture (random-init bf16, 32 layers, hidden 4096, Hq32 Hkv8, RoPE theta
     5e5, vocab 128256) on uniform-random token ids, SharePrefill patched into every layer with the shipped
@@ -319,6 +337,7 @@ def main():
         # what back-to-back MFMAs alone sustain on this chip (power-managed clocks): the practical ceiling
         line["mfma_sustained_tflops"] = {"random_operands": round(ops.mfma_probe_tflops(True), 1),
                                          "constant_operands": round(ops.mfma_probe_tflops(False), 1),
+                                         "library_gemm_8192_random_data": round(library_gemm_tflops(dev), 1),
                                          "nominal_peak": PEAK_BF16_TFLOPS}
         if args.sweep:
             sweep = []
