@@ -27,8 +27,8 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define LQ_PITCH 136         // LDS row pitch (floats) of the probability tile
 
 // lane's A operand: scaled last-block queries, 8 k-steps x 8 bf16
-__device__ static inline void lq_load_q(const sp_bf16* __restrict__ q, int64_t n, int64_t sq_n, int wave, int lane,
-                                        float inv_sqrt_d, bf16x8 qa[8]) {
+__device__ static __forceinline__ void lq_load_q(const sp_bf16* __restrict__ q, int64_t n, int64_t sq_n, int wave, int lane,
+                                        float inv_sqrt_d, bf16x8 (&qa)[8]) {
   const int row = wave * 32 + (lane & 31);
   const sp_bf16* src = q + (n - LQ_ROWS + row) * sq_n + 8 * (lane >> 5);
 #pragma unroll
@@ -47,31 +47,93 @@ __device__ static inline void lq_load_q(const sp_bf16* __restrict__ q, int64_t n
   }
 }
 
-// logits of this wave's 32 query rows against the 128 keys of tile `kb`:
+// ---- K tile staging: 128 keys x 128 channels bf16 through LDS (row pitch 272 bytes), coalesced ---------------
+#define LQ_KPITCH 136  // bf16 elements per LDS row of the K tile
+
+typedef uint32_t lq_u32x4 __attribute__((ext_vector_type(4)));
+struct LqKRegs {
+  lq_u32x4 v[8];
+};
+
+// thread t fetches chunk t%16 (16 bytes) of key rows t/16, t/16+16, ...; keys past the end are clamped (masked later)
+__device__ static __forceinline__ void lq_fetch_k(const sp_bf16* __restrict__ k, int64_t n, int64_t sk_n, int64_t kb, int t,
+                                         LqKRegs& kr) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    int64_t key = kb + i * 16 + (t >> 4);
+    if (key > n - 1) key = n - 1;
+    kr.v[i] = *reinterpret_cast<const lq_u32x4*>(k + key * sk_n + (t & 15) * 8);
+  }
+}
+
+__device__ static __forceinline__ void lq_store_k(sp_bf16* Ks, int t, const LqKRegs& kr) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    *reinterpret_cast<lq_u32x4*>(Ks + (i * 16 + (t >> 4)) * LQ_KPITCH + (t & 15) * 8) = kr.v[i];
+}
+
+// logits of this wave's 32 query rows against the 128 keys of the staged tile:
 // acc[nt][r] = S[row 32w + 8(r/4) + 4(lane/32) + r%4][key kb + 32nt + lane%32]
-__device__ static inline void lq_tile_logits(const sp_bf16* __restrict__ k, int64_t n, int64_t sk_n, int64_t kb,
-                                             int lane, const bf16x8 qa[8], floatx16 acc[4]) {
+__device__ static __forceinline__ void lq_tile_logits(const sp_bf16* Ks, int lane, const bf16x8 (&qa)[8], floatx16 (&acc)[4]) {
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
-    int64_t key = kb + 32 * nt + (lane & 31);
-    if (key > n - 1) key = n - 1;  // out-of-range keys are masked by the caller
-    const sp_bf16* src = k + key * sk_n + 8 * (lane >> 5);
+    const sp_bf16* src = Ks + (32 * nt + (lane & 31)) * LQ_KPITCH + 8 * (lane >> 5);
     floatx16 c = {0};
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      uint4 raw = *reinterpret_cast<const uint4*>(src + 16 * ks);
+      const uint4 raw = *reinterpret_cast<const uint4*>(src + 16 * ks);
       c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[ks], __builtin_bit_cast(bf16x8, raw), c, 0, 0, 0);
     }
     acc[nt] = c;
   }
 }
 
-__device__ static inline int lq_row_of(int wave, int lane, int r) {
+__device__ static __forceinline__ int lq_row_of(int wave, int lane, int r) {
   return wave * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
 }
 
+typedef float lq_floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 lq_bf16x2 __attribute__((ext_vector_type(2)));
+
+// Rounds the logits to bf16 (the reference's qk tensor is bf16, attention_sharing.py:129-139) with the hardware
+// round-to-nearest-even conversion, two at a time, and masks what the last query block must not see.  Only the
+// tiles that reach into the last 128 tokens (or past the sequence end) need the mask: MASKED is tile-uniform.
+template <bool MASKED>
+__device__ static __forceinline__ void lq_finish_logits(floatx16 (&acc)[4], uint32_t flags, int64_t kb, int64_t n, int wave,
+                                               int lane) {
+  if (flags & SP_FLAG_LOGITS_BF16) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        lq_floatx2 f;
+        f[0] = acc[nt][r];
+        f[1] = acc[nt][r + 1];
+        const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, lq_bf16x2));
+        acc[nt][r] = __uint_as_float(pk << 16);
+        acc[nt][r + 1] = __uint_as_float(pk & 0xffff0000u);
+      }
+  }
+  if (MASKED) {
+    // key <= query position  <=>  c - row <= (n - 128) - kb;  key < n  <=>  c < n - kb   (c, row: offsets in the tile)
+    const int64_t d64 = (n - LQ_ROWS) - kb, e64 = n - kb;
+    const int dlim = d64 > 1024 ? 1024 : (int)d64, elim = e64 > 1024 ? 1024 : (int)e64;
+    int ln = lane;
+    asm volatile("" : "+v"(ln));  // keeps this rare path's lane arithmetic out of the tile loop's registers
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = lq_row_of(wave, ln, r);
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int c = 32 * nt + (ln & 31);
+        if (!(c - row <= dlim && c < elim)) acc[nt][r] = -INFINITY;
+      }
+    }
+  }
+}
+
 // ---- kernel 1: chunk partials of the row max / row sum ------------------------------------------
-__global__ __launch_bounds__(LQ_THREADS) void sp_lastq_stats_kernel(
+__global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_stats_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
     int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, int n_chunks,
     float2* __restrict__ partial /* [hq][n_chunks][128] */) {
@@ -89,32 +151,33 @@ __global__ __launch_bounds__(LQ_THREADS) void sp_lastq_stats_kernel(
     m[r] = -INFINITY;
     l[r] = 0.f;
   }
+  __shared__ sp_bf16 Ks[LQ_TILE * LQ_KPITCH];
   const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
+  const int64_t tile0 = (int64_t)chunk * LQ_STAT_TILES;
+  LqKRegs kr;
+  if (tile0 < n_tiles) lq_fetch_k(kh, n, sk_n, tile0 * LQ_TILE, threadIdx.x, kr);
   for (int t = 0; t < LQ_STAT_TILES; ++t) {
-    const int64_t tile = (int64_t)chunk * LQ_STAT_TILES + t;
+    const int64_t tile = tile0 + t;
     if (tile >= n_tiles) break;
     const int64_t kb = tile * LQ_TILE;
+    __syncthreads();  // the previous tile's operand reads are done
+    lq_store_k(Ks, threadIdx.x, kr);
+    __syncthreads();
+    if (t + 1 < LQ_STAT_TILES && tile + 1 < n_tiles) lq_fetch_k(kh, n, sk_n, kb + LQ_TILE, threadIdx.x, kr);
     floatx16 acc[4];
-    lq_tile_logits(kh, n, sk_n, kb, lane, qa, acc);
+    lq_tile_logits(Ks, lane, qa, acc);
+    if (kb + LQ_TILE <= n - LQ_ROWS)
+      lq_finish_logits<false>(acc, flags, kb, n, wave, lane);
+    else
+      lq_finish_logits<true>(acc, flags, kb, n, wave, lane);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int64_t qpos = n - LQ_ROWS + lq_row_of(wave, lane, r);
-      float s[4];
-      float tmax = -INFINITY;
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        const int64_t key = kb + 32 * nt + (lane & 31);
-        float v = acc[nt][r];
-        if (flags & SP_FLAG_LOGITS_BF16) v = sp_round_bf16(v);
-        v = (key <= qpos && key < n) ? v : -INFINITY;
-        s[nt] = v;
-        tmax = fmaxf(tmax, v);
-      }
+      const float tmax = fmaxf(fmaxf(acc[0][r], acc[1][r]), fmaxf(acc[2][r], acc[3][r]));
       if (tmax > -INFINITY) {
         const float mn = fmaxf(m[r], tmax);
         float add = 0.f;
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt) add += __expf(s[nt] - mn);
+        for (int nt = 0; nt < 4; ++nt) add += __expf(acc[nt][r] - mn);
         l[r] = l[r] * __expf(m[r] - mn) + add;
         m[r] = mn;
       }
@@ -156,7 +219,7 @@ __global__ __launch_bounds__(LQ_ROWS) void sp_lastq_combine_kernel(const float2*
 }
 
 // ---- kernel 3: probabilities -> vertical / slash ------------------------------------------------------
-__global__ __launch_bounds__(LQ_THREADS) void sp_lastq_probs_kernel(
+__global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
     int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, const float2* __restrict__ rowstat,
     float* __restrict__ vert_tok, float* __restrict__ slash_tok, float* __restrict__ vert_blk,
@@ -183,24 +246,30 @@ __global__ __launch_bounds__(LQ_THREADS) void sp_lastq_probs_kernel(
   float carry = 0.f;  // upper anti-diagonal part handed from the previous tile to bin (u) of this one
   const int u = threadIdx.x & 127;
 
-  for (int64_t tile = first - 1; tile < first + LQ_PROB_TILES && tile < n_tiles; ++tile) {
-    if (tile < 0) continue;
+  // the K tile is staged in the same LDS region the probability tile is written to afterwards
+  sp_bf16* Ks = reinterpret_cast<sp_bf16*>(lds);
+  const int64_t t_begin = first > 0 ? first - 1 : 0;
+  const int64_t t_end = first + LQ_PROB_TILES < n_tiles ? first + LQ_PROB_TILES : n_tiles;
+  LqKRegs kr;
+  if (t_begin < t_end) lq_fetch_k(kh, n, sk_n, t_begin * LQ_TILE, threadIdx.x, kr);
+  for (int64_t tile = t_begin; tile < t_end; ++tile) {
     const int64_t kb = tile * LQ_TILE;
+    lq_store_k(Ks, threadIdx.x, kr);  // (the previous iteration ended with a barrier)
+    __syncthreads();
+    if (tile + 1 < t_end) lq_fetch_k(kh, n, sk_n, kb + LQ_TILE, threadIdx.x, kr);
     floatx16 acc[4];
-    lq_tile_logits(kh, n, sk_n, kb, lane, qa, acc);
+    lq_tile_logits(Ks, lane, qa, acc);
+    __syncthreads();  // every wave has its logits: the K tile may be overwritten by P
+    if (kb + LQ_TILE <= n - LQ_ROWS)
+      lq_finish_logits<false>(acc, flags, kb, n, wave, lane);
+    else
+      lq_finish_logits<true>(acc, flags, kb, n, wave, lane);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int row = lq_row_of(wave, lane, r);
-      const int64_t qpos = n - LQ_ROWS + row;
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        const int c = 32 * nt + (lane & 31);
-        const int64_t key = kb + c;
-        float v = acc[nt][r];
-        if (flags & SP_FLAG_LOGITS_BF16) v = sp_round_bf16(v);
-        const float p = (key <= qpos && key < n) ? __expf(v - rm[r]) * rinv[r] : 0.f;
-        P[row * LQ_PITCH + c] = p;
-      }
+      for (int nt = 0; nt < 4; ++nt)  // exp(-inf) = 0 for the masked entries
+        P[row * LQ_PITCH + 32 * nt + (lane & 31)] = __expf(acc[nt][r] - rm[r]) * rinv[r];
     }
     __syncthreads();
     const bool emit = tile >= first;
