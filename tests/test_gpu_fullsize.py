@@ -1,0 +1,154 @@
+"""GPU checks at the full benchmark size (C3: B1 Hq32 Hkv8 D128 N131072, nb 1024), where the CPU oracle cannot
+run the whole layer: size-independent properties of every stage, plus exact-tolerance spot checks of single
+query blocks against a plain fp32 torch computation of the same rows.
+
+Properties used: softmax mass conservation of the last-query scores (vertical and slash vectors each sum to 1),
+block sums equal to sums of tokens, budget bounds and monotonicity, masks lower-triangular with sink column and
+diagonal kept, row pointers equal to popcounts, the id-list view round-tripping to the mask, rows of a pivot's
+block-average map summing to 1, linearity of attention in V, run-to-run bit reproducibility.
+"""
+
+import math
+import types
+
+import pytest
+import torch
+
+from shareprefill_amd import synthetic
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_REL = 2e-2, 2.5e-3  # see tests/test_gpu_attention.py for the mean-rel floor of a bf16 result
+
+
+@pytest.fixture(scope="module")
+def c3(gpu_device, tmp_path_factory):
+    from shareprefill_amd import AttentionSharing, shareprefill_attention_forward
+
+    w = synthetic.WORKLOADS["C3"]
+    q, k, v = synthetic.workload_inputs(w, device=gpu_device)
+    table = synthetic.random_cluster_table(w.hq, w.n_clusters, 2, w.seed)
+    path = synthetic.write_cluster_table(table, str(tmp_path_factory.mktemp("c3") / "table.json"))
+    sharing = AttentionSharing(path)
+    cfg = types.SimpleNamespace(block_size=128, min_budget=w.min_budget, max_budget=None,
+                                pattern_threshold=w.pattern_threshold, similarity_threshold=w.similarity_threshold,
+                                fallback_threshold=w.fallback_threshold, queryaware_threshold=w.queryaware_threshold)
+    outs, plans, avgs = [], [], []
+    for layer in (0, 1):
+        mod = types.SimpleNamespace(config=cfg, attention_sharing=sharing, layer_idx=layer, scaling=128 ** -0.5)
+        out, avg = shareprefill_attention_forward(mod, q, k, v, None, scaling=128 ** -0.5)
+        outs.append(out)
+        avgs.append(avg)
+        plans.append(sharing.plans[-1])
+    torch.cuda.synchronize()
+    return types.SimpleNamespace(w=w, q=q, k=k, v=v, outs=outs, plans=plans, avgs=avgs, nb=w.seq_len // 128)
+
+
+def test_scores_conserve_mass_and_block_sums(c3):
+    from shareprefill_amd import ops
+
+    vt, st, vb, sb = ops.lastq_scores(c3.q[0], c3.k[0], 128)
+    ones = torch.ones(c3.w.hq, dtype=torch.float64, device=vt.device)
+    assert torch.allclose(vt.double().sum(1), ones, atol=2e-4)
+    assert torch.allclose(st.double().sum(1), ones, atol=2e-4)
+    assert torch.allclose(vt.view(c3.w.hq, c3.nb, 128).sum(2), vb, rtol=1e-4, atol=1e-7)
+    assert torch.allclose(st.view(c3.w.hq, c3.nb, 128).sum(2), sb, rtol=1e-4, atol=1e-7)
+    assert (vt >= 0).all() and (st >= 0).all()
+    # same call again: bit-identical (every sum runs in a fixed order)
+    vt2, st2, vb2, sb2 = ops.lastq_scores(c3.q[0], c3.k[0], 128)
+    assert torch.equal(vt, vt2) and torch.equal(st, st2) and torch.equal(vb, vb2) and torch.equal(sb, sb2)
+    # budgets: within [min_budget blocks, nb], monotone in the threshold
+    prev = None
+    for thr in (0.5, 0.9, 0.95, 0.99):
+        nv, ns = ops.cover_budgets(vt, st, 128, thr, 8, c3.nb)
+        assert int(nv.min()) >= 8 and int(nv.max()) <= c3.nb and int(ns.min()) >= 8 and int(ns.max()) <= c3.nb
+        if prev is not None:
+            assert (nv >= prev[0]).all() and (ns >= prev[1]).all()
+        prev = (nv, ns)
+
+
+def test_masks_are_causal_keep_sink_and_diagonal_and_match_their_views(c3):
+    from shareprefill_amd import ops
+
+    nb = c3.nb
+    for plan in c3.plans:
+        mb = ops.mask_to_bool(plan.mask, nb)
+        assert not torch.triu(mb, diagonal=1).any()
+        idx = torch.arange(nb, device=mb.device)
+        vs_or_dense = (plan.decision == 0) | (plan.decision == 1) | (plan.decision == 2)
+        assert mb[vs_or_dense][:, :, 0].all()
+        assert mb[vs_or_dense][:, idx, idx].all()
+        assert mb[:, 0, 0].all()
+        ptr = ops.mask_row_pointers(plan.mask)
+        assert torch.equal(ptr[:, 1:] - ptr[:, :-1], mb.sum(2).to(ptr.dtype))
+        assert torch.equal(ops.bool_to_mask(mb), plan.mask)
+        ids = plan.block_idx()[0]
+        for h in (0, c3.w.hq - 1):
+            flat = torch.zeros(nb * nb, dtype=torch.bool, device=mb.device)
+            flat[ids[h].long()] = True
+            assert torch.equal(flat.view(nb, nb), mb[h])
+    dense = c3.plans[0].decision == 1
+    assert int(dense.sum()) == c3.w.n_clusters  # one pivot per shared cluster in layer 0
+    tri = torch.tril(torch.ones(nb, nb, dtype=torch.bool, device=dense.device))
+    assert (ops.mask_to_bool(c3.plans[0].mask, nb)[dense] == tri).all()
+
+
+def test_pivot_average_maps_are_row_stochastic(c3):
+    avg = c3.avgs[0][0]
+    dense = c3.plans[0].decision == 1
+    rows = avg[dense].double().sum(-1)
+    assert torch.allclose(rows, torch.ones_like(rows), atol=5e-3)
+    assert (avg[~dense] == 0).all()
+    assert not torch.triu(avg[dense], diagonal=1).any()
+
+
+def _rows_reference(q, k, v, mask_row, h, r, hkv_group, scale):
+    """fp32 masked attention of query block r of head h against all keys (plain torch on the GPU)."""
+    n = q.shape[2]
+    qs = q[0, h, r * 128:(r + 1) * 128].float()
+    kf, vf = k[0, h // hkv_group].float(), v[0, h // hkv_group].float()
+    s = (qs @ kf.t()) * scale
+    keep = mask_row.repeat_interleave(128)[:n]
+    qpos = torch.arange(r * 128, (r + 1) * 128, device=q.device)[:, None]
+    kpos = torch.arange(n, device=q.device)[None, :]
+    s = s.masked_fill(~(keep[None, :] & (kpos <= qpos)), float("-inf"))
+    return torch.softmax(s, dim=-1) @ vf
+
+
+def test_attention_rows_match_fp32_reference_at_full_size(c3):
+    from shareprefill_amd import ops
+
+    w, nb = c3.w, c3.nb
+    scale = 1.0 / math.sqrt(128)
+    for layer in (0, 1):
+        mb = ops.mask_to_bool(c3.plans[layer].mask, nb)
+        out = c3.outs[layer][0]  # [N, Hq, D]
+        for h, r in ((0, nb - 1), (5, nb - 2), (w.hq - 1, 511), (17, 640), (9, 0), (30, 1)):
+            ref = _rows_reference(c3.q, c3.k, c3.v, mb[h, r], h, r, w.hq // w.hkv, scale)
+            got = out[r * 128:(r + 1) * 128, h].float()
+            assert (got - ref).abs().max().item() <= MAX_ABS
+            assert ((got - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL
+
+
+def test_attention_is_linear_in_v_and_reproducible(c3):
+    from shareprefill_amd import ops
+
+    w = c3.w
+    mask = c3.plans[1].mask
+    scale = 1.0 / math.sqrt(128)
+    g = torch.Generator(device=c3.v.device).manual_seed(7)
+    v2 = torch.randn(c3.v.shape, device=c3.v.device, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    v2 = v2.transpose(1, 2).contiguous().transpose(1, 2)  # token-major storage like the workload's tensors
+    o1 = ops.block_sparse_attention(c3.q[0], c3.k[0], c3.v[0], mask, 128, scale)
+    o1b = ops.block_sparse_attention(c3.q[0], c3.k[0], c3.v[0], mask, 128, scale)
+    assert torch.equal(o1, o1b)
+    o2 = ops.block_sparse_attention(c3.q[0], c3.k[0], v2[0], mask, 128, scale)
+    vsum = (c3.v.float() + v2.float()).to(torch.bfloat16)
+    o12 = ops.block_sparse_attention(c3.q[0], c3.k[0], vsum[0], mask, 128, scale)
+    lhs, rhs = o12.float(), o1.float() + o2.float()
+    # bf16 roundings of the outputs (2^-9 of their magnitude) plus those of v1+v2 and of the probabilities inside
+    # the three products (2^-9 of sum p|v|, |v| up to ~5 -- not of the possibly cancelling result)
+    scale_of = o1.float().abs() + o2.float().abs() + lhs.abs()
+    assert ((lhs - rhs).abs() <= 2.0 ** -7 * scale_of + 5e-2).all()
+    assert ((lhs - rhs).abs().mean() / rhs.abs().mean()).item() <= 1e-2
+    assert torch.equal(o1, c3.outs[1][0])  # the layer call produced exactly this
