@@ -40,6 +40,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the stage breakdown / dense baseline / sweep")
     ap.add_argument("--sweep", action="store_true", help="also time pattern_threshold 0.9 and 0.99")
+    ap.add_argument("--length-sweep", default=None,
+                    help="C4 only: comma-separated prompt lengths; adds TTFT per length for the SharePrefill path and for "
+                         "the model's stock causal attention (torch SDPA), the protocol of eval/efficiency/latency.py")
     return ap.parse_args()
 
 
@@ -181,6 +184,32 @@ def run_c4(args):
                                    "pattern 0.95, similarity 0.5, fallback 0.95, min_budget 1024), logits_to_keep=1"},
             "tokens_per_s": round(args.seq_len / sec, 1), "mean_block_density": round(dens, 4),
             "decisions": sharing.decision_histogram(), "finite_logits": bool(torch.isfinite(out).all())}
+    if args.length_sweep:
+        # the reference's latency protocol (eval/efficiency/latency.py:21-108): same model, growing prompts,
+        # sparse path against the stock dense causal attention
+        sweep = []
+        for length in [int(x) for x in args.length_sweep.split(",") if x]:
+            ids_l = torch.randint(0, cfg.vocab_size, (1, length), generator=gen, device=dev)
+            row = {"seq_len": length}
+            for name, impl in (("shareprefill_s", "shareprefill"), ("dense_sdpa_s", "sdpa")):
+                model.config._attn_implementation = impl
+                try:
+                    with torch.no_grad():
+                        model(ids_l, use_cache=False, logits_to_keep=1)
+                        torch.cuda.synchronize()
+                        t1 = time.perf_counter()
+                        model(ids_l, use_cache=False, logits_to_keep=1)
+                        torch.cuda.synchronize()
+                    row[name] = round(time.perf_counter() - t1, 4)
+                except Exception as exc:  # e.g. the dense path running out of memory at the longest prompts
+                    row[name] = None
+                    row[name + "_error"] = type(exc).__name__
+                    torch.cuda.empty_cache()
+            model.config._attn_implementation = "shareprefill"
+            if row.get("shareprefill_s") and row.get("dense_sdpa_s"):
+                row["speedup"] = round(row["dense_sdpa_s"] / row["shareprefill_s"], 3)
+            sweep.append(row)
+        line["length_sweep"] = sweep
     print(json.dumps(line))
 
 
