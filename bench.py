@@ -363,6 +363,15 @@ def main():
         line["dense_causal_baseline"] = {"ms": round(dms, 3), "blocks": tri,
                                          "tflops": round(tri * FLOP_PER_BLOCK / dms / 1e9, 1),
                                          "frac": round(tri * FLOP_PER_BLOCK / dms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+        # decode step over the same cache (one query token per head; HBM-bound: K and V read once)
+        q1 = qh[:, -1].contiguous()
+        dec_ms = event_ms(lambda: ops.decode_attention(q1, kh, vh, w.head_dim ** -0.5), reps=5)
+        sdpa_ms = event_ms(lambda: torch.nn.functional.scaled_dot_product_attention(
+            q1[None, :, None, :], k, v, scale=w.head_dim ** -0.5, enable_gqa=True), reps=5)
+        dec_bytes = 2 * w.seq_len * w.hkv * w.head_dim * 2
+        line["decode_step"] = {"ms": round(dec_ms, 4), "GBps": round(dec_bytes / dec_ms / 1e6, 1),
+                               "frac_of_hbm_peak": round(dec_bytes / dec_ms / 1e6 / PEAK_HBM_GBS, 4),
+                               "torch_sdpa_ms": round(sdpa_ms, 4)}
         # what back-to-back MFMAs alone sustain on this chip (power-managed clocks): the practical ceiling
         line["mfma_sustained_tflops"] = {"random_operands": round(ops.mfma_probe_tflops(True), 1),
                                          "constant_operands": round(ops.mfma_probe_tflops(False), 1),

@@ -186,6 +186,17 @@ int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const void* v, i
                                   float* avg_attn, void* workspace, size_t workspace_bytes, uint32_t flags,
                                   sp_stream_t stream);
 
+/* ---- decode step -------------------------------------------------------------------------------
+ * Replaces the flash_attn_func call of the decode branch (shareprefill_attn.py:146-155): one query token per
+ * head against the whole KV cache, no mask.  q: bf16 [hq][d] (head stride in elements), k / v: bf16
+ * [hkv][n][d] with token and head strides, out: bf16 [hq][d] contiguous.  d = 128, hq / hkv <= 8.
+ * workspace: sp_decode_workspace_bytes(n, hq, hkv) bytes of device scratch, 8-byte aligned. */
+size_t sp_decode_workspace_bytes(int64_t n, int32_t hq, int32_t hkv);
+int sp_decode_attn_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv, int32_t d,
+                        int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n,
+                        int64_t v_stride_h, float softmax_scale, void* out, void* workspace,
+                        size_t workspace_bytes, sp_stream_t stream);
+
 /* ---- pivot state update (attention_sharing.py:94-103, attn/utils.py:60-76) ------------------
  * For each head with decision == SP_DEC_DENSE: per-row cumulative-mass selection (>= threshold,
  * crossing entry included) of avg_attn[h] -> state.pattern, the pivot's vs_ratio

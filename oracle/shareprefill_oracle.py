@@ -32,6 +32,7 @@ Parity pins (what each function is checked against, besides the HIP path):
   vs_ratio ........... literal gather-with-duplicates over vs_id_list
   csr_row_pointers ... reference docstring vector [0,5,8,9,13,14] -> [0,1,2,4,6]
   masked_attention ... torch SDPA (full mask), per-block causal attention (diagonal mask)
+  decode_attention ... torch SDPA with enable_gqa; one-key and uniform-logit closed forms
   layer() ............ scripted sharing scenarios (pivot / same-layer sibling / share / fallback)
 """
 
@@ -325,6 +326,25 @@ def block_probs(qbar_h, kbar_h, logits_in_input_dtype=True):
     tri = torch.tril(torch.ones(nb, nb, dtype=torch.bool))
     s = s.masked_fill(~tri, float("-inf"))
     return torch.softmax(s, dim=-1, dtype=torch.float32)
+
+
+# --------------------------------------------------------------------------- #
+# decode step
+# --------------------------------------------------------------------------- #
+def decode_attention(q, k, v, scale):
+    """fp32 attention of one query token per head over the whole cache (no mask), the decode
+    branch shareprefill_attn.py:146-155 (flash_attn_func with q_len = 1).
+
+    q [Hq,D], k/v [Hkv,N,D] -> out fp32 [Hq,D]; query head h reads kv head h // (Hq/Hkv).
+    """
+    hq, d = q.shape
+    g = hq // k.shape[0]
+    out = torch.zeros(hq, d, dtype=torch.float32)
+    for h in range(hq):
+        s = (k[h // g].float() @ q[h].float()) * scale
+        p = torch.softmax(s, dim=0)
+        out[h] = p @ v[h // g].float()
+    return out
 
 
 # --------------------------------------------------------------------------- #

@@ -254,6 +254,25 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
     return out
 
 
+def decode_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float) -> torch.Tensor:
+    """q bf16 [Hq, D] (one token), k / v bf16 [Hkv, N, D] views -> out bf16 [Hq, D].
+
+    Reference: the flash_attn_func decode branch (shareprefill_attn.py:146-155)."""
+    lib = _lib.load()
+    _check_hnd(k, "k")
+    _check_hnd(v, "v")
+    hq, d = q.shape
+    hkv, n, _ = k.shape
+    if q.dtype != torch.bfloat16 or q.stride(1) != 1:
+        raise ValueError("q must be bfloat16 [Hq, D] with a contiguous head_dim axis")
+    out = torch.empty(hq, d, dtype=torch.bfloat16, device=q.device)
+    ws = _workspace("decode", lib.sp_decode_workspace_bytes(n, hq, hkv), q.device)
+    st = lib.sp_decode_attn_bf16(_ptr(q), _ptr(k), _ptr(v), n, hq, hkv, d, q.stride(0), k.stride(1), k.stride(0),
+                                 v.stride(1), v.stride(0), softmax_scale, _ptr(out), _ptr(ws), ws.numel(), _stream())
+    _lib.check(st, "sp_decode_attn_bf16")
+    return out
+
+
 def attention_clock_mhz(n: int, hkv: int, d: int, block_size: int, device) -> float:
     """Average shader clock (MHz) seen by workgroup 0 of the last block_sparse_attention launch on this device
     (measurement aid; synchronises the current stream)."""

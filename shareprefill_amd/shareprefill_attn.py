@@ -39,9 +39,18 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
         raise NotImplementedError("gqa_interleave=True (query head h -> kv head h % Hkv) is not supported")
 
     if q_len == 1:
+        # decode step (shareprefill_attn.py:146-155): one query against the whole cache, nothing is selected
+        hkv = key_states.shape[1]
+        native = (query_states.dtype == torch.bfloat16 and head_dim == 128 and num_heads % hkv == 0
+                  and num_heads // hkv <= 8 and key_states.stride(3) == 1 and value_states.stride(3) == 1
+                  and key_states.stride(2) % 8 == 0 and value_states.stride(2) % 8 == 0)
+        if native:
+            outs = [ops.decode_attention(query_states[b, :, 0], key_states[b], value_states[b], softmax_scale)
+                    for b in range(bsz)]
+            return torch.stack(outs).unsqueeze(2), None
         out = torch.nn.functional.scaled_dot_product_attention(
             query_states, key_states, value_states, dropout_p=0.0, is_causal=False, scale=softmax_scale,
-            enable_gqa=key_states.shape[1] != num_heads)
+            enable_gqa=hkv != num_heads)
         return out, None
 
     if bsz != 1:

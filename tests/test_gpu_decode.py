@@ -1,0 +1,70 @@
+"""GPU parity of the decode step (one query token per head against the whole KV cache) with the fp32 oracle.
+
+Tolerance: max-abs <= 2e-2, mean-rel <= 2.5e-3 -- the output is rounded to bf16 (unit roundoff 2^-8 -> 1.3e-3
+mean-rel on its own); the kernel itself works in fp32 on the bf16 inputs."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import shareprefill_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_REL = 2e-2, 2.5e-3
+
+
+def _inputs(hq, hkv, n, seed, token_major=True):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(hq, 128, generator=g).to(torch.bfloat16)
+    if token_major:  # the layout of a Hugging Face cache after transpose: [N, Hkv, D] storage viewed as [Hkv, N, D]
+        k = torch.randn(n, hkv, 128, generator=g).to(torch.bfloat16).transpose(0, 1)
+        v = torch.randn(n, hkv, 128, generator=g).to(torch.bfloat16).transpose(0, 1)
+    else:
+        k = torch.randn(hkv, n, 128, generator=g).to(torch.bfloat16)
+        v = torch.randn(hkv, n, 128, generator=g).to(torch.bfloat16)
+    return q, k, v
+
+
+@pytest.mark.parametrize("hq,hkv,n", [(32, 8, 4096), (28, 4, 1000), (8, 8, 129), (4, 1, 1), (16, 2, 70000),
+                                      (8, 1, 127)])
+@pytest.mark.parametrize("token_major", [True, False])
+def test_decode_matches_oracle(gpu_device, hq, hkv, n, token_major):
+    from shareprefill_amd import ops
+
+    q, k, v = _inputs(hq, hkv, n, n + hq, token_major)
+    scale = 1.0 / math.sqrt(128)
+    ref = O.decode_attention(q, k, v, scale)
+    out = ops.decode_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), scale).cpu().float()
+    assert (out - ref).abs().max().item() <= MAX_ABS
+    assert ((out - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL
+    again = ops.decode_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), scale).cpu().float()
+    assert torch.equal(out, again)
+
+
+def test_decode_peaked_and_large_logits(gpu_device):
+    """A key that dominates (logit far above the rest) and large-magnitude logits: the online softmax across
+    tiles and chunks must neither overflow nor lose the winner."""
+    from shareprefill_amd import ops
+
+    q, k, v = _inputs(8, 2, 5000, 3)
+    k = k.clone()
+    k[:, 3333] = (q.float().view(2, 4, 128).mean(1) * 4).to(torch.bfloat16)  # strongly aligned with the queries
+    scale = 1.0
+    ref = O.decode_attention(q, k, v, scale)
+    out = ops.decode_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), scale).cpu().float()
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max().item() <= 4e-2  # values of magnitude up to ~4: bf16 ulp 0.03
+    assert ((out - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL
+
+
+def test_decode_rejects_unsupported(gpu_device):
+    from shareprefill_amd import ops
+
+    q, k, v = _inputs(9, 1, 256, 1)
+    with pytest.raises(NotImplementedError):
+        ops.decode_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), 0.1)  # 9 heads per kv head
+    q, k, v = _inputs(4, 2, 256, 1)
+    with pytest.raises(ValueError):
+        ops.decode_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), 0.0)

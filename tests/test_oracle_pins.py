@@ -317,6 +317,27 @@ KW = dict(bs=128, min_budget=128, max_budget=None, pattern_threshold=0.9, simila
           fallback_threshold=1e9, queryaware_threshold=0.0)
 
 
+def test_decode_attention_is_sdpa_with_gqa_and_closed_forms():
+    g = torch.Generator().manual_seed(11)
+    hq, hkv, n, d = 8, 2, 300, 16
+    q = torch.randn(hq, d, generator=g)
+    k = torch.randn(hkv, n, d, generator=g)
+    v = torch.randn(hkv, n, d, generator=g)
+    out = O.decode_attention(q, k, v, 0.3)
+    ref = torch.nn.functional.scaled_dot_product_attention(q[None, :, None, :], k[None], v[None], scale=0.3,
+                                                           enable_gqa=True)[0, :, 0]
+    assert torch.allclose(out, ref, atol=1e-5)
+    # a single key: the output is that key's value, whatever the logit
+    one = O.decode_attention(q, k[:, :1], v[:, :1], 7.0)
+    assert torch.allclose(one, v[:, 0].repeat_interleave(hq // hkv, 0), atol=1e-6)
+    # equal logits (zero query): the plain mean of the values
+    mean = O.decode_attention(torch.zeros(hq, d), k, v, 1.0)
+    assert torch.allclose(mean, v.mean(1).repeat_interleave(hq // hkv, 0), atol=1e-5)
+    # a transposed head mapping (h % hkv instead of h // g) must differ
+    wrong = torch.stack([torch.softmax((k[h % hkv] @ q[h]) * 0.3, 0) @ v[h % hkv] for h in range(hq)])
+    assert not torch.allclose(out, wrong, atol=1e-3)
+
+
 def test_sharing_scenarios():
     q, k, v = _toy()
     sh = O.OracleSharing(O.ClusterTable(TOY_TABLE["clusters"], TOY_TABLE["shared_clusters"]))
