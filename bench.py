@@ -369,9 +369,13 @@ def main():
         sdpa_ms = event_ms(lambda: torch.nn.functional.scaled_dot_product_attention(
             q1[None, :, None, :], k, v, scale=w.head_dim ** -0.5, enable_gqa=True), reps=5)
         dec_bytes = 2 * w.seq_len * w.hkv * w.head_dim * 2
-        line["decode_step"] = {"ms": round(dec_ms, 4), "GBps": round(dec_bytes / dec_ms / 1e6, 1),
-                               "frac_of_hbm_peak": round(dec_bytes / dec_ms / 1e6 / PEAK_HBM_GBS, 4),
-                               "torch_sdpa_ms": round(sdpa_ms, 4)}
+        kc, vc = kh.contiguous(), vh.contiguous()  # [Hkv, N, D] contiguous: the layout of a Hugging Face KV cache
+        dec_hm_ms = event_ms(lambda: ops.decode_attention(q1, kc, vc, w.head_dim ** -0.5), reps=5)
+        line["decode_step"] = {"ms": round(dec_hm_ms, 4), "GBps": round(dec_bytes / dec_hm_ms / 1e6, 1),
+                               "frac_of_hbm_peak": round(dec_bytes / dec_hm_ms / 1e6 / PEAK_HBM_GBS, 4),
+                               "layout": "k, v [Hkv, N, D] contiguous",
+                               "token_major_kv_ms": round(dec_ms, 4), "torch_sdpa_ms": round(sdpa_ms, 4)}
+        del kc, vc
         # what back-to-back MFMAs alone sustain on this chip (power-managed clocks): the practical ceiling
         line["mfma_sustained_tflops"] = {"random_operands": round(ops.mfma_probe_tflops(True), 1),
                                          "constant_operands": round(ops.mfma_probe_tflops(False), 1),

@@ -1,174 +1,183 @@
 // Decode step: one query token per head against the whole KV cache (GQA, no mask), bf16 in / bf16 out, fp32
 // softmax.  Replaces the flash_attn_func call of the reference's decode branch (shareprefill_attn.py:146-155).
 //
-// HBM-bound: K and V are read exactly once (2 * n * hkv * d * 2 bytes); everything else is noise.  The cache of
-// one kv head is split into chunks; one workgroup streams a chunk for all query heads of the group (so the
-// group's `g` heads share every K / V byte), keeps an online softmax, and leaves an unnormalised partial
-// (o, m, l); a second tiny kernel merges the partials in chunk order.  No matrix core: with at most 8 query rows
-// the products are a few hundred FMAs per thread and tile.
+// HBM-bound: K and V are read exactly once (2 * n * hkv * d * 2 bytes); everything else has to stay out of the
+// way.  The cache of one kv head is split into chunks; one workgroup streams a chunk for all query heads of the
+// group (so the group's `g` heads share every K / V byte), keeps an online softmax, and leaves an unnormalised
+// partial (o, m, l); a second tiny kernel merges the partials in chunk order.
+//
+// Both products run on the matrix core with the group's heads as a (mostly empty) 32-wide operand -- the MFMAs
+// are free here, the point is to keep the vector ALU out of the inner loop:
+//   S^T[keys x heads] = K . Q^T    A = K rows from LDS, B = the queries in registers (columns >= g are zero)
+//   O[heads x d]     += P . V      A = P (bf16, from LDS), B = V read from its row-major LDS tile with the
+//                                  transposing LDS load (ds_read_b64_tr_b16), which hands every lane four
+//                                  consecutive keys of one channel.
 #include "sp_common.h"
 
 #define DC_THREADS 256
-#define DC_TILE 128  // keys per tile
+#define DC_TILE 128   // keys per tile
 #define DC_D 128
-#define DC_GMAX 8    // query heads per kv head
+#define DC_GMAX 8     // query heads per kv head
+#define DC_PITCH 136  // bf16 elements per LDS row (272 bytes: conflict-free 128-bit reads)
 
 typedef uint32_t dc_u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 dc_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 dc_bf16x4 __attribute__((ext_vector_type(4)));
+typedef float dc_floatx16 __attribute__((ext_vector_type(16)));
+typedef float dc_floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 dc_bf16x2 __attribute__((ext_vector_type(2)));
 
-__device__ static __forceinline__ float dc_lo(uint32_t w) { return __uint_as_float(w << 16); }
-__device__ static __forceinline__ float dc_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ static __forceinline__ uint32_t dc_pack2(float a, float b) {
+  dc_floatx2 f;
+  f[0] = a;
+  f[1] = b;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, dc_bf16x2));
+}
+
+// thread t fetches chunk t%16 (16 bytes) of rows t/16, t/16+16, ... of a 128-row tile; rows past the end are clamped
+__device__ static __forceinline__ void dc_fetch(const sp_bf16* __restrict__ x, int64_t n, int64_t stride_n, int64_t kb,
+                                               int t, dc_u32x4 (&r)[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    int64_t key = kb + i * 16 + (t >> 4);
+    if (key > n - 1) key = n - 1;
+    r[i] = *reinterpret_cast<const dc_u32x4*>(x + key * stride_n + (t & 15) * 8);
+  }
+}
+
+__device__ static __forceinline__ void dc_store(sp_bf16* tile, int t, const dc_u32x4 (&r)[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) *reinterpret_cast<dc_u32x4*>(tile + (i * 16 + (t >> 4)) * DC_PITCH + (t & 15) * 8) = r[i];
+}
 
 // grid (splits, hkv); partial layout: o [hkv][splits][g][128] fp32, ml [hkv][splits][g] float2 (m in log2 units, l)
 __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ v, int64_t n, int g,
     int64_t sq_h, int64_t sk_n, int64_t sk_h, int64_t sv_n, int64_t sv_h, float scale_log2, int64_t keys_per_split,
     float* __restrict__ o_part, float2* __restrict__ ml_part) {
-  __shared__ float Qs[DC_GMAX][DC_D];     // the group's queries, fp32
-  __shared__ float Ps[DC_GMAX][DC_TILE];  // logits, then probabilities of the current tile
-  __shared__ float alpha_s[DC_GMAX];
-  __shared__ float red[4][DC_GMAX][DC_D];  // cross-wave reduction of the output partials (16 KiB)
+  __shared__ __attribute__((aligned(16))) sp_bf16 Ks[DC_TILE * DC_PITCH];
+  __shared__ __attribute__((aligned(16))) sp_bf16 Vs[DC_TILE * DC_PITCH];
+  __shared__ __attribute__((aligned(16))) sp_bf16 Ps[DC_GMAX * DC_PITCH];  // probabilities [head][key]
+  __shared__ float wmax[4][DC_GMAX], wsum[4][DC_GMAX], alpha_s[DC_GMAX];
   const int split = blockIdx.x, kvh = blockIdx.y, splits = gridDim.x;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int lh = lane & 31, hi = lane >> 5;  // operand column / row inside a 32-wide tile, lane half
+  const bool head_ok = lh < g;               // this lane's S^T column is a real head
   const sp_bf16* kh = k + (int64_t)kvh * sk_h;
   const sp_bf16* vh = v + (int64_t)kvh * sv_h;
-  for (int i = t; i < g * DC_D; i += DC_THREADS)
-    Qs[i / DC_D][i % DC_D] = sp_bf16_to_f32(q[(int64_t)(kvh * g + i / DC_D) * sq_h + i % DC_D]);
-  __syncthreads();
+
+  // B operand of S^T = K . Q^T: column lh = head, k-step ks covers channels 16ks + 8hi .. +7
+  dc_bf16x8 qb[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    dc_u32x4 raw = {0, 0, 0, 0};
+    if (head_ok) raw = *reinterpret_cast<const dc_u32x4*>(q + (int64_t)(kvh * g + lh) * sq_h + 16 * ks + 8 * hi);
+    qb[ks] = __builtin_bit_cast(dc_bf16x8, raw);
+  }
 
   const int64_t key_begin = (int64_t)split * keys_per_split;
   int64_t key_end = key_begin + keys_per_split;
   if (key_end > n) key_end = n;
 
-  // roles: logits -- thread handles key t/2, channel half t%2;  softmax -- head t/32, keys 4*(t%32)..+3;
-  //        output -- thread handles channels 8*(t%16)..+7 for keys t/16, t/16+16, ...
-  const int qk_key = t >> 1, qk_half = t & 1;
-  const int sm_head = t >> 5, sm_k0 = (t & 31) * 4;
-  const int pv_chunk = t & 15, pv_sub = t >> 4;
-  float acc[DC_GMAX][8];
-#pragma unroll
-  for (int h = 0; h < DC_GMAX; ++h)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[h][j] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;  // of head sm_head (replicated over its 32 threads)
-
+  dc_floatx16 o = {0};                   // rows = heads 8(r/4) + 4hi + r%4 (only r < 4 can be real), col = channel 32*wave + lh
+  float m_run = -INFINITY, l_run = 0.f;  // of head lh (every wave keeps the same copy)
+  dc_u32x4 kr[8], vr[8];
+  if (key_begin < key_end) {
+    dc_fetch(kh, n, sk_n, key_begin, t, kr);
+    dc_fetch(vh, n, sv_n, key_begin, t, vr);
+  }
   for (int64_t kb = key_begin; kb < key_end; kb += DC_TILE) {
-    // ---- loads of this tile: K half row for the logits, eight V chunks for the output ----
-    dc_u32x4 kr[8], vr[8];
+    __syncthreads();  // the previous tile's operand reads are done
+    dc_store(Ks, t, kr);
+    dc_store(Vs, t, vr);
+    __syncthreads();
+    if (kb + DC_TILE < key_end) {  // next tile on its way while this one is used
+      dc_fetch(kh, n, sk_n, kb + DC_TILE, t, kr);
+      dc_fetch(vh, n, sv_n, kb + DC_TILE, t, vr);
+    }
+    // ---- S^T for this wave's 32 keys: acc[r] = logit(key 32*wave + 8(r/4) + 4hi + r%4, head lh) ----
+    dc_floatx16 acc = {0};
     {
-      int64_t key = kb + qk_key;
-      if (key > n - 1) key = n - 1;
-      const dc_u32x4* src = reinterpret_cast<const dc_u32x4*>(kh + key * sk_n + qk_half * 64);
+      const sp_bf16* arow = Ks + (32 * wave + lh) * DC_PITCH + 8 * hi;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) kr[i] = src[i];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        int64_t vk = kb + pv_sub + 16 * i;
-        if (vk > n - 1) vk = n - 1;
-        vr[i] = *reinterpret_cast<const dc_u32x4*>(vh + vk * sv_n + pv_chunk * 8);
+      for (int ks = 0; ks < 8; ++ks) {
+        const dc_u32x4 raw = *reinterpret_cast<const dc_u32x4*>(arow + 16 * ks);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(dc_bf16x8, raw), qb[ks], acc, 0, 0, 0);
       }
     }
-    // ---- logits: s[h] = q_h . k over this thread's 64 channels, summed with the partner thread ----
-    float s[DC_GMAX];
+    const int valid = (int)((key_end - kb) < DC_TILE ? (key_end - kb) : DC_TILE);
+    float mx = -INFINITY;
 #pragma unroll
-    for (int h = 0; h < DC_GMAX; ++h) s[h] = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float kf[8];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        kf[2 * j] = dc_lo(kr[i][j]);
-        kf[2 * j + 1] = dc_hi(kr[i][j]);
-      }
-#pragma unroll
-      for (int h = 0; h < DC_GMAX; ++h) {
-        if (h < g) {
-          const float4 qa = *reinterpret_cast<const float4*>(&Qs[h][qk_half * 64 + i * 8]);
-          const float4 qb = *reinterpret_cast<const float4*>(&Qs[h][qk_half * 64 + i * 8 + 4]);
-          s[h] += kf[0] * qa.x + kf[1] * qa.y + kf[2] * qa.z + kf[3] * qa.w + kf[4] * qb.x + kf[5] * qb.y +
-                  kf[6] * qb.z + kf[7] * qb.w;
-        }
-      }
+    for (int r = 0; r < 16; ++r) {
+      const int key = 32 * wave + 8 * (r >> 2) + 4 * hi + (r & 3);
+      acc[r] = key < valid ? acc[r] * scale_log2 : -INFINITY;
+      mx = fmaxf(mx, acc[r]);
     }
-    const bool key_ok = kb + qk_key < key_end;
+    mx = fmaxf(mx, __shfl_xor(mx, 32, SP_WAVE));
+    if (head_ok && hi == 0) wmax[wave][lh] = mx;
+    __syncthreads();
+    float m_new = m_run, alpha = 1.f;
+    if (head_ok) {
+      m_new = fmaxf(fmaxf(fmaxf(wmax[0][lh], wmax[1][lh]), fmaxf(wmax[2][lh], wmax[3][lh])), m_run);  // finite
+      alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile
+      float ls = 0.f;
+      sp_bf16* prow = Ps + lh * DC_PITCH + 32 * wave + 4 * hi;
 #pragma unroll
-    for (int h = 0; h < DC_GMAX; ++h) {
-      if (h < g) {
-        const float tot = s[h] + __shfl_xor(s[h], 1, SP_WAVE);
-        if (qk_half == 0) Ps[h][qk_key] = key_ok ? tot * scale_log2 : -INFINITY;
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const float p0 = __builtin_amdgcn_exp2f(acc[4 * r4 + 0] - m_new), p1 = __builtin_amdgcn_exp2f(acc[4 * r4 + 1] - m_new);
+        const float p2 = __builtin_amdgcn_exp2f(acc[4 * r4 + 2] - m_new), p3 = __builtin_amdgcn_exp2f(acc[4 * r4 + 3] - m_new);
+        ls += (p0 + p1) + (p2 + p3);
+        *reinterpret_cast<uint2*>(prow + 8 * r4) = make_uint2(dc_pack2(p0, p1), dc_pack2(p2, p3));
+      }
+      ls += __shfl_xor(ls, 32, SP_WAVE);
+      if (hi == 0) {
+        wsum[wave][lh] = ls;
+        if (wave == 0) alpha_s[lh] = alpha;
       }
     }
     __syncthreads();
-    // ---- online softmax per head (32 threads a head, fixed xor tree) ----
-    if (sm_head < g) {
-      float4 sv = *reinterpret_cast<const float4*>(&Ps[sm_head][sm_k0]);
-      float mx = fmaxf(fmaxf(sv.x, sv.y), fmaxf(sv.z, sv.w));
-#pragma unroll
-      for (int o = 1; o < 32; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, SP_WAVE));
-      const float m_new = fmaxf(m_run, mx);  // finite: the tile holds at least one real key
-      sv.x = __builtin_amdgcn_exp2f(sv.x - m_new);
-      sv.y = __builtin_amdgcn_exp2f(sv.y - m_new);
-      sv.z = __builtin_amdgcn_exp2f(sv.z - m_new);
-      sv.w = __builtin_amdgcn_exp2f(sv.w - m_new);
-      float ls = (sv.x + sv.y) + (sv.z + sv.w);
-#pragma unroll
-      for (int o = 1; o < 32; o <<= 1) ls += __shfl_xor(ls, o, SP_WAVE);
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf)
-      l_run = l_run * alpha + ls;
+    if (head_ok) {
+      l_run = l_run * alpha + ((wsum[0][lh] + wsum[1][lh]) + (wsum[2][lh] + wsum[3][lh]));
       m_run = m_new;
-      *reinterpret_cast<float4*>(&Ps[sm_head][sm_k0]) = sv;
-      if ((t & 31) == 0) alpha_s[sm_head] = alpha;
     }
-    __syncthreads();
-    // ---- output: acc[h][ch] = acc * alpha_h + sum_keys p[h][key] * v[key][ch] ----
+    // ---- O += P . V for this wave's 32 channels; only accumulator rows of real heads need the rescale ----
 #pragma unroll
-    for (int h = 0; h < DC_GMAX; ++h) {
-      if (h < g) {
-        const float a = alpha_s[h];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[h][j] *= a;
-      }
+    for (int r = 0; r < 4; ++r) {
+      const int h = 4 * hi + r;
+      if (h < g) o[r] *= alpha_s[h];
     }
+    {
+      const sp_bf16* prow = Ps + lh * DC_PITCH + 8 * hi;
+      // transposing read: the 16 lanes of a block address 4 key rows x 16 channels (4 lanes x 8 bytes per row) and
+      // each lane receives 4 consecutive keys of its channel
+      const sp_bf16* vtr = Vs + (8 * hi + ((lane & 15) >> 2)) * DC_PITCH + 32 * wave + 16 * ((lane >> 4) & 1) +
+                           4 * (lane & 3);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float vf[8];
+      for (int kk = 0; kk < 8; ++kk) {
+        dc_u32x4 praw = {0, 0, 0, 0};
+        if (head_ok) praw = *reinterpret_cast<const dc_u32x4*>(prow + 16 * kk);
+        const dc_bf16x4 b0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+            (__attribute__((address_space(3))) dc_bf16x4*)(vtr + (16 * kk) * DC_PITCH));
+        const dc_bf16x4 b1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+            (__attribute__((address_space(3))) dc_bf16x4*)(vtr + (16 * kk + 4) * DC_PITCH));
+        dc_bf16x8 bv;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        vf[2 * j] = dc_lo(vr[i][j]);
-        vf[2 * j + 1] = dc_hi(vr[i][j]);
-      }
-#pragma unroll
-      for (int h = 0; h < DC_GMAX; ++h) {
-        if (h < g) {
-          const float p = Ps[h][pv_sub + 16 * i];  // 0 for keys past the chunk
-#pragma unroll
-          for (int j = 0; j < 8; ++j) acc[h][j] += p * vf[j];
+        for (int j = 0; j < 4; ++j) {
+          bv[j] = b0[j];
+          bv[4 + j] = b1[j];
         }
+        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(dc_bf16x8, praw), bv, o, 0, 0, 0);
       }
     }
-    __syncthreads();  // Ps / alpha_s are rewritten by the next tile
   }
 
-  // ---- reduce the 16 key groups: inside the wave (lanes l, l^16, l^32, l^48), then across the four waves ----
-#pragma unroll
-  for (int h = 0; h < DC_GMAX; ++h) {
-    if (h < g) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        float x = acc[h][j];
-        x += __shfl_xor(x, 16, SP_WAVE);
-        x += __shfl_xor(x, 32, SP_WAVE);
-        if (lane < 16) red[wave][h][pv_chunk * 8 + j] = x;
-      }
-    }
-  }
-  __syncthreads();
   float* op = o_part + (((int64_t)kvh * splits + split) * g) * DC_D;
-  for (int i = t; i < g * DC_D; i += DC_THREADS) {
-    const int h = i / DC_D, c = i % DC_D;
-    op[i] = (red[0][h][c] + red[1][h][c]) + (red[2][h][c] + red[3][h][c]);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int h = 4 * hi + r;
+    if (h < g) op[h * DC_D + 32 * wave + lh] = o[r];
   }
-  if (sm_head < g && (t & 31) == 0)
-    ml_part[((int64_t)kvh * splits + split) * g + sm_head] = make_float2(m_run, l_run);
+  if (wave == 0 && hi == 0 && head_ok) ml_part[((int64_t)kvh * splits + split) * g + lh] = make_float2(m_run, l_run);
 }
 
 // one workgroup of 128 threads per query head: merges the chunk partials in chunk order
