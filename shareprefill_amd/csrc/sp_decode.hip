@@ -180,20 +180,32 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
   if (wave == 0 && hi == 0 && head_ok) ml_part[((int64_t)kvh * splits + split) * g + lh] = make_float2(m_run, l_run);
 }
 
-// one workgroup of 128 threads per query head: merges the chunk partials in chunk order
+// one workgroup of 128 threads per query head: merges the chunk partials (sums in chunk order)
+#define DC_MAX_SPLITS 512
 __global__ __launch_bounds__(DC_D) void sp_decode_combine_kernel(const float* __restrict__ o_part,
                                                                  const float2* __restrict__ ml_part, int g, int splits,
                                                                  sp_bf16* __restrict__ out) {
+  __shared__ float w_s[DC_MAX_SPLITS];  // weight of chunk s: exp2(m_s - m), 0 for an empty chunk
+  __shared__ float red[2];
   const int hq_idx = blockIdx.x, kvh = hq_idx / g, h = hq_idx % g, c = threadIdx.x;
+  const float2* ml = ml_part + (int64_t)kvh * splits * g + h;
   float m = -INFINITY;
-  for (int s = 0; s < splits; ++s) m = fmaxf(m, ml_part[((int64_t)kvh * splits + s) * g + h].x);
+  for (int s = c; s < splits; s += DC_D) m = fmaxf(m, ml[(int64_t)s * g].x);
+  m = sp_wave_max(m);
+  if ((c & 63) == 0) red[c >> 6] = m;
+  __syncthreads();
+  m = fmaxf(red[0], red[1]);
+  for (int s = c; s < splits; s += DC_D) {
+    const float ms = ml[(int64_t)s * g].x;
+    w_s[s] = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - m);
+  }
+  __syncthreads();
+  const float* op = o_part + ((int64_t)kvh * splits * g + h) * DC_D + c;
   float l = 0.f, o = 0.f;
+#pragma unroll 8
   for (int s = 0; s < splits; ++s) {
-    const float2 ml = ml_part[((int64_t)kvh * splits + s) * g + h];
-    if (ml.x == -INFINITY) continue;  // empty chunk
-    const float w = __builtin_amdgcn_exp2f(ml.x - m);
-    l += ml.y * w;
-    o += o_part[(((int64_t)kvh * splits + s) * g + h) * DC_D + c] * w;
+    l += ml[(int64_t)s * g].y * w_s[s];
+    o += op[(int64_t)s * g * DC_D] * w_s[s];
   }
   out[(int64_t)hq_idx * DC_D + c] = sp_f32_to_bf16(o / l);
 }
@@ -204,6 +216,7 @@ static int dc_splits(int64_t n, int32_t hkv) {
   int64_t want = sp_ceil_div(512, hkv);  // about two workgroups per CU
   if (want > tiles) want = tiles;
   if (want < 1) want = 1;
+  if (want > DC_MAX_SPLITS) want = DC_MAX_SPLITS;
   return (int)want;
 }
 

@@ -204,18 +204,32 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_stats_kernel(
 }
 
 // ---- kernel 2: fold chunk partials ------------------------------------------------------------------
-__global__ __launch_bounds__(LQ_ROWS) void sp_lastq_combine_kernel(const float2* __restrict__ partial, int n_chunks,
-                                                                   float2* __restrict__ rowstat /* [hq][128] */) {
-  const int h = blockIdx.x, row = threadIdx.x;
+// One workgroup per head: 8 groups of 128 threads; group j folds chunks j, j+8, ... of every row, then the eight
+// group results are merged in a fixed order.
+#define LQ_COMBINE_GROUPS 8
+__global__ __launch_bounds__(LQ_ROWS * LQ_COMBINE_GROUPS) void sp_lastq_combine_kernel(
+    const float2* __restrict__ partial, int n_chunks, float2* __restrict__ rowstat /* [hq][128] */) {
+  __shared__ float gm[LQ_COMBINE_GROUPS][LQ_ROWS], gl[LQ_COMBINE_GROUPS][LQ_ROWS];
+  const int h = blockIdx.x, row = threadIdx.x % LQ_ROWS, grp = threadIdx.x / LQ_ROWS;
   const float2* p = partial + (int64_t)h * n_chunks * LQ_ROWS + row;
   float m = -INFINITY;
-  for (int c = 0; c < n_chunks; ++c) m = fmaxf(m, p[(int64_t)c * LQ_ROWS].x);
+  for (int c = grp; c < n_chunks; c += LQ_COMBINE_GROUPS) m = fmaxf(m, p[(int64_t)c * LQ_ROWS].x);
+  gm[grp][row] = m;
+  __syncthreads();
+  m = gm[0][row];
+#pragma unroll
+  for (int j = 1; j < LQ_COMBINE_GROUPS; ++j) m = fmaxf(m, gm[j][row]);
   float l = 0.f;
-  for (int c = 0; c < n_chunks; ++c) {
+  for (int c = grp; c < n_chunks; c += LQ_COMBINE_GROUPS) {
     const float2 v = p[(int64_t)c * LQ_ROWS];
     if (v.x > -INFINITY) l += v.y * __expf(v.x - m);
   }
-  rowstat[h * LQ_ROWS + row] = make_float2(m, 1.0f / l);
+  gl[grp][row] = l;
+  __syncthreads();
+  if (grp == 0) {
+    l = ((gl[0][row] + gl[1][row]) + (gl[2][row] + gl[3][row])) + ((gl[4][row] + gl[5][row]) + (gl[6][row] + gl[7][row]));
+    rowstat[h * LQ_ROWS + row] = make_float2(m, 1.0f / l);
+  }
 }
 
 // ---- kernel 3: probabilities -> vertical / slash ------------------------------------------------------
@@ -347,7 +361,8 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
                      (const sp_bf16*)k, n, hkv, group, q_stride_n, q_stride_h, k_stride_n, k_stride_h, inv_sqrt_d,
                      flags, n_chunks, partial);
   SP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sp_lastq_combine_kernel, dim3(hq), dim3(LQ_ROWS), 0, s, partial, n_chunks, rowstat);
+  hipLaunchKernelGGL(sp_lastq_combine_kernel, dim3(hq), dim3(LQ_ROWS * LQ_COMBINE_GROUPS), 0, s, partial, n_chunks,
+                     rowstat);
   SP_LAUNCH_CHECK();
   const size_t lds_bytes = (LQ_ROWS * LQ_PITCH + 4) * sizeof(float);
   static bool attr_set = false;
