@@ -667,26 +667,40 @@ extern "C" int sp_queryaware_test_bf16(const void* q, const void* kbar, const fl
 // cols[c] = 1 for the nv best columns (column 0 forced), dists[dd] = 1 for the ns best distances
 // (distance 0 forced); slash index i holds distance nb-1-i.
 // ------------------------------------------------------------------------------------------------
+// rank of element i in the order (key descending, index ascending) = #{j < i: key_j >= key_i} + #{j > i: key_j > key_i};
+// keys [nbp] in LDS, padded with zeros to a multiple of 4 (a zero key never outranks anything but zeros behind i)
+__device__ static inline int vs_rank(const uint32_t* keys, int nb, int i) {
+  const uint32_t ki = keys[i];
+  int r = 0;
+  const int i4 = i & ~3;
+  for (int j = 0; j < i4; j += 4) {
+    const uint4 k4 = *reinterpret_cast<const uint4*>(keys + j);
+    r += (k4.x >= ki) + (k4.y >= ki) + (k4.z >= ki) + (k4.w >= ki);
+  }
+  for (int j = i4; j < i; ++j) r += keys[j] >= ki;
+  const int e4 = (i + 4) & ~3;
+  for (int j = i + 1; j < e4 && j < nb; ++j) r += keys[j] > ki;
+  for (int j = e4; j < nb; j += 4) {  // reads up to 3 padding zeros past nb: they never count (0 > ki is false)
+    const uint4 k4 = *reinterpret_cast<const uint4*>(keys + j);
+    r += (k4.x > ki) + (k4.y > ki) + (k4.z > ki) + (k4.w > ki);
+  }
+  return r;
+}
+
 __device__ static void vs_sets(const float* __restrict__ vert, const float* __restrict__ slash, int nb, int nv,
-                               int ns, uint32_t* keys /* LDS [nb] */, uint8_t* cols, uint8_t* dists, int nthreads) {
+                               int ns, uint32_t* keys /* LDS [RS_MAX], 16-byte aligned */, uint8_t* cols,
+                               uint8_t* dists, int nthreads) {
   const uint32_t inf_key = 0x7f800000u;
-  for (int i = threadIdx.x; i < nb; i += nthreads) keys[i] = (i == 0) ? inf_key : sp_sort_key(vert[i]);
+  const int nbp = (nb + 3) & ~3;
+  for (int i = threadIdx.x; i < nbp; i += nthreads)
+    keys[i] = i >= nb ? 0u : ((i == 0) ? inf_key : sp_sort_key(vert[i]));
   __syncthreads();
-  for (int i = threadIdx.x; i < nb; i += nthreads) {
-    const uint32_t ki = keys[i];
-    int r = 0;
-    for (int j = 0; j < nb; ++j) r += (keys[j] > ki) || (keys[j] == ki && j < i);
-    cols[i] = r < nv;
-  }
+  for (int i = threadIdx.x; i < nb; i += nthreads) cols[i] = vs_rank(keys, nb, i) < nv;
   __syncthreads();
-  for (int i = threadIdx.x; i < nb; i += nthreads) keys[i] = (i == nb - 1) ? inf_key : sp_sort_key(slash[i]);
+  for (int i = threadIdx.x; i < nbp; i += nthreads)
+    keys[i] = i >= nb ? 0u : ((i == nb - 1) ? inf_key : sp_sort_key(slash[i]));
   __syncthreads();
-  for (int i = threadIdx.x; i < nb; i += nthreads) {
-    const uint32_t ki = keys[i];
-    int r = 0;
-    for (int j = 0; j < nb; ++j) r += (keys[j] > ki) || (keys[j] == ki && j < i);
-    dists[nb - 1 - i] = r < ns;
-  }
+  for (int i = threadIdx.x; i < nb; i += nthreads) dists[nb - 1 - i] = vs_rank(keys, nb, i) < ns;
   __syncthreads();
 }
 
@@ -703,7 +717,7 @@ __global__ __launch_bounds__(DEC_THREADS) void sp_share_decide_kernel(
     int32_t* __restrict__ ns_f) {
   __shared__ float s_jv[DEC_MAX_HEADS], s_js[DEC_MAX_HEADS];
   __shared__ int32_t s_new[DEC_MAX_HEADS];
-  __shared__ uint32_t s_keys[RS_MAX];
+  __shared__ __attribute__((aligned(16))) uint32_t s_keys[RS_MAX];
   const int nb = st.nb;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   // similarity of every candidate head against its cluster's stored pivot (pivots of EARLIER layers only)
@@ -798,27 +812,31 @@ extern "C" int sp_share_decide(const sp_cluster_state* state, const int32_t* hea
 // ------------------------------------------------------------------------------------------------
 // mask construction (attention_sharing.py:303-337 and attn/utils.py:99-128 as a set)
 // ------------------------------------------------------------------------------------------------
-#define MASK_THREADS 256
+#define MASK_THREADS 1024
+#define MASK_SPLIT 8  // workgroups per head: each ranks the head's vectors itself and writes a share of the rows
 __global__ __launch_bounds__(MASK_THREADS) void sp_build_mask_kernel(
     sp_cluster_state st, const int32_t* __restrict__ head_cluster, const int32_t* __restrict__ decision,
     const float* __restrict__ vert_blk, const float* __restrict__ slash_blk, const int32_t* __restrict__ nv_f,
     const int32_t* __restrict__ ns_f, int nb, int nbw, uint64_t* __restrict__ mask) {
-  __shared__ uint32_t s_keys[RS_MAX];
+  __shared__ __attribute__((aligned(16))) uint32_t s_keys[RS_MAX];
   __shared__ uint8_t s_cols[RS_MAX], s_dists[RS_MAX];
   const int h = blockIdx.x;
   const int dec = decision[h];
-  vs_sets(vert_blk + (int64_t)h * nb, slash_blk + (int64_t)h * nb, nb, nv_f[h], ns_f[h], s_keys, s_cols, s_dists,
-          MASK_THREADS);
+  if (dec != SP_DEC_DENSE)
+    vs_sets(vert_blk + (int64_t)h * nb, slash_blk + (int64_t)h * nb, nb, nv_f[h], ns_f[h], s_keys, s_cols, s_dists,
+            MASK_THREADS);
   const uint64_t* pat = nullptr;
   if (dec == SP_DEC_SHARE) pat = st.pattern + (int64_t)head_cluster[h] * nb * nbw;
   uint64_t* mh = mask + (int64_t)h * nb * nbw;
-  for (int idx = threadIdx.x; idx < nb * nbw; idx += MASK_THREADS) {
+  const int rows_per = (nb + MASK_SPLIT - 1) / MASK_SPLIT;
+  const int r_begin = blockIdx.y * rows_per, r_end = min(nb, r_begin + rows_per);
+  for (int idx = r_begin * nbw + threadIdx.x; idx < r_end * nbw; idx += MASK_THREADS) {
     const int r = idx / nbw, w = idx - r * nbw;
     uint64_t bits = 0;
     const int c0 = w * 64;
     const int cend = min(c0 + 64, r + 1);
     if (dec == SP_DEC_DENSE) {
-      for (int c = c0; c < cend; ++c) bits |= 1ull << (c - c0);
+      if (cend > c0) bits = (cend - c0 == 64) ? ~0ull : ((1ull << (cend - c0)) - 1ull);
     } else {
       for (int c = c0; c < cend; ++c) {
         if (s_cols[c] | s_dists[r - c]) bits |= 1ull << (c - c0);
@@ -839,7 +857,8 @@ extern "C" int sp_build_mask(const sp_cluster_state* state, const int32_t* head_
              SP_ERR_INVALID_ARGUMENT, "sp_build_mask: null pointer");
   SP_REQUIRE(hq > 0 && nb > 0 && nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_build_mask: nb=%d unsupported (max %d)", nb,
              RS_MAX);
-  hipLaunchKernelGGL(sp_build_mask_kernel, dim3(hq), dim3(MASK_THREADS), 0, (hipStream_t)stream, *state, head_cluster,
+  hipLaunchKernelGGL(sp_build_mask_kernel, dim3(hq, MASK_SPLIT), dim3(MASK_THREADS), 0, (hipStream_t)stream, *state,
+                     head_cluster,
                      decision, vert_blk, slash_blk, nv_final, ns_final, nb, (nb + 63) / 64, mask);
   SP_LAUNCH_CHECK();
   return SP_OK;
