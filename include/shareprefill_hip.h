@@ -105,13 +105,16 @@ int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int32_t hq, in
  * sums of the values truncated to unsigned 2^-48 fixed point.  Inputs: finite, >= 0, row sum < 2^14.
  *
  * sp_cover_count: score_cover_topk (utils.py:47-50): out[v] = count(cumsum <= thr) + 1 for each of
- * n_vec vectors of length len (row stride = len). */
-int sp_cover_count(const float* x, int32_t n_vec, int64_t len, float thr, int32_t* out, sp_stream_t stream);
+ * n_vec vectors of length len (row stride = len).
+ * workspace (both functions): sp_cover_select_workspace_bytes(n_vec resp. 2*hq) bytes of device scratch, 8-byte
+ * aligned. */
+int sp_cover_count(const float* x, int32_t n_vec, int64_t len, float thr, int32_t* out, void* workspace,
+                   size_t workspace_bytes, sp_stream_t stream);
 
 /* budgets of attention_sharing.py:169-176: clamp(cover_count(.)/bs + 1, minb, maxb) for both vectors */
 int sp_cover_budgets(const float* vert_tok, const float* slash_tok, int32_t hq, int64_t n, int32_t bs,
                      float pattern_threshold, int32_t min_blocks, int32_t max_blocks, int32_t* nv, int32_t* ns,
-                     sp_stream_t stream);
+                     void* workspace, size_t workspace_bytes, sp_stream_t stream);
 
 /* ---- query-aware test (attention_sharing.py:193-202) ----------------------------------------
  * avg_qk[h] = softmax_fp32(mean_i(last_q[h]) . kbar[:, h/g]); js_qa[h] = sqrt_JS(avg_qk[h], vert_blk[h]);

@@ -43,8 +43,8 @@ SIGNATURES = {
     "sp_lastq_scores_workspace_bytes": (_SZ, [_I64, _I32, _I32]),
     "sp_lastq_scores_bf16": (_I32, [_P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I32, _U32, _P, _SZ,
                                     _P, _P, _P, _P, _P]),
-    "sp_cover_count": (_I32, [_P, _I32, _I64, _F, _P, _P]),
-    "sp_cover_budgets": (_I32, [_P, _P, _I32, _I64, _I32, _F, _I32, _I32, _P, _P, _P]),
+    "sp_cover_count": (_I32, [_P, _I32, _I64, _F, _P, _P, _SZ, _P]),
+    "sp_cover_budgets": (_I32, [_P, _P, _I32, _I64, _I32, _F, _I32, _I32, _P, _P, _P, _SZ, _P]),
     "sp_queryaware_test_bf16": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I32, _U32, _F, _P, _P, _P,
                                        _P]),
     "sp_share_decide": (_I32, [_ST, _P, _I32, _I32, _P, _P, _P, _P, _P, _I32, _F, _D, _P, _P, _P, _P, _P, _P]),

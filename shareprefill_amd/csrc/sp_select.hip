@@ -18,16 +18,8 @@
 #define SEL_BINS 2048
 
 // ------------------------------------------------------------------------------------------------
-// radix mass descent (one workgroup of SEL_THREADS threads per vector)
+// radix mass descent: shared state of the per-vector pick step (one workgroup of SEL_THREADS threads)
 // ------------------------------------------------------------------------------------------------
-struct MassCut {
-  uint32_t key;        // boundary key k*: every element with key > k* is in the prefix
-  uint32_t n_equal;    // elements with key == k*
-  uint32_t n_take;     // how many of them (lowest indices first) are in the prefix
-  uint32_t n_above;    // elements with key > k*
-  int32_t all;         // 1 when the whole vector is in the prefix
-};
-
 struct SelShared {
   unsigned long long sum[SEL_BINS];
   uint32_t cnt[SEL_BINS];
@@ -50,148 +42,6 @@ __device__ static void sel_suffix_scan(SelShared& sh) {
     sh.sum[t + SEL_THREADS] += a1;
     __syncthreads();
   }
-}
-
-// One descent level: histogram the elements whose key matches `prefix` on the bits above
-// (shift+width), pick the bin in which the running mass (high keys first) first exceeds `budget`.
-// Returns false when no bin crosses (only possible at the top level).
-__device__ static bool sel_level(const float* __restrict__ x, int64_t len, uint32_t prefix, int prefix_shift,
-                                 int shift, int width, unsigned long long budget, SelShared& sh) {
-  const int t = threadIdx.x;
-  sh.sum[t] = 0;
-  sh.sum[t + SEL_THREADS] = 0;
-  sh.cnt[t] = 0;
-  sh.cnt[t + SEL_THREADS] = 0;
-  if (t == 0) {
-    sh.bin = -1;
-    sh.cnt_above = 0;
-  }
-  __syncthreads();
-  const uint32_t maskw = (1u << width) - 1u;
-  for (int64_t i = t; i < len; i += SEL_THREADS) {
-    const float v = x[i];
-    const uint32_t key = sp_sort_key(v);
-    if (prefix_shift < 32 && (key >> prefix_shift) != prefix) continue;
-    const uint32_t b = (key >> shift) & maskw;
-    atomicAdd(&sh.cnt[b], 1u);
-    const unsigned long long fx = sp_to_fixed(v);
-    if (fx) atomicAdd(&sh.sum[b], fx);
-  }
-  __syncthreads();
-  // keep the per-bin mass of the candidate bins before the scan overwrites it
-  const unsigned long long own0 = sh.sum[t], own1 = sh.sum[t + SEL_THREADS];
-  __syncthreads();
-  sel_suffix_scan(sh);
-  const int nbins = 1 << width;
-#pragma unroll
-  for (int rep = 0; rep < 2; ++rep) {
-    const int b = t + rep * SEL_THREADS;
-    if (b < nbins) {
-      const unsigned long long incl = sh.sum[b];
-      const unsigned long long excl = (b + 1 < SEL_BINS) ? sh.sum[b + 1] : 0ull;
-      if (incl > budget && excl <= budget) {
-        sh.bin = b;
-        sh.sum_above = excl;
-        sh.bin_sum = rep ? own1 : own0;
-        sh.bin_cnt = sh.cnt[b];
-      }
-    }
-  }
-  __syncthreads();
-  const int bin = sh.bin;
-  if (bin < 0) return false;
-  // count of the bins above the chosen one
-  uint32_t c = 0;
-#pragma unroll
-  for (int rep = 0; rep < 2; ++rep) {
-    const int b = t + rep * SEL_THREADS;
-    if (b < nbins && b > bin) c += sh.cnt[b];
-  }
-  if (c) atomicAdd(&sh.cnt_above, c);
-  __syncthreads();
-  return true;
-}
-
-// prefix of sort_desc(x) whose running mass stays <= budget
-__device__ static MassCut sel_mass_cut(const float* __restrict__ x, int64_t len, unsigned long long budget,
-                                       SelShared& sh) {
-  MassCut cut;
-  cut.all = 0;
-  if (!sel_level(x, len, 0u, 32, 21, 11, budget, sh)) {
-    cut.all = 1;
-    cut.key = 0;
-    cut.n_equal = 0;
-    cut.n_take = 0;
-    cut.n_above = (uint32_t)len;
-    return cut;
-  }
-  uint32_t prefix = (uint32_t)sh.bin;
-  uint32_t above = sh.cnt_above;
-  unsigned long long rem = budget - sh.sum_above;
-  __syncthreads();
-  sel_level(x, len, prefix, 21, 10, 11, rem, sh);
-  prefix = (prefix << 11) | (uint32_t)sh.bin;
-  above += sh.cnt_above;
-  rem -= sh.sum_above;
-  __syncthreads();
-  sel_level(x, len, prefix, 10, 0, 10, rem, sh);
-  cut.key = (prefix << 10) | (uint32_t)sh.bin;
-  above += sh.cnt_above;
-  rem -= sh.sum_above;
-  cut.n_equal = sh.bin_cnt;
-  cut.n_above = above;
-  const unsigned long long each = sh.bin_sum / (sh.bin_cnt ? sh.bin_cnt : 1u);
-  unsigned long long take = each ? rem / each : (unsigned long long)cut.n_equal;
-  if (take > cut.n_equal) take = cut.n_equal;
-  cut.n_take = (uint32_t)take;
-  __syncthreads();
-  return cut;
-}
-
-// ---- score_cover_topk (attn/utils.py:47-50) ---------------------------------------------------------
-__global__ __launch_bounds__(SEL_THREADS) void sp_cover_count_kernel(const float* __restrict__ x, int64_t len,
-                                                                     long long t_le, int32_t* __restrict__ out,
-                                                                     int bs, int minb, int maxb) {
-  __shared__ SelShared sh;
-  const float* v = x + (int64_t)blockIdx.x * len;
-  long long m = 0;
-  if (t_le >= 0) {
-    MassCut cut = sel_mass_cut(v, len, (unsigned long long)t_le, sh);
-    m = cut.all ? (long long)len : (long long)cut.n_above + cut.n_take;
-  }
-  if (threadIdx.x == 0) {
-    long long r = m + 1;
-    if (bs > 0) {  // budgets: tokens // bs + 1, clamped (attention_sharing.py:169-176)
-      r = r / bs + 1;
-      if (r < minb) r = minb;
-      if (r > maxb) r = maxb;
-    }
-    out[blockIdx.x] = (int32_t)r;
-  }
-}
-
-extern "C" int sp_cover_count(const float* x, int32_t n_vec, int64_t len, float thr, int32_t* out,
-                              sp_stream_t stream) {
-  SP_REQUIRE(x && out && n_vec > 0 && len > 0, SP_ERR_INVALID_ARGUMENT, "sp_cover_count: bad arguments");
-  hipLaunchKernelGGL(sp_cover_count_kernel, dim3(n_vec), dim3(SEL_THREADS), 0, (hipStream_t)stream, x, len,
-                     (long long)sp_thr_le(thr), out, 0, 0, 0);
-  SP_LAUNCH_CHECK();
-  return SP_OK;
-}
-
-extern "C" int sp_cover_budgets(const float* vert_tok, const float* slash_tok, int32_t hq, int64_t n, int32_t bs,
-                                float pattern_threshold, int32_t min_blocks, int32_t max_blocks, int32_t* nv,
-                                int32_t* ns, sp_stream_t stream) {
-  SP_REQUIRE(vert_tok && slash_tok && nv && ns && hq > 0 && n > 0 && bs > 0, SP_ERR_INVALID_ARGUMENT,
-             "sp_cover_budgets: bad arguments");
-  const long long t = (long long)sp_thr_le(pattern_threshold);
-  hipLaunchKernelGGL(sp_cover_count_kernel, dim3(hq), dim3(SEL_THREADS), 0, (hipStream_t)stream, vert_tok, n, t, nv,
-                     bs, min_blocks, max_blocks);
-  SP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sp_cover_count_kernel, dim3(hq), dim3(SEL_THREADS), 0, (hipStream_t)stream, slash_tok, n, t, ns,
-                     bs, min_blocks, max_blocks);
-  SP_LAUNCH_CHECK();
-  return SP_OK;
 }
 
 // ---- score_cover_idx (attn/utils.py:53-57) on [nb][nb] maps, written into bit masks -----------------
@@ -238,7 +88,7 @@ __global__ void sp_gsel_init_kernel(GselState* st, uint32_t* cnt, unsigned long 
     s.enabled = (gsel_enabled(enable, enable_match, v) && t_le >= 0) ? 1 : 0;
     for (int i = 0; i < 8; ++i) s.pad[i] = 0;
     st[v] = s;
-    if (gsel_enabled(enable, enable_match, v))  // block (0,0): the padding id of the reference
+    if (mask != nullptr && gsel_enabled(enable, enable_match, v))  // block (0,0): the padding id of the reference
       atomicOr(reinterpret_cast<uint32_t*>(mask + (int64_t)v * nb * nbw), 1u);
   }
 }
@@ -423,6 +273,76 @@ __global__ __launch_bounds__(SEL_THREADS) void sp_gsel_emit_ranked_kernel(const 
   }
 }
 
+// ---- score_cover_topk (attn/utils.py:47-50) on flat vectors: the same descent, the count instead of the set ----
+template <int LEVEL>
+__global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_hist_flat_kernel(const float* __restrict__ x0,
+                                                                         const float* __restrict__ x1, int n0,
+                                                                         int64_t len,
+                                                                         const GselState* __restrict__ st,
+                                                                         uint32_t* __restrict__ gcnt,
+                                                                         unsigned long long* __restrict__ gsum) {
+  __shared__ unsigned long long lsum[SEL_BINS];
+  __shared__ uint32_t lcnt[SEL_BINS];
+  const int v = blockIdx.y;
+  const GselState s = st[v];
+  if (!s.enabled || s.all) return;
+  constexpr int shift = LEVEL == 0 ? 21 : (LEVEL == 1 ? 10 : 0);
+  constexpr int width = LEVEL == 2 ? 10 : 11;
+  constexpr int pshift = LEVEL == 0 ? 32 : (LEVEL == 1 ? 21 : 10);
+  for (int i = threadIdx.x; i < SEL_BINS; i += GSEL_THREADS) {
+    lsum[i] = 0;
+    lcnt[i] = 0;
+  }
+  __syncthreads();
+  const float* xv = v < n0 ? x0 + (int64_t)v * len : x1 + (int64_t)(v - n0) * len;  // vectors n0.. live in x1
+  for (int64_t i0 = (int64_t)blockIdx.x * GSEL_THREADS; i0 < len; i0 += (int64_t)GSEL_SPLIT * GSEL_THREADS) {
+    const int64_t i = i0 + threadIdx.x;
+    bool live = i < len;
+    uint32_t b = 0;
+    unsigned long long fx = 0;
+    if (live) {
+      const float val = xv[i];
+      const uint32_t key = sp_sort_key(val);
+      live = !(pshift < 32 && (key >> (pshift & 31)) != s.prefix);
+      b = (key >> shift) & ((1u << width) - 1u);
+      fx = sp_to_fixed(val);
+    }
+    if (live) {
+      atomicAdd(&lcnt[b], 1u);
+      if (fx) atomicAdd(&lsum[b], fx);
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < (1 << width); i += GSEL_THREADS) {
+    if (lcnt[i]) atomicAdd(&gcnt[(int64_t)v * SEL_BINS + i], lcnt[i]);
+    if (lsum[i]) atomicAdd(&gsum[(int64_t)v * SEL_BINS + i], lsum[i]);
+  }
+}
+
+__global__ void sp_gsel_count_kernel(const GselState* __restrict__ st, int n_vec, long long t_le, int64_t len,
+                                     int32_t* __restrict__ out0, int32_t* __restrict__ out1, int n0, int bs,
+                                     int minb, int maxb) {
+  const int v = blockIdx.x * blockDim.x + threadIdx.x;
+  if (v >= n_vec) return;
+  const GselState s = st[v];
+  long long m = 0;
+  if (t_le >= 0) m = s.all ? (long long)len : (long long)s.above + s.n_take;
+  long long r = m + 1;
+  if (bs > 0) {  // budgets: tokens // bs + 1, clamped (attention_sharing.py:169-176)
+    r = r / bs + 1;
+    if (r < minb) r = minb;
+    if (r > maxb) r = maxb;
+  }
+  if (v < n0)
+    out0[v] = (int32_t)r;
+  else
+    out1[v - n0] = (int32_t)r;
+}
+
+static int gsel_count_run(const float* x0, const float* x1, int n0, int n_vec, int64_t len, float thr, int32_t* out0,
+                          int32_t* out1, int bs, int minb, int maxb, void* workspace, size_t workspace_bytes,
+                          hipStream_t s, const char* who);
+
 extern "C" size_t sp_cover_select_workspace_bytes(int32_t n_vec) {
   if (n_vec <= 0) return 0;
   return (size_t)n_vec * (sizeof(GselState) + SEL_BINS * (sizeof(uint32_t) + sizeof(unsigned long long)));
@@ -450,6 +370,49 @@ static int gsel_run(const float* x, const int32_t* enable, int enable_match, int
   hipLaunchKernelGGL(sp_gsel_emit_ranked_kernel, dim3(n_vec), dim3(SEL_THREADS), 0, s, x, nb, nbw, st, mask);
   SP_LAUNCH_CHECK();
   return SP_OK;
+}
+
+// vectors 0..n0-1 are rows of x0 (results to out0), vectors n0..n_vec-1 rows of x1 (results to out1)
+static int gsel_count_run(const float* x0, const float* x1, int n0, int n_vec, int64_t len, float thr, int32_t* out0,
+                          int32_t* out1, int bs, int minb, int maxb, void* workspace, size_t workspace_bytes,
+                          hipStream_t s, const char* who) {
+  SP_REQUIRE(workspace && workspace_bytes >= sp_cover_select_workspace_bytes(n_vec) && ((uintptr_t)workspace % 8) == 0,
+             SP_ERR_WORKSPACE, "%s: workspace missing, misaligned or too small", who);
+  GselState* st = reinterpret_cast<GselState*>(workspace);
+  unsigned long long* gsum = reinterpret_cast<unsigned long long*>(st + n_vec);
+  uint32_t* gcnt = reinterpret_cast<uint32_t*>(gsum + (size_t)n_vec * SEL_BINS);
+  const long long t_le = (long long)sp_thr_le(thr);
+  hipLaunchKernelGGL(sp_gsel_init_kernel, dim3(n_vec), dim3(256), 0, s, st, gcnt, gsum, (const int32_t*)nullptr, -1,
+                     n_vec, t_le, (uint64_t*)nullptr, 0, 0);
+  SP_LAUNCH_CHECK();
+  const dim3 hgrid(GSEL_SPLIT, n_vec);
+  hipLaunchKernelGGL(sp_gsel_hist_flat_kernel<0>, hgrid, dim3(GSEL_THREADS), 0, s, x0, x1, n0, len, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_pick_kernel<0>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_hist_flat_kernel<1>, hgrid, dim3(GSEL_THREADS), 0, s, x0, x1, n0, len, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_pick_kernel<1>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_hist_flat_kernel<2>, hgrid, dim3(GSEL_THREADS), 0, s, x0, x1, n0, len, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_pick_kernel<2>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_count_kernel, dim3((n_vec + 63) / 64), dim3(64), 0, s, st, n_vec, t_le, len, out0, out1, n0,
+                     bs, minb, maxb);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_cover_count(const float* x, int32_t n_vec, int64_t len, float thr, int32_t* out, void* workspace,
+                              size_t workspace_bytes, sp_stream_t stream) {
+  SP_REQUIRE(x && out && n_vec > 0 && len > 0, SP_ERR_INVALID_ARGUMENT, "sp_cover_count: bad arguments");
+  return gsel_count_run(x, x, n_vec, n_vec, len, thr, out, out, 0, 0, 0, workspace, workspace_bytes,
+                        (hipStream_t)stream, "sp_cover_count");
+}
+
+// both vectors of every head in one descent: 2*hq vectors
+extern "C" int sp_cover_budgets(const float* vert_tok, const float* slash_tok, int32_t hq, int64_t n, int32_t bs,
+                                float pattern_threshold, int32_t min_blocks, int32_t max_blocks, int32_t* nv,
+                                int32_t* ns, void* workspace, size_t workspace_bytes, sp_stream_t stream) {
+  SP_REQUIRE(vert_tok && slash_tok && nv && ns && hq > 0 && n > 0 && bs > 0, SP_ERR_INVALID_ARGUMENT,
+             "sp_cover_budgets: bad arguments");
+  return gsel_count_run(vert_tok, slash_tok, hq, 2 * hq, n, pattern_threshold, nv, ns, bs, min_blocks, max_blocks,
+                        workspace, workspace_bytes, (hipStream_t)stream, "sp_cover_budgets");
 }
 
 extern "C" int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec, int32_t nb, float score,

@@ -93,7 +93,9 @@ def cover_count(x: torch.Tensor, thr: float) -> torch.Tensor:
     lib = _lib.load()
     assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and x.is_cuda
     out = torch.empty(x.shape[0], dtype=torch.int32, device=x.device)
-    _lib.check(lib.sp_cover_count(_ptr(x), x.shape[0], x.shape[1], thr, _ptr(out), _stream()), "sp_cover_count")
+    ws = _workspace("cover_select", lib.sp_cover_select_workspace_bytes(x.shape[0]), x.device)
+    _lib.check(lib.sp_cover_count(_ptr(x), x.shape[0], x.shape[1], thr, _ptr(out), _ptr(ws), ws.numel(), _stream()),
+               "sp_cover_count")
     return out
 
 
@@ -104,8 +106,9 @@ def cover_budgets(vert_tok, slash_tok, block_size, pattern_threshold, min_blocks
     hq, n = vert_tok.shape
     nv = torch.empty(hq, dtype=torch.int32, device=vert_tok.device)
     ns = torch.empty(hq, dtype=torch.int32, device=vert_tok.device)
+    ws = _workspace("cover_select", lib.sp_cover_select_workspace_bytes(2 * hq), vert_tok.device)
     st = lib.sp_cover_budgets(_ptr(vert_tok), _ptr(slash_tok), hq, n, block_size, pattern_threshold, min_blocks,
-                              max_blocks, _ptr(nv), _ptr(ns), _stream())
+                              max_blocks, _ptr(nv), _ptr(ns), _ptr(ws), ws.numel(), _stream())
     _lib.check(st, "sp_cover_budgets")
     return nv, ns
 
