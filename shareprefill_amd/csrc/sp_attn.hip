@@ -804,8 +804,8 @@ __global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const uint64_t* __restrict__ mask,
     const int32_t* __restrict__ decision, const float2* __restrict__ rowstat, float* __restrict__ avg_attn, int64_t n,
     int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n, int64_t sk_h, int nb, int nbw, float scale_log2) {
-  __shared__ sp_bf16 Ks[AT_BS * AT_PITCH];
-  __shared__ float wred[4];
+  __shared__ __attribute__((aligned(16))) sp_bf16 Ks[AT_BS * AT_PITCH];
+  __shared__ float wred[2][4];
   const int r = nb - 1 - blockIdx.x, h = blockIdx.y;
   if (decision[h] != SP_DEC_DENSE) return;
   const int kvh = h / (hq / hkv);
@@ -830,17 +830,33 @@ __global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_kernel(
   float* arow_out = avg_attn + ((int64_t)h * nb + r) * nb;
   AtBlocks it;
   it.init(mask + ((int64_t)h * nb + r) * nbw, r);
-  for (int c = it.next(); c >= 0; c = it.next()) {
-    __syncthreads();
+  // thread t stages chunk t%16 (16 bytes) of key rows t/16, t/16+16, ...; the next block's tile is fetched into
+  // registers while the current one is used
+  at_u32x4 kr[8];
+  auto fetch = [&](int c) {
 #pragma unroll
     for (int i8 = 0; i8 < 8; ++i8) {
-      const int row = i8 * 16 + (t >> 4);
-      int64_t key = (int64_t)c * AT_BS + row;
+      int64_t key = (int64_t)c * AT_BS + i8 * 16 + (t >> 4);
       if (key > n - 1) key = n - 1;
-      *reinterpret_cast<uint4*>(&Ks[row * AT_PITCH + (t & 15) * 8]) =
-          *reinterpret_cast<const uint4*>(kh + key * sk_n + (t & 15) * 8);
+      kr[i8] = *reinterpret_cast<const at_u32x4*>(kh + key * sk_n + (t & 15) * 8);
     }
+  };
+  int c = it.next();
+  if (c >= 0) fetch(c);
+  int c_done = -1, par = 0;  // block whose wave partials wait in wred[par ^ 1]
+  const float inv_q = 1.0f / (float)valid_q;
+  while (c >= 0) {
+    __syncthreads();  // the previous block's operand reads are done, its wave partials are written
+    if (c_done >= 0 && t == 0)
+      arow_out[c_done] = ((wred[par ^ 1][0] + wred[par ^ 1][1]) + (wred[par ^ 1][2] + wred[par ^ 1][3])) * inv_q;
+#pragma unroll
+    for (int i8 = 0; i8 < 8; ++i8)
+      *reinterpret_cast<at_u32x4*>(&Ks[(i8 * 16 + (t >> 4)) * AT_PITCH + (t & 15) * 8]) = kr[i8];
     __syncthreads();
+    const int c_next = it.next();
+    if (c_next >= 0) fetch(c_next);
+    // only the diagonal block and a block that runs past the sequence end need the per-element predicate
+    const bool plain = c < r && (int64_t)(c + 1) * AT_BS <= n && valid_q == AT_BS;
     float part = 0.f;
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
@@ -851,18 +867,27 @@ __global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_kernel(
         const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + 16 * ks));
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qb[ks], acc, 0, 0, 0);
       }
+      if (plain) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key_off = kt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-        const bool ok = q_valid && (c < r || key_off <= q_off) && ((int64_t)c * AT_BS + key_off < n);
-        part += ok ? __builtin_amdgcn_exp2f(__builtin_fmaf(acc[i], scale_log2, -m_row)) * inv_l : 0.f;
+        for (int i = 0; i < 16; ++i) part += __builtin_amdgcn_exp2f(__builtin_fmaf(acc[i], scale_log2, -m_row));
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key_off = kt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+          const bool ok = q_valid && (c < r || key_off <= q_off) && ((int64_t)c * AT_BS + key_off < n);
+          part += ok ? __builtin_amdgcn_exp2f(__builtin_fmaf(acc[i], scale_log2, -m_row)) : 0.f;
+        }
       }
     }
-    part = sp_wave_sum(part);
-    if (lane == 0) wred[wave] = part;
-    __syncthreads();
-    if (t == 0) arow_out[c] = ((wred[0] + wred[1]) + (wred[2] + wred[3])) / (float)valid_q;
+    part = sp_wave_sum(part * inv_l);
+    if (lane == 0) wred[par][wave] = part;
+    c_done = c;
+    par ^= 1;
+    c = c_next;
   }
+  __syncthreads();
+  if (c_done >= 0 && t == 0)
+    arow_out[c_done] = ((wred[par ^ 1][0] + wred[par ^ 1][1]) + (wred[par ^ 1][2] + wred[par ^ 1][3])) * inv_q;
 }
 
 // ---- host ---------------------------------------------------------------------------------------------
