@@ -714,6 +714,10 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       // ---- steady state: four half-tile steps per block ----
       while (mine) {  // (mine implies c_cur >= 0)
         top();
+        // The instruction arbiter favours the older waves (the even row's), which then finish the block early and
+        // idle at the barrier while the odd row's waves run alone at half the matrix-core rate: the odd row gets
+        // priority for the first half of the block, which evens the two out.
+        if (grp) __builtin_amdgcn_s_setprio(1);
         feed(0);
         // S(previous block, keys 96..127) -> P;  S(keys 0..31) on the matrix core;  O += V^T(2b-1, keys 0..31) . P
         at_step<true, true, 0, 0, 0>(ad, vb, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
@@ -721,6 +725,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         feed(1);
         at_step<true, true, 1, 0, 1>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
                                      c_cur == r, 0, tq);
+        if (grp) __builtin_amdgcn_s_setprio(0);
         feed(2);
         at_step<true, true, 2, 1, 0>(ad, vb1, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
                                      c_cur == r, 32, tq);
