@@ -116,7 +116,7 @@ def cpu_baseline(w, q, k, v, mask_bool, decision, kept_blocks, pt):
 MEASURED_ATTN_TRAFFIC_BYTES = {("C3", 0.95): int((105.1 + 1.0) * 2 ** 30)}
 
 
-def library_gemm_tflops(dev, n=8192, reps=10):
+def library_gemm_tflops(dev, n=8192, reps=200):
     """bf16 GEMM rate of the vendor library (torch.matmul) on N(0,1) data: what a tuned dense kernel sustains on
     this chip with operands that toggle -- a calibration point beside the nominal peak, nothing the path uses."""
     import torch
@@ -377,8 +377,9 @@ def main():
                                "token_major_kv_ms": round(dec_ms, 4), "torch_sdpa_ms": round(sdpa_ms, 4)}
         del kc, vc
         # what back-to-back MFMAs alone sustain on this chip (power-managed clocks): the practical ceiling
-        line["mfma_sustained_tflops"] = {"random_operands": round(ops.mfma_probe_tflops(True), 1),
-                                         "constant_operands": round(ops.mfma_probe_tflops(False), 1),
+        line["mfma_sustained_tflops"] = {"random_operands_changing_every_instruction": round(ops.mfma_probe_tflops(2), 1),
+                                         "random_operands_held_in_registers": round(ops.mfma_probe_tflops(1), 1),
+                                         "constant_operands": round(ops.mfma_probe_tflops(0), 1),
                                          "library_gemm_8192_random_data": round(library_gemm_tflops(dev), 1),
                                          "nominal_peak": PEAK_BF16_TFLOPS}
         if args.sweep:

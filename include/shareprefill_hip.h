@@ -72,8 +72,10 @@ int sp_version(void);
 const char* sp_arch(void);       /* "gfx950" */
 const char* sp_last_error(void); /* host string, valid until the next failing call on this thread */
 /* Measurement aid (no counterpart in the reference): runs `iters` x 4 back-to-back bf16 32x32x16 MFMAs per wave on
- * every CU (8 waves per CU) with either random-valued (random_operands != 0) or constant operand registers.  The
- * caller times it; flops = sp_diag_mfma_flops(iters).  Used to calibrate the sustained matrix-core rate, which
+ * every CU (8 waves per CU).  random_operands 0: one constant in every operand element; 1: random values per lane,
+ * the same registers for every instruction (operand inputs never toggle); 2: four different random operand pairs in
+ * rotation, so both operands change with every instruction as in a real product.  The caller times it; flops =
+ * sp_diag_mfma_flops(iters).  Used to calibrate the sustained matrix-core rate under the board's power limit, which
  * depends on how much the operand bits toggle.  out: 512 floats of device scratch. */
 int sp_diag_mfma_bf16(int32_t iters, int32_t random_operands, float* out, sp_stream_t stream);
 double sp_diag_mfma_flops(int32_t iters);

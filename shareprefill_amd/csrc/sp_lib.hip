@@ -22,7 +22,6 @@ typedef __bf16 diag_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float diag_floatx16 __attribute__((ext_vector_type(16)));
 
 __global__ __launch_bounds__(512, 1) void sp_diag_mfma_kernel(float* out, int iters, int random_operands) {
-  uint4 ra, rb;
   unsigned h = (threadIdx.x * 2654435761u) ^ (blockIdx.x * 40503u) ^ 0x9e3779b9u;
   auto next = [&]() {
     h ^= h << 13;
@@ -31,14 +30,27 @@ __global__ __launch_bounds__(512, 1) void sp_diag_mfma_kernel(float* out, int it
     // two bf16 values in [0.25, 0.5) with random sign and mantissa, or one constant
     return random_operands ? ((h & 0x807F807Fu) | 0x3E803E80u) : 0x3E803E80u;
   };
-  ra = make_uint4(next(), next(), next(), next());
-  rb = make_uint4(next(), next(), next(), next());
-  const diag_bf16x8 a = __builtin_bit_cast(diag_bf16x8, ra), b = __builtin_bit_cast(diag_bf16x8, rb);
+  // random_operands 1: one random operand pair per lane, the same for every instruction (the inputs of the
+  // multipliers never toggle); 2: four different pairs in rotation, so both operands change with every
+  // instruction as they do in a real product
+  diag_bf16x8 a[4], b[4];
+  for (int u = 0; u < 4; ++u) {
+    if (u == 0 || random_operands == 2) {
+      a[u] = __builtin_bit_cast(diag_bf16x8, make_uint4(next(), next(), next(), next()));
+      b[u] = __builtin_bit_cast(diag_bf16x8, make_uint4(next(), next(), next(), next()));
+    } else {
+      a[u] = a[0];
+      b[u] = b[0];
+    }
+  }
   diag_floatx16 acc[4];
   for (int i = 0; i < 4; ++i) acc[i] = (diag_floatx16){0};
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) acc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[u], 0, 0, 0);
+    for (int u = 0; u < 4; ++u) {
+      asm volatile("" : "+v"(a[u]), "+v"(b[u]));  // four live operand pairs, no merging of equal ones
+      acc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[u], b[u], acc[u], 0, 0, 0);
+    }
   }
   float s = 0.f;
   for (int i = 0; i < 4; ++i) s += acc[i][0] + acc[i][7];

@@ -290,7 +290,7 @@ def attention_clock_mhz(n: int, hkv: int, d: int, block_size: int, device) -> fl
     return float(buf[0]) / (float(buf[1]) / 100.0) if buf[1] > 0 else float("nan")
 
 
-def mfma_probe_tflops(random_operands: bool, iters: int = 1500000, reps: int = 2) -> float:
+def mfma_probe_tflops(random_operands, iters: int = 1500000, reps: int = 2) -> float:
     """Sustained bf16 MFMA rate of back-to-back 32x32x16 MFMAs on every CU (measurement aid).  The default runs
     about 0.2 s per repetition, long enough for the clocks to settle under the load; the last repetition counts."""
     lib = _lib.load()
@@ -299,7 +299,7 @@ def mfma_probe_tflops(random_operands: bool, iters: int = 1500000, reps: int = 2
     for _ in range(reps):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record(torch.cuda.current_stream())
-        _lib.check(lib.sp_diag_mfma_bf16(iters, 1 if random_operands else 0, _ptr(out), _stream()), "sp_diag_mfma_bf16")
+        _lib.check(lib.sp_diag_mfma_bf16(iters, int(random_operands), _ptr(out), _stream()), "sp_diag_mfma_bf16")
         b.record(torch.cuda.current_stream())
         b.synchronize()
         ms = a.elapsed_time(b)
