@@ -40,6 +40,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the stage breakdown / dense baseline / sweep")
     ap.add_argument("--sweep", action="store_true", help="also time pattern_threshold 0.9 and 0.99")
+    ap.add_argument("--fuse-rope", action="store_true",
+                    help="C4 only: rotary embedding by the one-pass in-place HIP kernel instead of the model's "
+                         "elementwise kernels (bit-identical)")
     ap.add_argument("--length-sweep", default=None,
                     help="C4 only: comma-separated prompt lengths; adds TTFT per length for the SharePrefill path and for "
                          "the model's stock causal attention (torch SDPA), the protocol of eval/efficiency/latency.py")
@@ -156,7 +159,7 @@ def run_c4(args):
     torch.set_default_dtype(old)
     model.eval()
     model = SharePrefill(model_name="meta-llama/Llama-3.1-8B-Instruct", pattern_threshold=0.95, similarity_threshold=0.5,
-                         fallback_threshold=0.95, block_size=128, min_budget=1024)(model)
+                         fallback_threshold=0.95, block_size=128, min_budget=1024, fuse_rope=args.fuse_rope)(model)
     gen = torch.Generator(device=dev)
     gen.manual_seed(1238)
     ids = torch.randint(0, cfg.vocab_size, (1, args.seq_len), generator=gen, device=dev)
@@ -181,7 +184,8 @@ def run_c4(args):
             "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": f"C4: Llama-3.1-8B architecture, random-init bf16, {args.seq_len} uniform-random token "
                                    "ids, SharePrefill in all 32 layers (shipped Llama-3.1-8B-Instruct table, "
-                                   "pattern 0.95, similarity 0.5, fallback 0.95, min_budget 1024), logits_to_keep=1"},
+                                   "pattern 0.95, similarity 0.5, fallback 0.95, min_budget 1024), logits_to_keep=1",
+                       "fuse_rope": bool(args.fuse_rope)},
             "tokens_per_s": round(args.seq_len / sec, 1), "mean_block_density": round(dens, 4),
             "decisions": sharing.decision_histogram(), "finite_logits": bool(torch.isfinite(out).all())}
     if args.length_sweep:
@@ -376,6 +380,20 @@ def main():
                                "layout": "k, v [Hkv, N, D] contiguous",
                                "token_major_kv_ms": round(dec_ms, 4), "torch_sdpa_ms": round(sdpa_ms, 4)}
         del kc, vc
+        # the step in front of the layer: rotary embedding of q and k, one in-place pass against the model's
+        # elementwise evaluation (bytes = q and k read and written once)
+        from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+        cs = torch.randn(2, w.seq_len, w.head_dim, device=dev, dtype=torch.float32).clamp_(-1, 1).to(torch.bfloat16)
+        rope_bytes = 2 * (w.hq + w.hkv) * w.seq_len * w.head_dim * 2
+        qr, kr = q.clone(), k.clone()  # (same strides; the workload's own tensors stay as they are)
+        rope_ms = event_ms(lambda: ops.rope_inplace(qr[0], kr[0], cs[0], cs[1]), reps=5)
+        stock_rope = getattr(apply_rotary_pos_emb, "_shareprefill_original", apply_rotary_pos_emb)
+        with torch.no_grad():
+            rope_torch_ms = event_ms(lambda: stock_rope(qr, kr, cs[0][None], cs[1][None]), reps=3)
+        line["rope_step"] = {"ms": round(rope_ms, 4), "GBps": round(rope_bytes / rope_ms / 1e6, 1),
+                             "frac_of_hbm_peak": round(rope_bytes / rope_ms / 1e6 / PEAK_HBM_GBS, 4),
+                             "elementwise_torch_ms": round(rope_torch_ms, 4)}
+        del cs, qr, kr
         # what back-to-back MFMAs alone sustain on this chip (power-managed clocks): the practical ceiling
         line["mfma_sustained_tflops"] = {"random_operands_changing_every_instruction": round(ops.mfma_probe_tflops(2), 1),
                                          "random_operands_held_in_registers": round(ops.mfma_probe_tflops(1), 1),

@@ -202,6 +202,18 @@ int sp_decode_attn_bf16(const void* q, const void* k, const void* v, int64_t n, 
                         int64_t v_stride_h, float softmax_scale, void* out, void* workspace,
                         size_t workspace_bytes, sp_stream_t stream);
 
+/* ---- rotary position embedding in front of the attention function ---------------------------------
+ * The reference's patched model produces (cos, sin) per position (model_patch.py:121) and leaves the rotation to
+ * the Hugging Face attention layer, which evaluates  x*cos + rotate_half(x)*sin  (rotate_half(x) =
+ * cat(-x[d/2:], x[:d/2])) with five elementwise bf16 kernels per tensor.  This entry point rotates q and k in
+ * place in one pass with the same roundings (each product and the sum rounded to bf16, nearest even): the result
+ * is bit-identical to that expression for finite inputs.
+ * q: bf16 [n][hq][d], k: bf16 [n][hkv][d] (token and head strides in elements), cos_t / sin_t: bf16 [n][d] with
+ * row stride cs_stride_n.  d a multiple of 16; pointers and strides 16-byte aligned.  hq or hkv may be 0. */
+int sp_rope_inplace_bf16(void* q, void* k, const void* cos_t, const void* sin_t, int64_t n, int32_t hq, int32_t hkv,
+                         int32_t d, int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                         int64_t cs_stride_n, sp_stream_t stream);
+
 /* ---- pivot state update (attention_sharing.py:94-103, attn/utils.py:60-76) ------------------
  * For each head with decision == SP_DEC_DENSE: per-row cumulative-mass selection (>= threshold,
  * crossing entry included) of avg_attn[h] -> state.pattern, the pivot's vs_ratio

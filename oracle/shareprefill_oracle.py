@@ -33,6 +33,7 @@ Parity pins (what each function is checked against, besides the HIP path):
   csr_row_pointers ... reference docstring vector [0,5,8,9,13,14] -> [0,1,2,4,6]
   masked_attention ... torch SDPA (full mask), per-block causal attention (diagonal mask)
   decode_attention ... torch SDPA with enable_gqa; one-key and uniform-logit closed forms
+  rope_rotate ........ Hugging Face apply_rotary_pos_emb on bf16 CPU tensors (bit-exact); angle 0 / quarter turn
   layer() ............ scripted sharing scenarios (pivot / same-layer sibling / share / fallback)
 """
 
@@ -350,6 +351,21 @@ def decode_attention(q, k, v, scale):
 # --------------------------------------------------------------------------- #
 # masked attention (the fp32 output oracle) and the pivot's block-average map
 # --------------------------------------------------------------------------- #
+def rope_rotate(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x bf16 [..., N, D], cos / sin bf16 [N, D] -> x*cos + rotate_half(x)*sin, bf16.
+
+    The step in front of the attention function: the reference's patched model produces (cos, sin)
+    (shareprefill/model_patch.py:121) and the Hugging Face attention layer it patches evaluates this
+    expression with elementwise bf16 kernels, each of which computes in fp32 and rounds its result to bf16
+    (nearest even).  Restated with those three roundings written out."""
+    half = x.shape[-1] // 2
+    xf = x.float()
+    rot = torch.cat((-xf[..., half:], xf[..., :half]), dim=-1)  # negation and concatenation are exact
+    a = (xf * cos.float()).to(torch.bfloat16).float()
+    b = (rot * sin.float()).to(torch.bfloat16).float()
+    return (a + b).to(torch.bfloat16)
+
+
 def masked_attention(q, k, v, mask, bs, scale, want_avg=None):
     """fp32 causal block-sparse attention, shareprefill_attn.py:272-471.
 

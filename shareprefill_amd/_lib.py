@@ -60,6 +60,7 @@ SIGNATURES = {
     "sp_decode_workspace_bytes": (_SZ, [_I64, _I32, _I32]),
     "sp_decode_attn_bf16": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I64, _F, _P, _P, _SZ,
                                    _P]),
+    "sp_rope_inplace_bf16": (_I32, [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I64, _P]),
     "sp_pivot_update": (_I32, [_ST, _P, _P, _P, _I32, _I32, _F, _P]),
     "sp_cover_select_rows": (_I32, [_P, _I32, _F, _P, _P]),
     "sp_mask_row_pointers": (_I32, [_P, _I32, _I32, _P, _P]),

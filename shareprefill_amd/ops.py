@@ -276,6 +276,29 @@ def decode_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_
     return out
 
 
+def rope_inplace(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+    """Rotates q bf16 [Hq, N, D] and k bf16 [Hkv, N, D] (views with any token / head strides, contiguous head_dim)
+    in place by the position embeddings cos / sin bf16 [N, D]:  x <- x*cos + rotate_half(x)*sin  with the roundings
+    of the elementwise bf16 evaluation in Hugging Face's apply_rotary_pos_emb (bit-identical result).
+
+    The reference leaves this step to the attention layer it patches (position embeddings: model_patch.py:121)."""
+    lib = _lib.load()
+    _check_hnd(q, "q")
+    _check_hnd(k, "k")
+    hq, n, d = q.shape
+    hkv = k.shape[0]
+    if k.shape[1] != n or k.shape[2] != d:
+        raise ValueError(f"q {tuple(q.shape)} and k {tuple(k.shape)} must share N and D")
+    for name, t in (("cos", cos), ("sin", sin)):
+        if t.dtype != torch.bfloat16 or tuple(t.shape) != (n, d) or (n > 0 and t.stride(1) != 1) or t.device != q.device:
+            raise ValueError(f"{name} must be bfloat16 [N, D] = [{n}, {d}] with a contiguous last axis on {q.device}")
+    if n > 1 and cos.stride(0) != sin.stride(0):
+        raise ValueError("cos and sin must share their row stride")
+    st = lib.sp_rope_inplace_bf16(_ptr(q), _ptr(k), _ptr(cos), _ptr(sin), n, hq, hkv, d, q.stride(1), q.stride(0),
+                                  k.stride(1), k.stride(0), cos.stride(0) if n > 1 else d, _stream())
+    _lib.check(st, "sp_rope_inplace_bf16")
+
+
 def attention_clock_mhz(n: int, hkv: int, d: int, block_size: int, device) -> float:
     """Average shader clock (MHz) seen by workgroup 0 of the last block_sparse_attention launch on this device
     (measurement aid; synchronises the current stream)."""

@@ -5,6 +5,8 @@ Mirror of shareprefill/shareprefill_patch.py:31-169 of the reference for the ins
     and selects it through config._attn_implementation (:85-94);
   * attaches _init_attention_sharing / reset_attention_sharing / attention_sharing to the model (:96-140);
   * wraps model.forward so the sharing state is reset at every forward (:156-166).
+Beyond the reference, `SharePrefill(..., fuse_rope=True)` replaces the model module's apply_rotary_pos_emb (five
+elementwise kernels per tensor in front of the attention function) by one in-place HIP pass with identical bits.
 The reference also swaps in a copy of LlamaModel.forward that avoids the 4-D causal mask
 (model_patch.py:41-170); transformers >= 5 already passes no mask to an attention implementation that has
 no mask function registered, so nothing N x N is ever built and no forward is replaced.
@@ -16,6 +18,9 @@ import functools
 import importlib
 import logging
 
+import torch
+
+from . import ops
 from .attention_sharing import AttentionSharing
 from .shareprefill_attn import shareprefill_attention_forward
 from .shareprefill_configurations import SharePrefillConfig
@@ -46,6 +51,31 @@ class SharePrefill:
         return shareprefill_patch(model, self.config)
 
 
+def _fused_rope(original):
+    """apply_rotary_pos_emb(q, k, cos, sin, unsqueeze_dim=1) -> (q_embed, k_embed) with the rotation done in place
+    by the HIP kernel when the call has the shape the attention layer produces at inference (bf16 GPU tensors
+    [B, H, N, D] that nothing else needs, no autograd); any other call goes to the original function."""
+
+    @functools.wraps(original)
+    def apply_rotary_pos_emb(q, k, cos, sin, unsqueeze_dim=1):
+        fusable = (unsqueeze_dim == 1 and q.dim() == 4 and k.dim() == 4 and cos.dim() == 3 and q.is_cuda
+                   and q.dtype == k.dtype == cos.dtype == sin.dtype == torch.bfloat16
+                   and not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad))
+                   and q.shape[-1] % 16 == 0 and q.stride(3) == 1 and k.stride(3) == 1
+                   and cos.shape == sin.shape == (q.shape[0], q.shape[2], q.shape[3]) and k.shape[2] == q.shape[2]
+                   and cos.stride(2) == 1 and sin.stride() == cos.stride()
+                   and all(st % 8 == 0 for st in (*q.stride()[:3], *k.stride()[:3], cos.stride(1)))
+                   and all(t.data_ptr() % 16 == 0 for t in (q, k, cos, sin)))
+        if not fusable:
+            return original(q, k, cos, sin, unsqueeze_dim=unsqueeze_dim)
+        for b in range(q.shape[0]):
+            ops.rope_inplace(q[b], k[b], cos[b], sin[b])
+        return q, k
+
+    apply_rotary_pos_emb._shareprefill_original = original
+    return apply_rotary_pos_emb
+
+
 def shareprefill_patch(model, config: SharePrefillConfig):
     try:
         attention_cls = model.model.layers[0].self_attn.__class__
@@ -59,6 +89,12 @@ def shareprefill_patch(model, config: SharePrefillConfig):
         raise TypeError("Expected the attention module to define ALL_ATTENTION_FUNCTIONS for integration.")
     attention_functions["shareprefill"] = shareprefill_attention_forward
     model.config._attn_implementation = "shareprefill"
+    if config.extra.get("fuse_rope", False):
+        rope = getattr(attention_module, "apply_rotary_pos_emb", None)
+        if rope is None:
+            raise TypeError(f"fuse_rope=True: {attention_module.__name__} has no apply_rotary_pos_emb to replace")
+        if not hasattr(rope, "_shareprefill_original"):
+            attention_module.apply_rotary_pos_emb = _fused_rope(rope)
 
     def _init_attention_sharing(self):
         self.attention_sharing = AttentionSharing(config.sharing_lookup_path)

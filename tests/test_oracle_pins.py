@@ -338,6 +338,44 @@ def test_decode_attention_is_sdpa_with_gqa_and_closed_forms():
     assert not torch.allclose(out, wrong, atol=1e-3)
 
 
+def _rope_tables(n, d, theta=10000.0, dtype=torch.bfloat16):
+    inv = 1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    ang = torch.arange(n, dtype=torch.float32)[:, None] * inv[None, :]
+    emb = torch.cat((ang, ang), dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+def test_rope_rotate_is_the_hugging_face_expression_and_closed_forms():
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+
+    g = torch.Generator().manual_seed(21)
+    hq, hkv, n, d = 4, 2, 77, 32
+    q = (torch.randn(1, hq, n, d, generator=g) * 3).to(torch.bfloat16)
+    k = (torch.randn(1, hkv, n, d, generator=g) * 3).to(torch.bfloat16)
+    cos, sin = _rope_tables(n, d)
+    q_hf, k_hf = apply_rotary_pos_emb(q, k, cos[None], sin[None])  # the elementwise bf16 evaluation, on the CPU
+    assert torch.equal(O.rope_rotate(q[0], cos, sin), q_hf[0])
+    assert torch.equal(O.rope_rotate(k[0], cos, sin), k_hf[0])
+    # angle 0: identity; quarter turn (cos 0, sin 1): rotate_half itself
+    one, zero = torch.ones(n, d, dtype=torch.bfloat16), torch.zeros(n, d, dtype=torch.bfloat16)
+    assert torch.equal(O.rope_rotate(q[0], one, zero), q[0])
+    quarter = O.rope_rotate(q[0], zero, one)
+    assert torch.equal(quarter[..., : d // 2], -q[0][..., d // 2:]) and torch.equal(quarter[..., d // 2:], q[0][..., : d // 2])
+    # a rotation: the (i, i + d/2) pairs keep their length, and q.k depends on the position difference only
+    # (both within the bf16 roundings of the three steps)
+    rq = O.rope_rotate(q[0], cos, sin).float()
+    pair_len = lambda x: (x[..., : d // 2] ** 2 + x[..., d // 2:] ** 2).sqrt()
+    assert torch.allclose(pair_len(rq), pair_len(q[0].float()), rtol=2e-2, atol=2e-2)
+    x = torch.randn(d, generator=g).to(torch.bfloat16)
+    same = O.rope_rotate(x.expand(1, n, d), cos, sin).float()[0]  # the same vector at every position
+    d5 = (same[5:] * same[:-5]).sum(-1)  # <R(p+5) x, R(p) x> must not depend on p
+    assert (d5 - d5[0]).abs().max().item() < 0.05 * d5.abs().max().item() + 0.3
+    # swapping the sign of the rotation (a transposed rotate_half) must differ
+    wrong = (q[0].float() * cos.float() - torch.cat((-q[0].float()[..., d // 2:], q[0].float()[..., : d // 2]), -1)
+             * sin.float()).to(torch.bfloat16)
+    assert not torch.equal(wrong, q_hf[0])
+
+
 def test_sharing_scenarios():
     q, k, v = _toy()
     sh = O.OracleSharing(O.ClusterTable(TOY_TABLE["clusters"], TOY_TABLE["shared_clusters"]))
