@@ -153,11 +153,16 @@ def test_decide_and_mask_match_oracle_on_identical_scores(gpu_device):
 
 def test_row_pointers_docstring_vector(gpu_device):
     """shareprefill_attn.py:235-236: ids [0,5,8,9,13,14] on a 4x4 grid -> [0,1,2,4,6]."""
+    import json
+    import os
+
     from shareprefill_amd import ops
 
-    b = torch.zeros(1, 4, 4, dtype=torch.bool)
-    for i in [0, 5, 8, 9, 13, 14]:
-        b[0, i // 4, i % 4] = True
+    with open(os.path.join(os.path.dirname(__file__), "golden", "reference_docstring_vectors.json")) as f:
+        v = json.load(f)["csr_row_pointers"]
+    b = torch.zeros(1, v["grid"], v["grid"], dtype=torch.bool)
+    for i in v["block_ids"]:
+        b[0, i // v["grid"], i % v["grid"]] = True
     m = ops.bool_to_mask(b).to(gpu_device)
-    assert ops.mask_row_pointers(m).cpu().tolist() == [[0, 1, 2, 4, 6]]
-    assert ops.mask_to_block_idx(m, 4)[0].cpu().tolist() == [0, 5, 8, 9, 13, 14]
+    assert ops.mask_row_pointers(m).cpu().tolist() == [v["row_pointers"]]
+    assert ops.mask_to_block_idx(m, v["grid"])[0].cpu().tolist() == v["block_ids"]

@@ -38,10 +38,19 @@ def rand_probs(n, seed, sharp=3.0):
     return torch.softmax(torch.randn(n, generator=g) * sharp, dim=-1)
 
 
-# ----- reference docstring vectors ----------------------------------------------------------------
+# ----- reference docstring vectors (tests/golden/reference_docstring_vectors.json) ------------------
+def golden_vectors():
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(__file__), "golden", "reference_docstring_vectors.json")) as f:
+        return json.load(f)
+
+
 def test_csr_docstring_vector():
-    # shareprefill_attn.py:235-236
-    assert O.csr_row_pointers(np.array([0, 5, 8, 9, 13, 14]), 4).tolist() == [0, 1, 2, 4, 6]
+    v = golden_vectors()["csr_row_pointers"]  # shareprefill_attn.py:235-236
+    assert O.csr_row_pointers(np.array(v["block_ids"]), v["grid"]).tolist() == v["row_pointers"]
+    assert np.diff(v["row_pointers"]).tolist() == v["blocks_per_row"]
 
 
 def test_csr_ignores_padding_ids():
@@ -51,11 +60,11 @@ def test_csr_ignores_padding_ids():
 
 
 def test_flat_id_docstring_vector():
-    # shareprefill_attn.py:491-492: blocks (0,0),(1,1),(2,0),(3,1),(3,2) <-> [0,5,8,13,14]
-    m = np.zeros((4, 4), dtype=bool)
-    for r, c in [(0, 0), (1, 1), (2, 0), (3, 1), (3, 2)]:
+    v = golden_vectors()["flat_block_ids"]  # shareprefill_attn.py:491-492
+    m = np.zeros((v["grid"], v["grid"]), dtype=bool)
+    for r, c in v["blocks_row_col"]:
         m[r, c] = True
-    assert O.mask_to_ids(m).tolist() == [0, 5, 8, 13, 14]
+    assert O.mask_to_ids(m).tolist() == v["block_ids"]
 
 
 # ----- pooling --------------------------------------------------------------------------------------
