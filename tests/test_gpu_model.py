@@ -63,3 +63,34 @@ def test_patched_model_sparse_prefill_and_generate(gpu_device, tmp_path):
     with torch.no_grad():
         gen = model.generate(ids[:, :300], max_new_tokens=4, do_sample=False)
     assert gen.shape == (1, 304)
+
+
+def test_patched_qwen2_model_prefill_and_generate(gpu_device, tmp_path):
+    """The patch is model-agnostic (any module with ALL_ATTENTION_FUNCTIONS): Qwen2's attention layer passes
+    sliding_window=None for its full-attention layers and has q/k/v biases."""
+    from transformers import Qwen2Config, Qwen2ForCausalLM
+
+    from shareprefill_amd import SharePrefill
+
+    cfg = Qwen2Config(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
+                      num_key_value_heads=2, vocab_size=512, max_position_embeddings=8192, use_sliding_window=False)
+    torch.manual_seed(0)
+    ref_model = Qwen2ForCausalLM(cfg).to(gpu_device, torch.bfloat16)
+    ref_model.config._attn_implementation = "eager"
+    ids = torch.randint(0, 512, (1, 1024), generator=torch.Generator().manual_seed(4)).to(gpu_device)
+    with torch.no_grad():
+        ref = ref_model(ids).logits.float()
+    torch.manual_seed(0)
+    model = SharePrefill(sharing_lookup_path=table(tmp_path, 2, 4), min_budget=8192, fuse_rope=True)(
+        Qwen2ForCausalLM(cfg).to(gpu_device, torch.bfloat16))
+    from transformers.models.qwen2 import modeling_qwen2
+    try:
+        with torch.no_grad():
+            out = model(ids, use_cache=False).logits.float()
+            gen = model.generate(ids[:, :200], max_new_tokens=3, do_sample=False)
+    finally:
+        stock = getattr(modeling_qwen2.apply_rotary_pos_emb, "_shareprefill_original", None)
+        if stock is not None:
+            modeling_qwen2.apply_rotary_pos_emb = stock
+    assert (out - ref).abs().max().item() < 0.15 and ((out - ref).abs().mean() / ref.abs().mean()).item() < 2e-2
+    assert gen.shape == (1, 203)
