@@ -176,6 +176,12 @@ int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec,
  * SP_ATTN_V_REPACKED (the caller already repacked this v into this workspace). */
 #define SP_ATTN_V_REPACKED 1u
 size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs);
+/* Optional extra workspace per pivot head (decision == SP_DEC_DENSE with avg_attn requested): with
+ * sp_attn_workspace_bytes rounded up to 256 bytes + p * sp_attn_pivot_scratch_bytes(n, bs) bytes of workspace, the
+ * first p pivot heads (ascending head index) are processed in a launch of their own that keeps per-query block sums,
+ * and their block-average maps (shareprefill_attn.py:425-457) are made from those instead of a second pass over
+ * Q.K^T; further pivots, or all of them with the base size, take that second pass.  Same results to rounding. */
+size_t sp_attn_pivot_scratch_bytes(int64_t n, int32_t bs);
 /* Measurement aid (no counterpart in the reference): shader-clock cycles and 100 MHz wall ticks that workgroup 0
  * of the LAST sp_block_sparse_attn_fwd_bf16 launch on this workspace spent in the kernel; cycles / (ticks / 100)
  * is the average shader clock in MHz under that load.  Copies two int64 to host memory after synchronising the

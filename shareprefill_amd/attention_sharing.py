@@ -48,6 +48,7 @@ class LayerPlan:
     js_v: Optional[torch.Tensor] = None
     js_s: Optional[torch.Tensor] = None
     qa_probs: Optional[torch.Tensor] = None
+    max_pivots: int = 0         # shared clusters with a head in this layer: no more heads than that can become pivots
 
     @property
     def use_dense(self) -> torch.Tensor:
@@ -185,6 +186,8 @@ class AttentionSharing:
         qa_probs = ops.queryaware_select(qbar, kbar, decision, mask, pattern_threshold, self.flags,
                                          probs=self._qa_scratch(hq, nb, dev))
         plan = LayerPlan(layer_idx, nb, mask, decision, nv, ns, nv_f, ns_f)
+        plan.max_pivots = len({self._slot[c] for h in range(hq)
+                               for c in (self._pair_to_cluster.get((layer_idx, h)),) if c in self._slot})
         if self.keep_debug:
             plan.vert_tok, plan.slash_tok, plan.vert_blk, plan.slash_blk = vert_tok, slash_tok, vert_blk, slash_blk
             plan.kbar, plan.avg_qk, plan.js_qa, plan.js_v, plan.js_s = kbar, avg_qk, js_qa, js_v, js_s

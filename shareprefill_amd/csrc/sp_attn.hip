@@ -83,7 +83,14 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 // other queues.  Pulling is by atomic tickets only: nobody ever waits for anybody, and every workgroup leaves
 // once all eight queues are exhausted.
 #define AT_GANG 32
-#define AT_CLOCK_SLOT 192  // int index inside the 1 KiB scheduler area: {shader cycles, 100 MHz ticks} of workgroup 0
+// The 1 KiB scheduler area (int indices): 0..127 eight queue tickets (one per 64 bytes), 128..191 the pivot slot of
+// every head (one byte each, AT_NO_SLOT = its block sums are not kept), 192..195 {shader cycles, 100 MHz ticks} of
+// workgroup 0, 196 the number of pivot slots in use.
+#define AT_SLOT_TABLE 128
+#define AT_CLOCK_SLOT 192
+#define AT_NPIV_SLOT 196
+#define AT_NO_SLOT 255
+#define AT_MAX_HEADS 256
 #define AT_FWD_THREADS 512
 
 struct AtGeom {
@@ -461,11 +468,13 @@ __device__ __forceinline__ float at_pairmax(float mx) {
 // When some query's running max moves, the pending P(j-1) -- computed against the old max -- is flushed into O
 // first, O and the row sums are rescaled, and P(j-1) is cleared so that the fused stage's P.V part adds nothing.
 // The fused stage itself exists once per step: O never lives in two register sets that would have to be merged.
-template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT>
+// PIVOT: l_mark (the row sum at the start of the current key block, see the block sums of pivot heads in the
+// kernel) follows every rescale.
+template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT, bool PIVOT>
 __device__ __forceinline__ void at_step(const AtAddr& ad, const char* vbuf, int voff, const bf16x8 (&qb)[8],
                                         floatx16& s_out, floatx16& s_in, bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
                                         floatx16 (&o)[4], float scale_log2, float& m_run, float& l_lane,
-                                        float& mx_carry, bool diag, int key_base, int t) {
+                                        float& mx_carry, bool diag, int key_base, int t, float& l_mark) {
   if (diag) {  // the causal predicate changes the maximum: take it again
     at_causal(s_in, key_base, t);
     mx_carry = at_lanemax(s_in);
@@ -479,6 +488,7 @@ __device__ __forceinline__ void at_step(const AtAddr& ad, const char* vbuf, int 
     }
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_run = -inf on a row's first keys: alpha = 0
     l_lane *= alpha;
+    if constexpr (PIVOT) l_mark *= alpha;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -490,13 +500,21 @@ __device__ __forceinline__ void at_step(const AtAddr& ad, const char* vbuf, int 
   at_fused<DO_QK, HAVE_PREV, KQ, VB, KT>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, l_lane, mx_carry);
 }
 
+// PIVOT = false: every head except the pivots that have a slot in the scheduler area's table (when skip_slotted).
+// PIVOT = true: only those pivots; besides the output it leaves, per (query, key block), the softmax mass of the
+// block relative to the running max at that time as u = log2(sum) + max, from which sp_attn_avg_finish_kernel makes
+// the block-average map without recomputing any logit.  pivot_u: fp32 [slot][r*(r+1)/2 + c][128 queries].
+template <bool PIVOT>
 __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ vt,
     const uint64_t* __restrict__ mask, const int32_t* __restrict__ decision, sp_bf16* __restrict__ out,
     float2* __restrict__ rowstat, int64_t n, int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n,
-    int64_t sk_h, int nb, int nbw, float scale_log2, int* __restrict__ sched) {
+    int64_t sk_h, int nb, int nbw, float scale_log2, int* __restrict__ sched, int skip_slotted,
+    float* __restrict__ pivot_u) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // K ring (4 x 16 KiB) | V^T ring (4 x 16 KiB)
   __shared__ int s_queue, s_ticket;
+  if (PIVOT && sched[AT_NPIV_SLOT] == 0) return;  // no pivot in this layer
+  const uint8_t* const slots = reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE);
 
   const long long clk0 = clock64(), tick0 = wall_clock64();  // see sp_attn_last_launch_clocks
   AtGeom gm;
@@ -551,7 +569,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     __syncthreads();
     const int queue = __builtin_amdgcn_readfirstlane(s_queue);
     if (queue < 0) {
-      if (blockIdx.x == 0 && t == 0) {
+      if (!PIVOT && blockIdx.x == 0 && t == 0) {
         long long* clk = reinterpret_cast<long long*>(sched + AT_CLOCK_SLOT);
         clk[0] = clock64() - clk0;
         clk[1] = wall_clock64() - tick0;
@@ -561,6 +579,8 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     const int ticket = __builtin_amdgcn_readfirstlane(s_ticket);
     int h, pair;
     if (!at_item(gm, queue, ticket, h, pair)) continue;
+    const int slot = slots[h];
+    if (PIVOT ? slot == AT_NO_SLOT : (skip_slotted && slot != AT_NO_SLOT)) continue;  // the other launch's head
     const int r0 = 2 * pair;
     const bool has_b = r0 + 1 < nb;
     const int r = r0 + grp;  // this wave's row
@@ -607,6 +627,21 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) o[dt] = (floatx16){0};
     float m_run = -INFINITY, l_lane = 0.f;
+    // Pivot heads: block sums.  l_lane - l_mark is the lane's share of the softmax mass of the key block whose
+    // last half-tile has just gone through the softmax, relative to the current running max (both follow every
+    // rescale); the two lanes of a query are added and the value is kept as u = log2(sum) + m_run.
+    float l_mark = 0.f;
+    const int64_t tri_row = (int64_t)slot * ((int64_t)nb * (nb + 1) / 2) + (int64_t)r * (r + 1) / 2;
+    float* const pu = PIVOT ? pivot_u + tri_row * AT_BS : nullptr;
+    auto emit = [&](int c) {
+      if constexpr (PIVOT) {
+        const float tl = l_lane - l_mark;
+        l_mark = l_lane;
+        const float u = __builtin_amdgcn_logf(tl + __shfl_xor(tl, 32, SP_WAVE)) + m_run;
+        AT_LANE_VIEW(tq);
+        if (g == 0) pu[(int64_t)c * AT_BS + q_off] = u;
+      }
+    };
 
     // Block b of the list is processed as sub-tiles 2b and 2b+1; sub-tile s lives in ring slot s % 4 (K and V^T
     // rings alike).  One wait + barrier + issue per BLOCK: while block b is computed on (K of sub-tiles 2b, 2b+1
@@ -701,14 +736,14 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       at_qk_only<0>(kb, koff, qb, sa);
       float mx_carry = at_lanemax(sa);
       feed(1);
-      at_step<true, false, 1, 0, 0>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
-                                    c_cur == r, 0, tq);
+      at_step<true, false, 1, 0, 0, PIVOT>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+                                           c_cur == r, 0, tq, l_mark);
       feed(2);
-      at_step<true, true, 2, 1, 0>(ad, vb1, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
-                                   c_cur == r, 32, tq);
+      at_step<true, true, 2, 1, 0, PIVOT>(ad, vb1, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+                                          c_cur == r, 32, tq, l_mark);
       feed(3);
-      at_step<true, true, 3, 1, 1>(ad, vb1, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
-                                   c_cur == r, AT_SUB, tq);
+      at_step<true, true, 3, 1, 1, PIVOT>(ad, vb1, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+                                          c_cur == r, AT_SUB, tq, l_mark);
       int c_prev = c_cur;
       step_walk();
       // ---- steady state: four half-tile steps per block ----
@@ -720,18 +755,19 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         if (grp) __builtin_amdgcn_s_setprio(1);
         feed(0);
         // S(previous block, keys 96..127) -> P;  S(keys 0..31) on the matrix core;  O += V^T(2b-1, keys 0..31) . P
-        at_step<true, true, 0, 0, 0>(ad, vb, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
-                                     c_prev == r, AT_SUB + 32, tq);
+        at_step<true, true, 0, 0, 0, PIVOT>(ad, vb, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+                                            c_prev == r, AT_SUB + 32, tq, l_mark);
+        emit(c_prev);
         feed(1);
-        at_step<true, true, 1, 0, 1>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
-                                     c_cur == r, 0, tq);
+        at_step<true, true, 1, 0, 1, PIVOT>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+                                            c_cur == r, 0, tq, l_mark);
         if (grp) __builtin_amdgcn_s_setprio(0);
         feed(2);
-        at_step<true, true, 2, 1, 0>(ad, vb1, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
-                                     c_cur == r, 32, tq);
+        at_step<true, true, 2, 1, 0, PIVOT>(ad, vb1, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+                                            c_cur == r, 32, tq, l_mark);
         feed(3);
-        at_step<true, true, 3, 1, 1>(ad, vb1, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
-                                     c_cur == r, AT_SUB, tq);
+        at_step<true, true, 3, 1, 1, PIVOT>(ad, vb1, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+                                            c_cur == r, AT_SUB, tq, l_mark);
         c_prev = c_cur;
         step_walk();
       }
@@ -747,8 +783,9 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         vb = vring + ((2 * b + 3) & 3) * AT_VBUF_BYTES;
         at_block_addr(ad, kb, vb, vb, koff, voff);
       }
-      at_step<false, true, 0, 0, 0>(ad, vb, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
-                                    c_prev == r, AT_SUB + 32, tq);
+      at_step<false, true, 0, 0, 0, PIVOT>(ad, vb, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+                                           c_prev == r, AT_SUB + 32, tq, l_mark);
+      emit(c_prev);
       at_pv_only<1>(vb, voff, pb, o);
     }
     if (!finished) {
@@ -801,18 +838,75 @@ __global__ void sp_zero_i32_kernel(int* p, int count) {
   for (int i = threadIdx.x; i < count; i += blockDim.x) p[i] = 0;
 }
 
+// Before the forward launches: clears the queue tickets and gives the first max_pivots heads whose decision is
+// DENSE a slot for their block sums (ascending head order); every other head gets AT_NO_SLOT.
+__global__ void sp_attn_prep_kernel(int* __restrict__ sched, const int32_t* __restrict__ decision, int hq,
+                                    int max_pivots) {
+  for (int i = threadIdx.x; i < AT_SLOT_TABLE; i += blockDim.x) sched[i] = 0;
+  if (threadIdx.x == 0) {
+    uint8_t* slots = reinterpret_cast<uint8_t*>(sched + AT_SLOT_TABLE);
+    int cnt = 0;
+    for (int h = 0; h < hq; ++h) {
+      const bool keep = decision != nullptr && decision[h] == SP_DEC_DENSE && cnt < max_pivots;
+      slots[h] = keep ? (uint8_t)cnt++ : (uint8_t)AT_NO_SLOT;
+    }
+    sched[AT_NPIV_SLOT] = cnt;
+  }
+}
+
+// ---- pivot heads with a slot: block-averaged attention map from the block sums the forward kernel kept ----
+// avg[h][r][c] = mean over the valid queries of block r of  exp2(u[q][c] - m[q]) / l[q]  (m, l: the query's final
+// softmax statistics).  One workgroup per (query block, head); a wave takes every fourth kept block.
+__global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_finish_kernel(
+    const uint64_t* __restrict__ mask, const int* __restrict__ sched, const float2* __restrict__ rowstat,
+    const float* __restrict__ pivot_u, float* __restrict__ avg_attn, int64_t n, int nb, int nbw) {
+  const int r = nb - 1 - blockIdx.x, h = blockIdx.y;
+  const int slot = reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE)[h];
+  if (slot == AT_NO_SLOT) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t rem = n - (int64_t)r * AT_BS;
+  const int valid_q = rem < AT_BS ? (int)rem : AT_BS;
+  float m[2], inv_l[2];
+  bool ok[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int qo = lane + 64 * j;
+    ok[j] = qo < valid_q;
+    const float2 st = rowstat[(int64_t)h * n + (int64_t)r * AT_BS + (ok[j] ? qo : 0)];
+    m[j] = st.x;
+    inv_l[j] = 1.0f / st.y;
+  }
+  const float inv_q = 1.0f / (float)valid_q;
+  const float* pu = pivot_u + ((int64_t)slot * ((int64_t)nb * (nb + 1) / 2) + (int64_t)r * (r + 1) / 2) * AT_BS;
+  float* arow_out = avg_attn + ((int64_t)h * nb + r) * nb;
+  AtBlocks it;
+  it.init(mask + ((int64_t)h * nb + r) * nbw, r);
+  int idx = 0;
+  for (int c = it.next(); c >= 0; c = it.next(), ++idx) {
+    if ((idx & 3) != wave) continue;
+    const float u0 = pu[(int64_t)c * AT_BS + lane], u1 = pu[(int64_t)c * AT_BS + 64 + lane];
+    float part = ok[0] ? __builtin_amdgcn_exp2f(u0 - m[0]) * inv_l[0] : 0.f;
+    part += ok[1] ? __builtin_amdgcn_exp2f(u1 - m[1]) * inv_l[1] : 0.f;
+    part = sp_wave_sum(part);
+    if (lane == 0) arow_out[c] = part * inv_q;
+  }
+}
+
 // ---- pivot heads: block-averaged attention map (shareprefill_attn.py:425-457) ---------------------------
 // avg[h][r][c] = mean over the valid queries of block r of the softmax mass that falls into key block c,
-// recomputed from the row statistics the forward kernel left behind.  One workgroup per (query block, head);
-// heads that are not pivots leave at once.
+// recomputed from the row statistics the forward kernel left behind (the pivots for which the workspace has no
+// room to keep block sums; the others go through sp_attn_avg_finish_kernel).  One workgroup per (query block,
+// head); heads that are not such pivots leave at once.
 __global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const uint64_t* __restrict__ mask,
     const int32_t* __restrict__ decision, const float2* __restrict__ rowstat, float* __restrict__ avg_attn, int64_t n,
-    int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n, int64_t sk_h, int nb, int nbw, float scale_log2) {
+    int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n, int64_t sk_h, int nb, int nbw, float scale_log2,
+    const int* __restrict__ sched) {
   __shared__ __attribute__((aligned(16))) sp_bf16 Ks[AT_BS * AT_PITCH];
   __shared__ float wred[2][4];
   const int r = nb - 1 - blockIdx.x, h = blockIdx.y;
   if (decision[h] != SP_DEC_DENSE) return;
+  if (reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE)[h] != AT_NO_SLOT) return;  // done from its block sums
   const int kvh = h / (hq / hkv);
   const int t = threadIdx.x;
   const int wave = t >> 6, lane = t & 63;
@@ -906,6 +1000,13 @@ extern "C" size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, in
   return at_vt_bytes(n, hkv, d, bs) + 1024 + (size_t)hq * (size_t)n * sizeof(float2);
 }
 
+// block sums of one pivot head: fp32 [nb*(nb+1)/2 lower-triangular blocks][128 queries]
+extern "C" size_t sp_attn_pivot_scratch_bytes(int64_t n, int32_t bs) {
+  if (n <= 0 || bs <= 0) return 0;
+  const size_t nb = (size_t)sp_ceil_div(n, bs);
+  return nb * (nb + 1) / 2 * (size_t)bs * sizeof(float);
+}
+
 extern "C" int sp_attn_last_launch_clocks(const void* workspace, int64_t n, int32_t hkv, int32_t d, int32_t bs,
                                           int64_t* cycles_and_ticks, sp_stream_t stream) {
   SP_REQUIRE(workspace && cycles_and_ticks && n > 0 && hkv > 0 && d > 0 && bs > 0, SP_ERR_INVALID_ARGUMENT,
@@ -946,6 +1047,8 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
              "sp_block_sparse_attn_fwd_bf16: null pointer");
   SP_REQUIRE(n > 0 && hq > 0 && hkv > 0 && hq % hkv == 0, SP_ERR_INVALID_ARGUMENT,
              "sp_block_sparse_attn_fwd_bf16: bad shape n=%lld hq=%d hkv=%d", (long long)n, hq, hkv);
+  SP_REQUIRE(hq <= AT_MAX_HEADS, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: more than %d query heads",
+             AT_MAX_HEADS);
   SP_REQUIRE(softmax_scale > 0.f, SP_ERR_INVALID_ARGUMENT, "sp_block_sparse_attn_fwd_bf16: softmax_scale must be > 0");
   SP_REQUIRE(bs == AT_BS, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: block size %d unsupported (only 128)",
              bs);
@@ -972,7 +1075,19 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   float2* rowstat = reinterpret_cast<float2*>(ws + at_vt_bytes(n, hkv, d, bs) + 1024);
   const bool want_avg = decision != nullptr && avg_attn != nullptr;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_zero_i32_kernel, dim3(1), dim3(128), 0, s, counter, 8 * 16);
+  // Workspace beyond the base size holds the block sums of pivot heads, one slab per pivot: those heads run in a
+  // launch of their own that keeps the sums, and their block-average maps are made from them; pivots beyond the
+  // slabs (or all of them, with a base-size workspace) take the recomputing pass.
+  const size_t base_bytes = sp_attn_workspace_bytes(n, hq, hkv, d, bs);
+  const size_t base_aligned = (base_bytes + 255) & ~(size_t)255;
+  const size_t slab = sp_attn_pivot_scratch_bytes(n, bs);
+  int max_pivots = 0;
+  if (want_avg && workspace_bytes > base_aligned) {
+    const size_t fit = (workspace_bytes - base_aligned) / slab;
+    max_pivots = fit > (size_t)(AT_NO_SLOT - 1) ? AT_NO_SLOT - 1 : (int)fit;
+  }
+  float* pivot_u = reinterpret_cast<float*>(ws + base_aligned);
+  hipLaunchKernelGGL(sp_attn_prep_kernel, dim3(1), dim3(128), 0, s, counter, decision, (int)hq, max_pivots);
   SP_LAUNCH_CHECK();
   const size_t lds_bytes = AT_LDS_BYTES;
   static int n_cu = 0;
@@ -981,21 +1096,37 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
     hipDeviceProp_t prop;
     SP_HIP(hipGetDevice(&dev));
     SP_HIP(hipGetDeviceProperties(&prop, dev));
-    SP_HIP(hipFuncSetAttribute((const void*)sp_attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+    SP_HIP(hipFuncSetAttribute((const void*)sp_attn_fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)lds_bytes));
+    SP_HIP(hipFuncSetAttribute((const void*)sp_attn_fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)lds_bytes));
     n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
   const int64_t total = ((nb + 1) / 2) * hq;  // row pairs
   const int grid = (int)(total < (int64_t)n_cu ? ((total + 7) / 8) * 8 : (int64_t)n_cu);
-  hipLaunchKernelGGL(sp_attn_fwd_kernel, dim3(grid), dim3(AT_FWD_THREADS), lds_bytes, s, (const sp_bf16*)q,
-                     (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out,
-                     want_avg ? rowstat : (float2*)nullptr, n, hq, hkv, q_stride_n, q_stride_h, k_stride_n,
-                     k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, counter);
+  float2* stats = want_avg ? rowstat : (float2*)nullptr;
+  hipLaunchKernelGGL(sp_attn_fwd_kernel<false>, dim3(grid), dim3(AT_FWD_THREADS), lds_bytes, s, (const sp_bf16*)q,
+                     (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out, stats, n, hq, hkv,
+                     q_stride_n, q_stride_h, k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2,
+                     counter, max_pivots > 0 ? 1 : 0, (float*)nullptr);
   SP_LAUNCH_CHECK();
+  if (max_pivots > 0) {
+    hipLaunchKernelGGL(sp_zero_i32_kernel, dim3(1), dim3(128), 0, s, counter, AT_SLOT_TABLE);  // the tickets again
+    SP_LAUNCH_CHECK();
+    hipLaunchKernelGGL(sp_attn_fwd_kernel<true>, dim3(grid), dim3(AT_FWD_THREADS), lds_bytes, s, (const sp_bf16*)q,
+                       (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out, stats, n, hq,
+                       hkv, q_stride_n, q_stride_h, k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64),
+                       scale_log2, counter, 0, pivot_u);
+    SP_LAUNCH_CHECK();
+    hipLaunchKernelGGL(sp_attn_avg_finish_kernel, dim3((unsigned)nb, hq), dim3(AT_THREADS), 0, s, mask,
+                       (const int*)counter, (const float2*)rowstat, (const float*)pivot_u, avg_attn, n, (int)nb,
+                       (int)((nb + 63) / 64));
+    SP_LAUNCH_CHECK();
+  }
   if (want_avg) {
     hipLaunchKernelGGL(sp_attn_avg_kernel, dim3((unsigned)nb, hq), dim3(AT_THREADS), 0, s, (const sp_bf16*)q,
                        (const sp_bf16*)k, mask, decision, rowstat, avg_attn, n, hq, hkv, q_stride_n, q_stride_h,
-                       k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2);
+                       k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, (const int*)counter);
     SP_LAUNCH_CHECK();
   }
   return SP_OK;

@@ -224,11 +224,13 @@ def cover_select_rows(x: torch.Tensor, thr: float) -> torch.Tensor:
     return pat
 
 
-def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=None, avg_attn=None):
+def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=None, avg_attn=None, max_pivots=0):
     """q [Hq,N,D], k/v [Hkv,N,D] views, mask int64 [Hq,nb,nbw] -> out bf16 [N,Hq,D] contiguous.
 
     Reference: triton_block_wise_prefill_attention (shareprefill_attn.py:474-620).  avg_attn (fp32 [Hq,nb,nb],
-    zero-filled) receives the block-averaged attention map of the heads whose decision is DENSE."""
+    zero-filled) receives the block-averaged attention map of the heads whose decision is DENSE; max_pivots = how
+    many such heads there can be (an upper bound the host knows): the workspace then has room to keep their block
+    sums during the forward pass, which saves the second pass over Q.K^T."""
     lib = _lib.load()
     _check_hnd(q, "q")
     _check_hnd(k, "k")
@@ -240,6 +242,8 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
     dev = q.device
     out = torch.empty(n, hq, d, dtype=torch.bfloat16, device=dev)
     need = lib.sp_attn_workspace_bytes(n, hq, hkv, d, block_size)
+    if avg_attn is not None and decision is not None and max_pivots > 0:
+        need = (need + 255) // 256 * 256 + min(max_pivots, hq) * lib.sp_attn_pivot_scratch_bytes(n, block_size)
     ws = _workspace("attn_vt", need, dev)
     st = lib.sp_attn_repack_v_bf16(_ptr(v), n, hkv, d, v.stride(1), v.stride(0), block_size, _ptr(ws), ws.numel(),
                                    _stream())
@@ -250,7 +254,7 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
     st = lib.sp_block_sparse_attn_fwd_bf16(_ptr(q), _ptr(k), _ptr(v), n, hq, hkv, d, q.stride(1), q.stride(0),
                                            k.stride(1), k.stride(0), v.stride(1), v.stride(0), block_size,
                                            softmax_scale, _ptr(mask), _ptr(decision), _ptr(out), _ptr(avg_attn),
-                                           _ptr(ws), ws.numel(), _lib.SP_ATTN_V_REPACKED, _stream())
+                                           _ptr(ws), need, _lib.SP_ATTN_V_REPACKED, _stream())
     if timer is not None:
         timer.stop("attn")
     _lib.check(st, "sp_block_sparse_attn_fwd_bf16")

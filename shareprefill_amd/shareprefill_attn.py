@@ -73,8 +73,11 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
     minb, maxb = budget_blocks(config.min_budget, config.max_budget, block_size)
     plan = sharing.plan_layer(q, k, module.layer_idx, block_size, minb, maxb, config.pattern_threshold,
                               config.similarity_threshold, config.fallback_threshold, config.queryaware_threshold)
+    # room for the block sums of this layer's possible pivots (at most 16 GiB of it; pivots beyond that take the
+    # recomputing pass)
+    slab = _lib.load().sp_attn_pivot_scratch_bytes(q_len, block_size)
     out = ops.block_sparse_attention(q, k, v, plan.mask, block_size, softmax_scale, decision=plan.decision,
-                                     avg_attn=avg_attn[0])
+                                     avg_attn=avg_attn[0], max_pivots=min(plan.max_pivots, (16 << 30) // slab))
     sharing.update_pivotal_attns(module.layer_idx, avg_attn, plan.decision, config.pattern_threshold)
     return out.unsqueeze(0).transpose(1, 2), avg_attn
 

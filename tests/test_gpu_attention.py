@@ -122,6 +122,39 @@ def test_full_mask_equals_sdpa_and_avg_map(gpu_device):
     assert float(avg[1].abs().sum()) == 0.0 and float(avg[3].abs().sum()) == 0.0
 
 
+@pytest.mark.parametrize("n,max_pivots", [(1152, 2), (1152, 1), (1000, 3), (130, 2)])
+def test_pivot_maps_from_kept_block_sums_equal_the_recomputing_pass(gpu_device, n, max_pivots):
+    """With workspace for their block sums, pivot heads run in a launch of their own and their block-average
+    maps come from those sums; without it (or for pivots beyond the room) the maps are recomputed from Q.K^T.
+    Same outputs bit for bit, same maps to rounding, whatever the split; also with a pivot whose mask is not
+    the full triangle and with a ragged last block."""
+    from shareprefill_amd import ops
+
+    hq, hkv = 6, 2
+    q, k, v = _qkv(hq, hkv, n, 9)
+    nb = -(-n // 128)
+    mask = np.tril(np.ones((hq, nb, nb), bool))
+    mask[4] = _random_mask(1, nb, 5)[0]
+    mask[1] = _random_mask(1, nb, 6)[0]
+    dec = torch.tensor([O.DEC_DENSE, O.DEC_VS, O.DEC_DENSE, O.DEC_SHARE, O.DEC_DENSE, O.DEC_QA], dtype=torch.int32)
+    mdev = ops.bool_to_mask(torch.from_numpy(mask)).to(gpu_device)
+    args = (q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), mdev, 128, 0.09)
+    avg_a = torch.zeros(hq, nb, nb, dtype=torch.float32, device=gpu_device)
+    out_a = ops.block_sparse_attention(*args, decision=dec.to(gpu_device), avg_attn=avg_a)
+    avg_b = torch.zeros(hq, nb, nb, dtype=torch.float32, device=gpu_device)
+    out_b = ops.block_sparse_attention(*args, decision=dec.to(gpu_device), avg_attn=avg_b, max_pivots=max_pivots)
+    assert torch.equal(out_a, out_b)
+    assert torch.allclose(avg_a, avg_b, rtol=1e-4, atol=1e-7)
+    _, avg_ref = O.masked_attention(q, k, v, mask, 128, 0.09, want_avg=(dec == O.DEC_DENSE).numpy())
+    for h in (0, 2, 4):
+        assert torch.allclose(avg_b[h].cpu(), avg_ref[h], rtol=2e-2, atol=1e-5)
+        assert torch.allclose(avg_b[h].sum(-1).cpu(), torch.ones(nb), atol=1e-3)
+    for h in (1, 3, 5):
+        assert float(avg_b[h].abs().sum()) == 0.0
+    ref, _ = O.masked_attention(q, k, v, mask, 128, 0.09)
+    _check(out_b.transpose(0, 1).cpu(), ref)
+
+
 def test_diagonal_only_mask_is_independent_block_attention(gpu_device):
     from shareprefill_amd import ops
 
