@@ -39,7 +39,7 @@ class FakeAttention:
         self.attention_dropout = 0.0
 
 
-def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, **thr):
+def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_free=True, **thr):
     from shareprefill_amd import AttentionSharing, shareprefill_attention_forward, ops
 
     kw = dict(block_size=128, min_budget=1024, max_budget=None, pattern_threshold=0.95, similarity_threshold=0.5,
@@ -73,8 +73,10 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, **thr):
                    fallback_threshold=kw["fallback_threshold"], queryaware_threshold=kw["queryaware_threshold"])
         forced = oracle_forced.layer(q[0], k[0], v[0], layer, compute_attention=False, inject=inject, **okw)
         oracle_forced.update_pivots(layer, forced.decision, avg[0].cpu().numpy(), kw["pattern_threshold"])
-        free = oracle_free.layer(q[0], k[0], v[0], layer, compute_attention=False, **okw)
-        oracle_free.update_pivots(layer, free.decision, avg[0].cpu().numpy(), kw["pattern_threshold"])
+        free = None
+        if with_free:
+            free = oracle_free.layer(q[0], k[0], v[0], layer, compute_attention=False, **okw)
+            oracle_free.update_pivots(layer, free.decision, avg[0].cpu().numpy(), kw["pattern_threshold"])
         results.append(dict(layer=layer, out=out.cpu(), avg=avg.cpu(), plan=plan, mask=gpu_mask, dec=dec,
                             forced=forced, free=free))
     return dict(q=q[0], k=k[0], v=v[0], table=table, sharing=sharing, oracle_forced=oracle_forced,
@@ -156,6 +158,36 @@ def test_layer_c1_shape(gpu_device, tmp_path):
     check_forced(run)
     check_free(run)
     check_outputs(run)
+
+
+def test_layer_c2_shape_masks_bit_exact(gpu_device, tmp_path):
+    """B1 Hq32 Hkv8 D128 N32768 (Llama-3.1-8B head shapes, nb 256), 8 clusters of 4, two layers: budgets, decisions,
+    masks, pivot patterns and coverage ratios identical to the oracle's integer logic on the GPU's own scores.
+    (The fp32 attention oracle does not finish at this size; outputs at large sizes: tests/test_gpu_fullsize.py.)"""
+    w = synthetic.WORKLOADS["C2"]
+    run = run_layers(gpu_device, tmp_path, hq=w.hq, hkv=w.hkv, n=w.seq_len, seed=w.seed, n_clusters=w.n_clusters,
+                     with_free=False, pattern_threshold=w.pattern_threshold)
+    check_forced(run)
+    assert (run["layers"][0]["dec"] == O.DEC_DENSE).sum() == w.n_clusters
+
+
+def test_layer_c3_shape_masks_bit_exact(gpu_device, tmp_path):
+    """The benchmark's own size, B1 Hq32 Hkv8 D128 N131072 (nb 1024): same bit-exact comparison of the selection."""
+    w = synthetic.WORKLOADS["C3"]
+    run = run_layers(gpu_device, tmp_path, hq=w.hq, hkv=w.hkv, n=w.seq_len, seed=w.seed, n_clusters=w.n_clusters,
+                     with_free=False, pattern_threshold=w.pattern_threshold)
+    check_forced(run)
+    assert (run["layers"][0]["dec"] == O.DEC_DENSE).sum() == w.n_clusters
+
+
+def test_layer_c5_shape_masks_bit_exact(gpu_device, tmp_path):
+    """Qwen2.5-7B head shapes at 262144 tokens (Hq28 Hkv4, GQA 7:1, nb 2048, 4 clusters of 7): the selection scan
+    and the mask sharing at 2048 query blocks, bit-exact against the oracle's integer logic."""
+    w = synthetic.WORKLOADS["C5"]
+    run = run_layers(gpu_device, tmp_path, hq=w.hq, hkv=w.hkv, n=w.seq_len, seed=w.seed, n_clusters=w.n_clusters,
+                     with_free=False, pattern_threshold=w.pattern_threshold)
+    check_forced(run)
+    assert (run["layers"][0]["dec"] == O.DEC_DENSE).sum() == w.n_clusters
 
 
 def test_layer_sharing_and_query_aware_paths(gpu_device, tmp_path):
