@@ -1090,18 +1090,22 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   hipLaunchKernelGGL(sp_attn_prep_kernel, dim3(1), dim3(128), 0, s, counter, decision, (int)hq, max_pivots);
   SP_LAUNCH_CHECK();
   const size_t lds_bytes = AT_LDS_BYTES;
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0;
+  // per device, once: the kernels' LDS allowance and the CU count (idempotent, so a race between two host threads
+  // at worst repeats it)
+  static int cu_of_device[64] = {0};
+  int dev = 0;
+  SP_HIP(hipGetDevice(&dev));
+  SP_REQUIRE(dev >= 0 && dev < 64, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: device index %d", dev);
+  if (cu_of_device[dev] == 0) {
     hipDeviceProp_t prop;
-    SP_HIP(hipGetDevice(&dev));
     SP_HIP(hipGetDeviceProperties(&prop, dev));
     SP_HIP(hipFuncSetAttribute((const void*)sp_attn_fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)lds_bytes));
     SP_HIP(hipFuncSetAttribute((const void*)sp_attn_fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)lds_bytes));
-    n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    cu_of_device[dev] = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
+  const int n_cu = cu_of_device[dev];
   const int64_t total = ((nb + 1) / 2) * hq;  // row pairs
   const int grid = (int)(total < (int64_t)n_cu ? ((total + 7) / 8) * 8 : (int64_t)n_cu);
   float2* stats = want_avg ? rowstat : (float2*)nullptr;

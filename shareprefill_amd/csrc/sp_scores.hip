@@ -365,11 +365,14 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
                      rowstat);
   SP_LAUNCH_CHECK();
   const size_t lds_bytes = (LQ_ROWS * LQ_PITCH + 4) * sizeof(float);
-  static bool attr_set = false;
-  if (!attr_set) {
+  static bool attr_set[64] = {false};  // per device, once (idempotent)
+  int dev = 0;
+  SP_HIP(hipGetDevice(&dev));
+  SP_REQUIRE(dev >= 0 && dev < 64, SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: device index %d", dev);
+  if (!attr_set[dev]) {
     SP_HIP(hipFuncSetAttribute((const void*)sp_lastq_probs_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)lds_bytes));
-    attr_set = true;
+    attr_set[dev] = true;
   }
   const int grid_x = (int)sp_ceil_div(nb, LQ_PROB_TILES);
   hipLaunchKernelGGL(sp_lastq_probs_kernel, dim3(grid_x, hq), dim3(LQ_THREADS), lds_bytes, s, (const sp_bf16*)q,
