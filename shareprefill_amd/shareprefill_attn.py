@@ -15,8 +15,13 @@ from typing import Optional, Tuple
 
 import torch
 
+import logging
+
 from . import _lib, ops
 from .attention_sharing import budget_blocks
+
+LOGGER = logging.getLogger(__name__)
+_warned_decode = False
 
 
 def _dense_causal_mask(hq: int, nb: int, device) -> torch.Tensor:
@@ -48,6 +53,13 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
             outs = [ops.decode_attention(query_states[b, :, 0], key_states[b], value_states[b], softmax_scale)
                     for b in range(bsz)]
             return torch.stack(outs).unsqueeze(2), None
+        global _warned_decode
+        if not _warned_decode:
+            _warned_decode = True
+            LOGGER.warning("SharePrefill decode step: %s head_dim %d with %d query heads per kv head is outside the HIP "
+                           "decode kernel (bf16, head_dim 128, at most 8 per kv head); using torch's "
+                           "scaled_dot_product_attention on the GPU for this model.", query_states.dtype, head_dim,
+                           num_heads // max(hkv, 1))
         out = torch.nn.functional.scaled_dot_product_attention(
             query_states, key_states, value_states, dropout_p=0.0, is_causal=False, scale=softmax_scale,
             enable_gqa=hkv != num_heads)
