@@ -10,12 +10,11 @@ Mirror of shareprefill/attn/shareprefill_attn.py:87-184 of the reference.  Diffe
 
 from __future__ import annotations
 
+import logging
 import math
 from typing import Optional, Tuple
 
 import torch
-
-import logging
 
 from . import _lib, ops
 from .attention_sharing import budget_blocks
