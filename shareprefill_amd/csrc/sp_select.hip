@@ -230,46 +230,75 @@ __global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_emit_kernel(const float*
   }
 }
 
-// boundary group taken partially: the n_take lowest indices (row-major) of the equal-valued entries win
-__global__ __launch_bounds__(SEL_THREADS) void sp_gsel_emit_ranked_kernel(const float* __restrict__ x, int nb, int nbw,
-                                                                          const GselState* __restrict__ st,
-                                                                          uint64_t* __restrict__ mask) {
-  __shared__ uint32_t wave_cnt[SEL_THREADS / SP_WAVE];
-  __shared__ uint32_t running;
-  const int v = blockIdx.x;
+// Boundary group taken partially: the n_take lowest indices (row-major) of the equal-valued entries win.  The
+// rows are cut into GSEL_SPLIT contiguous segments: a first kernel counts each segment's members of the group, the
+// second gives every segment the count of the segments before it and ranks inside the segment only.
+__device__ static inline void gsel_segment(int nb, int seg, int& r_lo, int& r_hi) {
+  const int per = (nb + GSEL_SPLIT - 1) / GSEL_SPLIT;
+  r_lo = seg * per < nb ? seg * per : nb;
+  r_hi = r_lo + per < nb ? r_lo + per : nb;
+}
+
+__device__ static inline bool gsel_ranked_needed(const GselState& s) {
+  return s.enabled && !s.all && s.n_take != 0 && s.n_take < s.n_equal;
+}
+
+__global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_tie_count_kernel(const float* __restrict__ x, int nb,
+                                                                         const GselState* __restrict__ st,
+                                                                         uint32_t* __restrict__ tie_cnt) {
+  __shared__ uint32_t total;
+  const int v = blockIdx.y, seg = blockIdx.x;
   const GselState s = st[v];
-  if (!s.enabled || s.all || s.n_take == 0 || s.n_take >= s.n_equal) return;
-  const int64_t len = (int64_t)nb * nb;
-  const float* xv = x + (int64_t)v * len;
-  uint32_t* mv = reinterpret_cast<uint32_t*>(mask + (int64_t)v * nb * nbw);
-  if (threadIdx.x == 0) running = 0;
+  if (!gsel_ranked_needed(s)) return;
+  if (threadIdx.x == 0) total = 0;
   __syncthreads();
+  int r_lo, r_hi;
+  gsel_segment(nb, seg, r_lo, r_hi);
+  const float* xv = x + (int64_t)v * nb * nb;
+  uint32_t mine = 0;
+  for (int r = r_lo; r < r_hi; ++r)
+    for (int c = threadIdx.x; c <= r; c += GSEL_THREADS) mine += sp_sort_key(xv[(int64_t)r * nb + c]) == s.prefix;
+  if (mine) atomicAdd(&total, mine);
+  __syncthreads();
+  if (threadIdx.x == 0) tie_cnt[(int64_t)v * SEL_BINS + seg] = total;
+}
+
+__global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_emit_ranked_kernel(const float* __restrict__ x, int nb, int nbw,
+                                                                           const GselState* __restrict__ st,
+                                                                           const uint32_t* __restrict__ tie_cnt,
+                                                                           uint64_t* __restrict__ mask) {
+  __shared__ uint32_t wave_cnt[GSEL_THREADS / SP_WAVE];
+  const int v = blockIdx.y, seg = blockIdx.x;
+  const GselState s = st[v];
+  if (!gsel_ranked_needed(s)) return;
+  uint32_t running = 0;  // members of the group in front of the current chunk (uniform)
+  for (int i = 0; i < seg; ++i) running += tie_cnt[(int64_t)v * SEL_BINS + i];
+  if (running >= s.n_take) return;
+  int r_lo, r_hi;
+  gsel_segment(nb, seg, r_lo, r_hi);
+  const float* xv = x + (int64_t)v * nb * nb;
+  uint32_t* mv = reinterpret_cast<uint32_t*>(mask + (int64_t)v * nb * nbw);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int64_t base = 0; base < len; base += SEL_THREADS) {
-    const int64_t i = base + threadIdx.x;
-    bool eq = false;
-    int r = 0, c = 0;
-    if (i < len) {
-      r = (int)(i / nb);
-      c = (int)(i - (int64_t)r * nb);
-      eq = c <= r && sp_sort_key(xv[i]) == s.prefix;
-    }
-    const unsigned long long bal = __ballot(eq);
-    const uint32_t before = __popcll(bal & ((1ull << lane) - 1ull));
-    if (lane == 0) wave_cnt[wave] = __popcll(bal);
-    __syncthreads();
-    uint32_t off = running;
-    for (int w = 0; w < wave; ++w) off += wave_cnt[w];
-    if (eq && off + before < s.n_take)
-      atomicOr(&mv[((int64_t)r * nbw + (c >> 6)) * 2 + ((c >> 5) & 1)], 1u << (c & 31));
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      uint32_t tot = 0;
-      for (int w = 0; w < SEL_THREADS / SP_WAVE; ++w) tot += wave_cnt[w];
+  for (int r = r_lo; r < r_hi; ++r) {
+    for (int c0 = 0; c0 <= r; c0 += GSEL_THREADS) {  // uniform trip count: every lane votes
+      const int c = c0 + threadIdx.x;
+      const bool eq = c <= r && sp_sort_key(xv[(int64_t)r * nb + c]) == s.prefix;
+      const unsigned long long bal = __ballot(eq);
+      const uint32_t before = __popcll(bal & ((1ull << lane) - 1ull));
+      __syncthreads();  // the previous chunk's counts have been read
+      if (lane == 0) wave_cnt[wave] = __popcll(bal);
+      __syncthreads();
+      uint32_t off = running, tot = 0;
+#pragma unroll
+      for (int w = 0; w < GSEL_THREADS / SP_WAVE; ++w) {
+        if (w < wave) off += wave_cnt[w];
+        tot += wave_cnt[w];
+      }
+      if (eq && off + before < s.n_take)
+        atomicOr(&mv[((int64_t)r * nbw + (c >> 6)) * 2 + ((c >> 5) & 1)], 1u << (c & 31));
       running += tot;
+      if (running >= s.n_take) return;  // uniform
     }
-    __syncthreads();
-    if (running >= s.n_take) break;
   }
 }
 
@@ -367,7 +396,10 @@ static int gsel_run(const float* x, const int32_t* enable, int enable_match, int
   hipLaunchKernelGGL(sp_gsel_hist_kernel<2>, hgrid, dim3(GSEL_THREADS), 0, s, x, nb, st, gcnt, gsum);
   hipLaunchKernelGGL(sp_gsel_pick_kernel<2>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
   hipLaunchKernelGGL(sp_gsel_emit_kernel, hgrid, dim3(GSEL_THREADS), 0, s, x, nb, nbw, st, mask);
-  hipLaunchKernelGGL(sp_gsel_emit_ranked_kernel, dim3(n_vec), dim3(SEL_THREADS), 0, s, x, nb, nbw, st, mask);
+  // (the histogram counters are free after the last pick: the segments' tie counts go there)
+  hipLaunchKernelGGL(sp_gsel_tie_count_kernel, hgrid, dim3(GSEL_THREADS), 0, s, x, nb, st, gcnt);
+  hipLaunchKernelGGL(sp_gsel_emit_ranked_kernel, hgrid, dim3(GSEL_THREADS), 0, s, x, nb, nbw, st,
+                     (const uint32_t*)gcnt, mask);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
