@@ -176,6 +176,35 @@ def test_patched_forward_resets_state_and_has_no_cpu_path(tmp_path):
     assert len(calls) == 1
 
 
+def test_fuse_rope_replaces_the_module_function_and_leaves_other_calls_alone(tmp_path):
+    """fuse_rope=True swaps the model module's apply_rotary_pos_emb for a wrapper that takes the in-place HIP pass
+    only for bf16 GPU tensors without autograd; CPU / fp32 / autograd calls get the original function's result."""
+    from shareprefill_amd import SharePrefill
+    from transformers.models.llama import modeling_llama
+
+    stock = modeling_llama.apply_rotary_pos_emb
+    try:
+        SharePrefill(sharing_lookup_path=tiny_table(tmp_path))(tiny_llama())
+        assert modeling_llama.apply_rotary_pos_emb is stock  # off by default
+        SharePrefill(sharing_lookup_path=tiny_table(tmp_path), fuse_rope=True)(tiny_llama())
+        wrapped = modeling_llama.apply_rotary_pos_emb
+        assert wrapped is not stock and wrapped._shareprefill_original is stock
+        SharePrefill(sharing_lookup_path=tiny_table(tmp_path), fuse_rope=True)(tiny_llama())
+        assert modeling_llama.apply_rotary_pos_emb is wrapped  # not wrapped twice
+        g = torch.Generator().manual_seed(0)
+        q, k = torch.randn(1, 4, 9, 32, generator=g), torch.randn(1, 2, 9, 32, generator=g)
+        cos, sin = torch.randn(1, 9, 32, generator=g), torch.randn(1, 9, 32, generator=g)
+        for cast in (torch.float32, torch.bfloat16):
+            a = wrapped(q.to(cast), k.to(cast), cos.to(cast), sin.to(cast))
+            b = stock(q.to(cast), k.to(cast), cos.to(cast), sin.to(cast))
+            assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        qg = q.clone().requires_grad_(True)
+        out, _ = wrapped(qg, k, cos, sin)
+        assert out.requires_grad and out is not qg
+    finally:
+        modeling_llama.apply_rotary_pos_emb = stock
+
+
 def test_patch_rejects_unsupported_models_and_types(tmp_path):
     from shareprefill_amd import SharePrefill
 
