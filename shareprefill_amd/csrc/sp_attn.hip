@@ -28,9 +28,10 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define AT_PITCH 136  // bf16 elements per LDS row
 #define AT_THREADS 256
 
-// position p (0..15) inside a group of 16 keys of the repacked V^T row holds key offset at_perm(p):
-// [0-3, 8-11, 4-7, 12-15], the order in which a lane half owns the rows of a 32x32 accumulator
-__host__ __device__ static inline int at_perm(int p) { return 8 * ((p & 7) >> 2) + 4 * (p >> 3) + (p & 3); }
+// position p (0..31) inside a group of 32 keys of the repacked V^T row holds key offset at_perm32(p):
+// [0-3, 16-19, 4-7, 20-23, 8-11, 24-27, 12-15, 28-31]: lane group g of a wave owns rows 4g .. 4g+3 of both 16x16
+// S^T accumulators of a half-tile, and its P^T operand is key slots 8g .. 8g+7
+__host__ __device__ static inline int at_perm32(int p) { return 16 * ((p >> 2) & 1) + 4 * (p >> 3) + (p & 3); }
 
 // ---- V repack: v[n][hkv][d] -> vt[hkv][nb][d][128 key slots] ------------------------------------------
 __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* __restrict__ v,
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int slot = p0 + j;
-      const int key = (slot & ~15) + at_perm(slot & 15);
+      const int key = (slot & ~31) + at_perm32(slot & 31);
       const uint32_t e = tile[key * AT_PITCH + dd];
       if (j & 1)
         w[j >> 1] |= e << 16;
@@ -235,27 +236,31 @@ __device__ static inline uint64_t at_trim(uint64_t x, int wi, int r) {
 #define AT_LANE_VIEW(tv)                         \
   int tv##_o = (tv);                             \
   asm volatile("" : "+v"(tv##_o));               \
-  const int lq = tv##_o & 31, g = (tv##_o >> 5) & 1; \
-  const int q_off = (tv##_o >> 6) * 32 + lq
+  const int lq = tv##_o & 15, g = (tv##_o >> 4) & 3; \
+  const int q_off = (tv##_o >> 6) * 32 + lq /* the first of the lane's two queries; the second is 16 further */
 
 // ---- the software pipeline of one wave ------------------------------------------------------------------------
-// Keys are consumed in half-tiles of 32 (one 32x32 accumulator of S^T per wave).  For half-tile j the wave issues,
-// in ONE instruction stream,
-//     S(j+1) = K(j+1) . Q^T        8 MFMAs   (matrix core)
-//     O     += V^T(j-1) . P(j-1)   8 MFMAs   (matrix core)
-//     P(j)   = exp2(S(j)*scale - m), row sums, bf16 packing     ~56 vector instructions
-// interleaved one MFMA : one LDS operand read : three or four vector instructions.  A wave issues in order but
-// an MFMA executes for 32 cycles after it is issued, so the vector work of half-tile j runs in the shadow of the
+// A wave owns 32 queries as two 16-query tiles (qt = 0, 1) and works with v_mfma_f32_16x16x32_bf16: A 16x32, B 32x16,
+// C/D 16x16 (lane l: column l%16, rows 4*(l/16) .. +3).  Against the 32x32x16 form the same flops read and rewrite
+// only half as many accumulator registers (K = 32 per instruction), which is what the power-limited chip rewards.
+//   S^T[16 keys x 16 q] = K frag[16 keys x 32 ch] . Q^T frag[32 ch x 16 q]      4 channel steps per tile
+//   O^T[16 ch x 16 q]  += V^T frag[16 ch x 32 key slots] . P^T[32 key slots x 16 q]
+// Every LDS operand (a K or V^T fragment, 1 KiB) feeds the two query tiles.  A lane holds, per query tile, the
+// logits of keys 4g .. 4g+3 of both 16-key tiles of a half-tile (g = l/16): exactly the eight key slots 8g .. 8g+7
+// of the P^T operand once the V^T repack orders the keys that way (at_perm32), so P is the S accumulator converted
+// to bf16 in place.
+// Keys are consumed in half-tiles of 32.  For half-tile j the wave issues, in ONE instruction stream,
+//     S(j+1) = K(j+1) . Q^T        16 MFMAs  (matrix core)
+//     O     += V^T(j-1) . P(j-1)   16 MFMAs  (matrix core)
+//     P(j)   = exp2(S(j)*scale - m), row sums, bf16 packing     ~60 vector instructions
+// interleaved one LDS operand read : two MFMAs : three or four vector instructions.  A wave issues in order but
+// an MFMA executes for 16 cycles after it is issued, so the vector work of half-tile j runs in the shadow of the
 // matrix work of its neighbours; scheduling barriers pin that order.  The running max is taken before the fused
 // stage; when it moves (rare after the first tiles) the pending P(j-1) is flushed into O first, O and the row
-// sums are rescaled, and the stage runs without its P.V part.
-struct AtPipe {
-  const int* koff;  // [8] lane-constant byte offsets of the K operand chunks (k-step ks), swizzle applied
-  const int* voff;  // [4] same for V^T, index kt*2 + s
-};
-
+// sums are rescaled, and the stage runs with an empty P.
 typedef uint32_t at_u32x4 __attribute__((ext_vector_type(4)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t at_pack2(float a, float b) {
   floatx2 f;
@@ -289,12 +294,35 @@ __device__ __forceinline__ uint32_t at_lds_addr(const char* p) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
 }
 
-// LDS addresses of a block's operands, one XOR each, made once per block: K k-step ks of sub-tile 2b at ka[ks]
-// (second half of the sub-tile and sub-tile 2b+1 via immediate offsets), V^T key group j of sub-tile 2b-1 at
-// va[0][j] and of sub-tile 2b at va[1][j].
+// The MFMAs of the pipeline are written as inline assembly that accumulates IN PLACE.  Through the builtin the
+// register allocator is free to give an MFMA's result other registers than its accumulator operand, and it does so
+// for this kernel: the accumulators then change registers from step to step and every step ends in ~80 register
+// copies where the rare rescale branch joins the main path.  The compiler does not know the result latency of
+// these instructions: a vector instruction that reads an MFMA result sits at least three operand slots behind it
+// by construction, and where that is not so (at_settle_*) explicit wait states are inserted.
+__device__ __forceinline__ void at_mfma_first(floatx4& d, bf16x8 a, bf16x8 b) {  // d = a . b
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void at_mfma_acc(floatx4& d, bf16x8 a, bf16x8 b) {  // d += a . b
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+}
+// 16 wait states (a 16x16x32 MFMA takes 4 passes), tied to the registers so that nothing that reads them moves up
+__device__ __forceinline__ void at_settle_s(floatx4 (&s)[2][2]) {
+  asm volatile("s_nop 15" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]));
+}
+__device__ __forceinline__ void at_settle_o(floatx4 (&o)[8][2]) {
+  asm volatile("s_nop 15"
+               : "+v"(o[0][0]), "+v"(o[0][1]), "+v"(o[1][0]), "+v"(o[1][1]), "+v"(o[2][0]), "+v"(o[2][1]),
+                 "+v"(o[3][0]), "+v"(o[3][1]), "+v"(o[4][0]), "+v"(o[4][1]), "+v"(o[5][0]), "+v"(o[5][1]),
+                 "+v"(o[6][0]), "+v"(o[6][1]), "+v"(o[7][0]), "+v"(o[7][1]));
+}
+
+// LDS addresses of a block's operands, one XOR each, made once per block: K channel step ks of sub-tile 2b at
+// ka[ks] (key tile, second half of the sub-tile and sub-tile 2b+1 via immediate offsets), V^T key-slot half h of
+// sub-tile 2b-1 at va[0][h] and of sub-tile 2b at va[1][h] (channel tile via immediate offsets).
 struct AtAddr {
-  uint32_t ka[8];
-  uint32_t va[2][4];
+  uint32_t ka[4];
+  uint32_t va[2][2];
 };
 
 __device__ __forceinline__ void at_block_addr(AtAddr& ad, const char* kb, const char* vb, const char* vb1, int koff,
@@ -302,100 +330,127 @@ __device__ __forceinline__ void at_block_addr(AtAddr& ad, const char* kb, const 
   const uint32_t k0 = at_lds_addr(kb) + (uint32_t)koff;  // buffers are 256-byte aligned: the XOR stays inside
   const uint32_t v0 = at_lds_addr(vb) + (uint32_t)voff, v1 = at_lds_addr(vb1) + (uint32_t)voff;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) ad.ka[i] = k0 ^ (uint32_t)(i << 5);
+  for (int i = 0; i < 4; ++i) ad.ka[i] = k0 ^ (uint32_t)(i << 6);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    ad.va[0][j] = v0 ^ (uint32_t)(j << 5);
-    ad.va[1][j] = v1 ^ (uint32_t)(j << 5);
+  for (int hh = 0; hh < 2; ++hh) {
+    ad.va[0][hh] = v0 ^ (uint32_t)(hh << 6);
+    ad.va[1][hh] = v1 ^ (uint32_t)(hh << 6);
   }
 }
 
+// max(a, b, c) / max(a, b) as single instructions: through fmaxf the compiler first quiets every operand it cannot
+// prove to be no signalling NaN (v_max x, x), which the MFMA results behind inline assembly all are to it
+__device__ __forceinline__ float at_max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+__device__ __forceinline__ float at_max2(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// the lane's 16 logits of a half-tile in softmax order: query tile idx / 8, then key slots 8g .. 8g+7 of the lane
+// (key tile (idx / 4) % 2, row idx % 4); s is indexed [key tile][query tile]
+#define AT_SVAL(s, idx) (s)[((idx) >> 2) & 1][(idx) >> 3][(idx) & 3]
+
 // KQ: which 32-key quarter (0..3) of the block's two K buffers S_out is computed from; VB / KT: which V^T buffer
 // (0: sub-tile 2b-1, 1: sub-tile 2b) and which half of it P_prev belongs to.
-// Slot order: the 8 MFMAs of S_out first (one dependent chain), then the 8 of O, so that S_out is complete early
-// enough for its in-lane maximum (mx_out) to be taken in the shadow of the last slots.
+// Slot order: the 8 operand slots of S_out first (channel step outermost, so that the four accumulators take turns),
+// then the 8 of O (one channel tile each), so that S_out is complete early enough for its in-lane maxima (mx_out)
+// to be taken in the shadow of the last slots.
 template <bool DO_QK, bool DO_PV, int KQ, int VB, int KT>
-__device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[8], floatx16& s_out,
-                                         const floatx16& s_in, const bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
-                                         floatx16 (&o)[4], float sc, float neg_m, float& l_lane, float& mx_out) {
-  constexpr int NM = (DO_QK ? 8 : 0) + (DO_PV ? 8 : 0);
-  static_assert(NM == 8 || NM == 16, "a fused stage has 8 or 16 MFMAs");
-  constexpr int EPS = 16 / NM;  // softmax elements handled per MFMA slot
-  constexpr int AHEAD = 2;      // LDS operands are fetched this many slots before their MFMA
-  constexpr int MX0 = 11;       // first slot that takes part in the maximum of S_out (16-slot stages)
-  bf16x8 opnd[NM];
+__device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2],
+                                         const floatx4 (&s_in)[2][2], const bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
+                                         floatx4 (&o)[8][2], float sc, const float (&neg_m)[2], float (&l_lane)[2],
+                                         float (&mx_out)[2]) {
+  constexpr int NP = (DO_QK ? 8 : 0) + (DO_PV ? 8 : 0);  // operand slots; each holds one MFMA per query tile
+  static_assert(NP == 8 || NP == 16, "a fused stage has 8 or 16 operand slots");
+  constexpr int EPS = 16 / NP;  // softmax elements handled per operand slot
+  constexpr int AHEAD = 2;      // LDS operands are fetched this many slots before their MFMAs
+  constexpr int MX0 = 11;       // first slot that takes part in the maxima of S_out (16-slot stages)
+  bf16x8 opnd[NP];
   float x[16], e[16];
   uint32_t pk[8];
-  float mx = -INFINITY;
+  float mx[2] = {-INFINITY, -INFINITY};
   auto fetch = [&](auto kc) {
     constexpr int k = decltype(kc)::value;
     constexpr bool qk = DO_QK && k < 8;
     constexpr int i = k & 7;
-    if constexpr (qk)
-      opnd[k] = at_lds128_async<(KQ >> 1) * AT_KBUF_BYTES + (KQ & 1) * 32 * 256>(ad.ka[i]);
-    else
-      opnd[k] = at_lds128_async<(i & 3) * 32 * 128>(ad.va[VB][KT * 2 + (i >> 2)]);
+    if constexpr (qk)  // slot i: channel step i / 2, key tile i % 2
+      opnd[k] = at_lds128_async<(KQ >> 1) * AT_KBUF_BYTES + ((KQ & 1) * 32 + (i & 1) * 16) * 256>(ad.ka[i >> 1]);
+    else  // slot i: channel tile i
+      opnd[k] = at_lds128_async<i * 16 * 128>(ad.va[VB][KT]);
   };
   at_static_for<0, AHEAD>(fetch);
   AT_PIN();
-  at_static_for<0, NM>([&](auto kc) {
+  at_static_for<0, NP>([&](auto kc) {
     constexpr int k = decltype(kc)::value;
     constexpr bool qk = DO_QK && k < 8;
     constexpr int i = k & 7;
-    constexpr int in_flight_after = (NM - 1 - k) < (AHEAD - 1) ? (NM - 1 - k) : (AHEAD - 1);
+    constexpr int in_flight_after = (NP - 1 - k) < (AHEAD - 1) ? (NP - 1 - k) : (AHEAD - 1);
     AT_WAIT_LGKM(in_flight_after);  // operand k has landed
     AT_PIN();
-    if constexpr (qk) {
-      if constexpr (i == 0)
-        s_out = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[k], qb[0], (floatx16){0}, 0, 0, 0);
-      else
-        s_out = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[k], qb[i], s_out, 0, 0, 0);
-    } else {
-      o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(opnd[k], p_prev[i >> 2], o[i & 3], 0, 0, 0);
-    }
-    if constexpr (k + AHEAD < NM) fetch(std::integral_constant<int, k + AHEAD>{});
+    auto mfma = [&](auto qc) {
+      constexpr int qt = decltype(qc)::value;
+      if constexpr (qk) {
+        if constexpr ((i >> 1) == 0)
+          at_mfma_first(s_out[i & 1][qt], opnd[k], qb[qt][0]);
+        else
+          at_mfma_acc(s_out[i & 1][qt], opnd[k], qb[qt][i >> 1]);
+      } else {
+        at_mfma_acc(o[i][qt], opnd[k], p_prev[qt]);
+      }
+    };
+    mfma(std::integral_constant<int, 0>{});
+    if constexpr (k + AHEAD < NP) fetch(std::integral_constant<int, k + AHEAD>{});
 #pragma unroll
     for (int u = 0; u < EPS; ++u) {
       const int idx = k * EPS + u;
       // The softmax arithmetic depends only on values known before the stage starts, and the optimiser would
       // otherwise move all of it in front of the stage (out of the MFMAs' shadow): the empty asm ties each
       // element to its slot.
-      float sv = s_in[idx];
+      float sv = AT_SVAL(s_in, idx);
       asm volatile("" : "+v"(sv));
-      x[idx] = __builtin_fmaf(sv, sc, neg_m);
+      x[idx] = __builtin_fmaf(sv, sc, neg_m[idx >> 3]);
       if (idx >= 1) e[idx - 1] = __builtin_amdgcn_exp2f(x[idx - 1]);
       if (idx >= 3 && ((idx - 3) & 1) == 0) {
         const int m = (idx - 3) >> 1;
         pk[m] = at_pack2(e[idx - 3], e[idx - 2]);
-        l_lane += e[idx - 3];
-        l_lane += e[idx - 2];
+        l_lane[(idx - 3) >> 3] += e[idx - 3];
+        l_lane[(idx - 3) >> 3] += e[idx - 2];
       }
       // ... and the results to the slot they were produced in (instruction selection lets pure arithmetic float)
       asm volatile("" : "+v"(x[idx]));
       if (idx >= 1) asm volatile("" : "+v"(e[idx - 1]));
-      if (idx >= 3 && ((idx - 3) & 1) == 0) asm volatile("" : "+v"(pk[(idx - 3) >> 1]), "+v"(l_lane));
+      if (idx >= 3 && ((idx - 3) & 1) == 0) asm volatile("" : "+v"(pk[(idx - 3) >> 1]), "+v"(l_lane[(idx - 3) >> 3]));
     }
-    if constexpr (DO_QK && DO_PV && k >= MX0) {  // three elements of S_out per slot; the last slot takes four
-      constexpr int j0 = (k - MX0) * 3;
-      mx = fmaxf(mx, fmaxf(s_out[j0], s_out[j0 + 1]));
-      mx = fmaxf(mx, s_out[j0 + 2]);
-      if constexpr (k == NM - 1) {
-        static_assert(j0 + 3 == 15, "the maximum must cover all 16 elements");
-        mx = fmaxf(mx, s_out[15]);
-      }
-      asm volatile("" : "+v"(mx));
+    AT_PIN();
+    mfma(std::integral_constant<int, 1>{});
+    if constexpr (DO_QK && DO_PV && k >= MX0 && k < MX0 + 4) {  // two elements of S_out per query tile and slot
+      constexpr int j0 = (k - MX0) * 2;
+      mx[0] = at_max3(mx[0], AT_SVAL(s_out, j0), AT_SVAL(s_out, j0 + 1));
+      mx[1] = at_max3(mx[1], AT_SVAL(s_out, 8 + j0), AT_SVAL(s_out, 8 + j0 + 1));
+      static_assert(MX0 + 4 <= NP, "the maxima must cover all 16 elements");
+      asm volatile("" : "+v"(mx[0]), "+v"(mx[1]));
     }
     AT_PIN();
   });
   e[15] = __builtin_amdgcn_exp2f(x[15]);
   pk[7] = at_pack2(e[14], e[15]);
-  l_lane += e[14];
-  l_lane += e[15];
-  if constexpr (DO_QK && !DO_PV) {  // start of a run: nothing to hide the maximum behind
+  l_lane[1] += e[14];
+  l_lane[1] += e[15];
+  if constexpr (DO_QK && !DO_PV) {  // start of a run: nothing to hide the maxima behind
+    at_settle_s(s_out);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_out[i]);
+    for (int j = 0; j < 8; j += 2) {
+      mx[0] = at_max3(mx[0], AT_SVAL(s_out, j), AT_SVAL(s_out, j + 1));
+      mx[1] = at_max3(mx[1], AT_SVAL(s_out, 8 + j), AT_SVAL(s_out, 8 + j + 1));
+    }
   }
-  mx_out = mx;
+  mx_out[0] = mx[0];
+  mx_out[1] = mx[1];
   at_u32x4 w0, w1;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -408,95 +463,130 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[8]
 
 // MFMA-only stages (no vector work to hide): first S of a row, flush of a pending P, last P.V of a row
 template <int KH>
-__device__ __forceinline__ void at_qk_only(const char* kb, int koff, const bf16x8 (&qb)[8], floatx16& s_out) {
-  bf16x8 a[8];
+__device__ __forceinline__ void at_qk_only(const char* kb, int koff, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2]) {
+  bf16x8 a[8];  // slot i: channel step i / 2, key tile i % 2
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) a[ks] = at_lds128(kb + (koff ^ (ks << 5)) + KH * 32 * 256);
-  AT_PIN();
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks) {
-    if (ks + 4 < 8) a[ks + 4] = at_lds128(kb + (koff ^ ((ks + 4) << 5)) + KH * 32 * 256);
-    if (ks == 0)
-      s_out = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qb[0], (floatx16){0}, 0, 0, 0);
-    else
-      s_out = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], qb[ks], s_out, 0, 0, 0);
-    AT_PIN();
-  }
-}
-
-template <int KT>
-__device__ __forceinline__ void at_pv_only(const char* vb, int voff, const bf16x8 (&p)[2], floatx16 (&o)[4]) {
-  bf16x8 a[8];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) a[i] = at_lds128(vb + (voff ^ ((KT * 2 + (i >> 2)) << 5)) + (i & 3) * 32 * 128);
+  for (int i = 0; i < 4; ++i) a[i] = at_lds128(kb + (koff ^ ((i >> 1) << 6)) + (KH * 32 + (i & 1) * 16) * 256);
   AT_PIN();
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    if (i + 4 < 8) a[i + 4] = at_lds128(vb + (voff ^ ((KT * 2 + ((i + 4) >> 2)) << 5)) + ((i + 4) & 3) * 32 * 128);
-    o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], p[i >> 2], o[i & 3], 0, 0, 0);
+    if (i + 4 < 8) a[i + 4] = at_lds128(kb + (koff ^ (((i + 4) >> 1) << 6)) + (KH * 32 + (i & 1) * 16) * 256);
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      if ((i >> 1) == 0)
+        at_mfma_first(s_out[i & 1][qt], a[i], qb[qt][0]);
+      else
+        at_mfma_acc(s_out[i & 1][qt], a[i], qb[qt][i >> 1]);
+    }
+    AT_PIN();
+  }
+  at_settle_s(s_out);
+}
+
+template <int KT>
+__device__ __forceinline__ void at_pv_only(const char* vb, int voff, const bf16x8 (&p)[2], floatx4 (&o)[8][2]) {
+  bf16x8 a[8];  // slot i: channel tile i
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a[i] = at_lds128(vb + (voff ^ (KT << 6)) + i * 16 * 128);
+  AT_PIN();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if (i + 4 < 8) a[i + 4] = at_lds128(vb + (voff ^ (KT << 6)) + (i + 4) * 16 * 128);
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) at_mfma_acc(o[i][qt], a[i], p[qt]);
     AT_PIN();
   }
 }
 
 // causal predicate inside the diagonal block; key_base = offset of the half-tile's first key inside the block
-__device__ __forceinline__ void at_causal(floatx16& s, int key_base, int t) {
+__device__ __forceinline__ void at_causal(floatx4 (&s)[2][2], int key_base, int t) {
   AT_LANE_VIEW(t);
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int key_off = key_base + 8 * (i >> 2) + 4 * g + (i & 3);
-    s[i] = (key_off <= q_off) ? s[i] : -INFINITY;
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int key_off = key_base + kt * 16 + 4 * g + j;
+        s[kt][qt][j] = (key_off <= q_off + qt * 16) ? s[kt][qt][j] : -INFINITY;
+      }
+}
+
+// max over the lane's 8 keys of each query tile
+__device__ __forceinline__ void at_lanemax(const floatx4 (&s)[2][2], float (&mx)[2]) {
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    float m = at_max3(s[0][qt][0], s[0][qt][1], s[0][qt][2]);
+    m = at_max3(m, s[0][qt][3], s[1][qt][0]);
+    m = at_max3(m, s[1][qt][1], s[1][qt][2]);
+    mx[qt] = at_max2(m, s[1][qt][3]);
   }
 }
 
-// max over the lane's 16 keys
-__device__ __forceinline__ float at_lanemax(const floatx16& s) {
-  float mx = s[0];
-#pragma unroll
-  for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
-  return mx;
+// ... and over the three partner lanes (lane ^ 16, ^ 32, ^ 48) that hold the other 24 keys of the query
+__device__ __forceinline__ float at_groupmax(float mx) {
+  uint32_t u = __builtin_bit_cast(uint32_t, mx);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);  // (own, lane ^ 16) in some order
+  const float m1 = at_max2(__builtin_bit_cast(float, (uint32_t)a[0]), __builtin_bit_cast(float, (uint32_t)a[1]));
+  u = __builtin_bit_cast(uint32_t, m1);
+  const auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // (own, lane ^ 32) in some order
+  return at_max2(__builtin_bit_cast(float, (uint32_t)b[0]), __builtin_bit_cast(float, (uint32_t)b[1]));
+}
+__device__ __forceinline__ float at_groupsum(float x) {
+  uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float s1 = __builtin_bit_cast(float, (uint32_t)a[0]) + __builtin_bit_cast(float, (uint32_t)a[1]);
+  u = __builtin_bit_cast(uint32_t, s1);
+  const auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (uint32_t)b[0]) + __builtin_bit_cast(float, (uint32_t)b[1]);
 }
 
-// ... and over the partner lane (lane ^ 32) that holds the other 16 keys of the query
-__device__ __forceinline__ float at_pairmax(float mx) {
-  const uint32_t u = __builtin_bit_cast(uint32_t, mx);
-  const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // (lower half's value, upper half's value)
-  return fmaxf(__builtin_bit_cast(float, (uint32_t)sw[0]), __builtin_bit_cast(float, (uint32_t)sw[1]));
-}
-
-// One pipeline step.  s_in = S(j) (complete) with in-lane maximum mx_carry, p_prev = P(j-1) not yet applied to O
-// (HAVE_PREV); on return mx_carry is the in-lane maximum of s_out.
+// One pipeline step.  s_in = S(j) (complete) with in-lane maxima mx_carry, p_prev = P(j-1) not yet applied to O
+// (HAVE_PREV); on return mx_carry holds the in-lane maxima of s_out.
 // When some query's running max moves, the pending P(j-1) -- computed against the old max -- is flushed into O
 // first, O and the row sums are rescaled, and P(j-1) is cleared so that the fused stage's P.V part adds nothing.
 // The fused stage itself exists once per step: O never lives in two register sets that would have to be merged.
-// PIVOT: l_mark (the row sum at the start of the current key block, see the block sums of pivot heads in the
+// PIVOT: l_mark (the row sums at the start of the current key block, see the block sums of pivot heads in the
 // kernel) follows every rescale.
 template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT, bool PIVOT>
-__device__ __forceinline__ void at_step(const AtAddr& ad, const char* vbuf, int voff, const bf16x8 (&qb)[8],
-                                        floatx16& s_out, floatx16& s_in, bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
-                                        floatx16 (&o)[4], float scale_log2, float& m_run, float& l_lane,
-                                        float& mx_carry, bool diag, int key_base, int t, float& l_mark) {
-  if (diag) {  // the causal predicate changes the maximum: take it again
+__device__ __forceinline__ void at_step(const AtAddr& ad, const char* vbuf, int voff, const bf16x8 (&qb)[2][4],
+                                        floatx4 (&s_out)[2][2], floatx4 (&s_in)[2][2], bf16x8 (&p_prev)[2],
+                                        bf16x8 (&p_out)[2], floatx4 (&o)[8][2], float scale_log2, float (&m_run)[2],
+                                        float (&l_lane)[2], float (&mx_carry)[2], bool diag, int key_base, int t,
+                                        float (&l_mark)[2]) {
+  if (diag) {  // the causal predicate changes the maxima: take them again
     at_causal(s_in, key_base, t);
-    mx_carry = at_lanemax(s_in);
+    at_lanemax(s_in, mx_carry);
   }
-  const float m_new = fmaxf(m_run, at_pairmax(mx_carry) * scale_log2);
-  if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {  // some row's max moved
+  // A row's max moves only if one of its four lanes saw a logit above it: one comparison per lane and a ballot
+  // decide; the exchange between the lanes runs only then.
+  const float c0 = mx_carry[0] * scale_log2, c1 = mx_carry[1] * scale_log2;
+  if (__builtin_amdgcn_ballot_w64(c0 > m_run[0] || c1 > m_run[1]) != 0ull) {  // some row's max moved
+    const float m_new0 = at_max2(m_run[0], at_groupmax(c0));
+    const float m_new1 = at_max2(m_run[1], at_groupmax(c1));
     if (HAVE_PREV) {
       at_pv_only<KT>(vbuf, voff, p_prev, o);
       p_prev[0] = __builtin_bit_cast(bf16x8, (at_u32x4){0, 0, 0, 0});
       p_prev[1] = p_prev[0];
     }
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // m_run = -inf on a row's first keys: alpha = 0
-    l_lane *= alpha;
-    if constexpr (PIVOT) l_mark *= alpha;
+    at_settle_o(o);
+    // m_run = -inf on a row's first keys: alpha = 0
+    const float alpha[2] = {__builtin_amdgcn_exp2f(m_run[0] - m_new0), __builtin_amdgcn_exp2f(m_run[1] - m_new1)};
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int qt = 0; qt < 2; ++qt) {
+      l_lane[qt] *= alpha[qt];
+      if constexpr (PIVOT) l_mark[qt] *= alpha[qt];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
-    m_run = m_new;
+      for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[dt][qt][j] *= alpha[qt];
+    }
+    at_settle_o(o);
+    m_run[0] = m_new0;
+    m_run[1] = m_new1;
   }
   // a query with nothing unmasked so far keeps m_run = -inf; exp2(-inf - (-inf)) must not be evaluated
-  const float neg_m = (m_run == -INFINITY) ? 0.f : -m_run;
+  const float neg_m[2] = {(m_run[0] == -INFINITY) ? 0.f : -m_run[0], (m_run[1] == -INFINITY) ? 0.f : -m_run[1]};
   at_fused<DO_QK, HAVE_PREV, KQ, VB, KT>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, l_lane, mx_carry);
 }
 
@@ -529,19 +619,19 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
   const int grp = wave >> 2;                                 // which row of the pair this wave works on
   const int tq = t & 255;                                    // thread index inside the row's four waves
 
-  // Lane-constant LDS read offsets (bytes) inside a buffer.  With lq = lane % 32 (the lane's row in a 32-row
-  // operand tile) and g = lane / 32, the XOR swizzle makes the operand of k-step ks (K) or of key group j (V^T)
-  // sit at (offset ^ (index << 5)):
-  //   K  : row lq (+32 via immediate), logical chunk 2*ks + g      -> lq*256 + (((2*ks + g) ^ (lq & 15)) << 4)
-  //   V^T: row lq (+32*dt via immediate), logical chunk 2*j + g    -> lq*128 + (((2*j + g) ^ ((lq >> 1) & 7)) << 4)
+  // Lane-constant LDS read offsets (bytes) inside a buffer.  With lq = lane % 16 (the lane's row in a 16-row
+  // operand tile) and g = lane / 16, the XOR swizzle makes the operand of channel step ks (K) or of key-slot half h
+  // (V^T) sit at (offset ^ (index << 6)):
+  //   K  : row lq (+16, +32 via immediate), logical chunk 4*ks + g  -> lq*256 + (((4*ks + g) ^ lq) << 4)
+  //   V^T: row lq (+16*dt via immediate), logical chunk 4*h + g     -> lq*128 + (((4*h + g) ^ ((lq >> 1) & 7)) << 4)
   // Only these, the two global load offsets and tq stay in registers across the key loop; everything else that
   // depends on the lane is recomputed where it is needed from an opaque copy of tq (AT_LANE_VIEW), so that the
   // compiler does not carry a dozen precomputed lane constants through the loop.
   int koff, voff;
   AtLoadOffsets lo;
   {
-    const int lane = t & 63, lq = lane & 31, g = lane >> 5;
-    koff = lq * 256 + ((g ^ (lq & 15)) << 4);
+    const int lane = t & 63, lq = lane & 15, g = lane >> 4;
+    koff = lq * 256 + ((g ^ lq) << 4);
     voff = lq * 128 + ((g ^ ((lq >> 1) & 7)) << 4);
     at_load_offsets(lo, sk_n, wave, lane);
   }
@@ -611,35 +701,43 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     }
     __syncthreads();
 
-    // Q^T operand: this lane's query, 8 k-steps of 8 channels
-    bf16x8 qb[8];
+    // Q^T operands: the lane's two queries (one per 16-query tile), 4 channel steps of 8 channels each
+    bf16x8 qb[2][4];
     {
       AT_LANE_VIEW(tq);
-      int64_t qrow = (int64_t)r * AT_BS + q_off;
-      if (qrow > n - 1) qrow = n - 1;
-      const sp_bf16* src = q + (int64_t)h * sq_h + qrow * sq_n + 8 * g;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
-        qb[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 16 * ks));
+      for (int qt = 0; qt < 2; ++qt) {
+        int64_t qrow = (int64_t)r * AT_BS + q_off + qt * 16;
+        if (qrow > n - 1) qrow = n - 1;
+        const sp_bf16* src = q + (int64_t)h * sq_h + qrow * sq_n + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+          qb[qt][ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 32 * ks));
+      }
     }
 
-    floatx16 o[4];
+    floatx4 o[8][2];  // [channel tile][query tile]
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) o[dt] = (floatx16){0};
-    float m_run = -INFINITY, l_lane = 0.f;
+    for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) o[dt][qt] = (floatx4){0, 0, 0, 0};
+    float m_run[2] = {-INFINITY, -INFINITY}, l_lane[2] = {0.f, 0.f};
     // Pivot heads: block sums.  l_lane - l_mark is the lane's share of the softmax mass of the key block whose
     // last half-tile has just gone through the softmax, relative to the current running max (both follow every
-    // rescale); the two lanes of a query are added and the value is kept as u = log2(sum) + m_run.
-    float l_mark = 0.f;
+    // rescale); the four lanes of a query are added and the value is kept as u = log2(sum) + m_run.
+    float l_mark[2] = {0.f, 0.f};
     const int64_t tri_row = (int64_t)slot * ((int64_t)nb * (nb + 1) / 2) + (int64_t)r * (r + 1) / 2;
     float* const pu = PIVOT ? pivot_u + tri_row * AT_BS : nullptr;
     auto emit = [&](int c) {
       if constexpr (PIVOT) {
-        const float tl = l_lane - l_mark;
-        l_mark = l_lane;
-        const float u = __builtin_amdgcn_logf(tl + __shfl_xor(tl, 32, SP_WAVE)) + m_run;
         AT_LANE_VIEW(tq);
-        if (g == 0) pu[(int64_t)c * AT_BS + q_off] = u;
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+          const float tl = l_lane[qt] - l_mark[qt];
+          l_mark[qt] = l_lane[qt];
+          const float u = __builtin_amdgcn_logf(at_groupsum(tl)) + m_run[qt];
+          if (g == 0) pu[(int64_t)c * AT_BS + q_off + qt * 16] = u;
+        }
       }
     };
 
@@ -729,12 +827,13 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         step_walk();
         continue;
       }
-      floatx16 sa, sb;
-      bf16x8 pa[2], pb[2];
+      floatx4 sa[2][2], sb[2][2];  // [key tile][query tile]
+      bf16x8 pa[2], pb[2];         // [query tile]
+      float mx_carry[2];
       // ---- start of a run: S of the first half-tile, nothing to overlap with yet ----
       feed(0);
       at_qk_only<0>(kb, koff, qb, sa);
-      float mx_carry = at_lanemax(sa);
+      at_lanemax(sa, mx_carry);
       feed(1);
       at_step<true, false, 1, 0, 0, PIVOT>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
                                            c_cur == r, 0, tq, l_mark);
@@ -792,32 +891,35 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       AT_WAIT_VMCNT0();
       __syncthreads();
     }
-    const float l_tot = l_lane + __shfl_xor(l_lane, 32, SP_WAVE);
+    at_settle_o(o);
+    const float l_tot[2] = {at_groupsum(l_lane[0]), at_groupsum(l_lane[1])};
     AT_LANE_VIEW(tq);
 
     // pivot heads: keep the softmax statistics of every query row for the block-average pass
     if (row_ok && rowstat != nullptr && decision != nullptr && decision[h] == SP_DEC_DENSE && g == 0) {
-      const int64_t qrow = (int64_t)r * AT_BS + q_off;
-      if (qrow < n) rowstat[(int64_t)h * n + qrow] = make_float2(m_run, l_tot);
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        const int64_t qrow = (int64_t)r * AT_BS + q_off + qt * 16;
+        if (qrow < n) rowstat[(int64_t)h * n + qrow] = make_float2(m_run[qt], l_tot[qt]);
+      }
     }
 
     // ---- epilogue: normalise, transpose through LDS (padded rows, one region per row), coalesced bf16 store ----
     __syncthreads();
     sp_bf16* stage_out = reinterpret_cast<sp_bf16*>(lds) + grp * (AT_BS * AT_PITCH);
-    {
-      const float inv_l = 1.0f / l_tot;
-      sp_bf16* orow = stage_out + q_off * AT_PITCH;
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
+    for (int qt = 0; qt < 2; ++qt) {
+      const float inv_l = 1.0f / l_tot[qt];
+      sp_bf16* orow = stage_out + (q_off + qt * 16) * AT_PITCH;
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          const int d0 = dt * 32 + 8 * i4 + 4 * g;
-          const uint32_t b0 = sp_f32_to_bf16(o[dt][4 * i4 + 0] * inv_l);
-          const uint32_t b1 = sp_f32_to_bf16(o[dt][4 * i4 + 1] * inv_l);
-          const uint32_t b2 = sp_f32_to_bf16(o[dt][4 * i4 + 2] * inv_l);
-          const uint32_t b3 = sp_f32_to_bf16(o[dt][4 * i4 + 3] * inv_l);
-          *reinterpret_cast<uint2*>(orow + d0) = make_uint2(b0 | (b1 << 16), b2 | (b3 << 16));
-        }
+      for (int dt = 0; dt < 8; ++dt) {
+        const int d0 = dt * 16 + 4 * g;
+        const uint32_t b0 = sp_f32_to_bf16(o[dt][qt][0] * inv_l);
+        const uint32_t b1 = sp_f32_to_bf16(o[dt][qt][1] * inv_l);
+        const uint32_t b2 = sp_f32_to_bf16(o[dt][qt][2] * inv_l);
+        const uint32_t b3 = sp_f32_to_bf16(o[dt][qt][3] * inv_l);
+        *reinterpret_cast<uint2*>(orow + d0) = make_uint2(b0 | (b1 << 16), b2 | (b3 << 16));
+      }
     }
     __syncthreads();
     if (row_ok) {
