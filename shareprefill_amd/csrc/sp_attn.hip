@@ -3,14 +3,14 @@
 // builder count_kernel (shareprefill/attn/shareprefill_attn.py:187-620): the kernel walks the set
 // bits of the row's mask words instead of a sorted id list with row pointers.
 //
-// Layout of the computation (one workgroup = one 128-query block of one head, 4 waves x 32 queries):
+// Layout of the computation (one workgroup = a pair of 128-query blocks of one head, 8 waves x 32 queries; a wave
+// works on its 32 queries as two 16-query tiles with 16x16x32 MFMAs):
 //   S^T = K . Q^T   : A operand = K tile rows from LDS, B operand = Q held in registers for the whole
-//                     row.  In the 32x32 accumulator a lane then owns ONE query (lane % 32) and 16 of
-//                     the tile's 32 keys, so the row max / row sum are in-lane reductions plus a single
-//                     exchange with lane ^ 32.
-//   O^T += V^T . P^T: the P^T operand is the S^T accumulator converted to bf16 in place (no LDS round
+//                     row.  In a 16x16 accumulator a lane owns ONE query (lane % 16) and 4 of the tile's 16
+//                     keys, so the row max / row sum are in-lane reductions plus exchanges with lanes ^ 16, ^ 32.
+//   O^T += V^T . P^T: the P^T operand is the S^T accumulators converted to bf16 in place (no LDS round
 //                     trip); the V^T operand comes from a key-major repack of V made once per call, whose
-//                     key order inside every group of 16 keys matches the accumulator's row order.
+//                     key order inside every group of 32 keys matches the accumulators' row order.
 // K and V^T sub-tiles (64 keys) are staged through LDS by direct global->LDS loads, XOR-swizzled; every wave runs a
 // software pipeline over 32-key half-tiles in which the softmax of one half-tile is issued between the MFMAs of
 // its neighbours (see "the software pipeline of one wave" below).
