@@ -22,9 +22,14 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define LQ_TILE 128          // keys per tile
 #define LQ_D 128             // head dim
 #define LQ_THREADS 256       // 4 waves, wave w owns query rows 32w..32w+31
-#define LQ_STAT_TILES 8      // key tiles per stats workgroup
-#define LQ_PROB_TILES 8      // output key tiles per probs workgroup (plus one leading tile)
+#define LQ_MIN_TILES 8       // key tiles per workgroup (probs: output tiles, plus one leading tile): 8 for short
+#define LQ_MAX_TILES 32      // sequences, up to 32 when that still leaves a thousand workgroups
 #define LQ_PITCH 136         // LDS row pitch (floats) of the probability tile
+// Row maxima are kept in base-2 units (max logit * log2 e), so a probability is one fused multiply-add and one
+// hardware exp2.  "No logit seen yet" is a large finite negative number, not -inf: then max, difference and exp2
+// need no special case (exp2(-inf - finite) = 0 for masked logits, exp2(0) * 0 for an empty history).
+#define LQ_LOG2E 1.4426950408889634f
+#define LQ_NO_MAX (-1.0e30f)
 
 // lane's A operand: scaled last-block queries, 8 k-steps x 8 bf16
 __device__ static __forceinline__ void lq_load_q(const sp_bf16* __restrict__ q, int64_t n, int64_t sq_n, int wave, int lane,
@@ -135,7 +140,7 @@ __device__ static __forceinline__ void lq_finish_logits(floatx16 (&acc)[4], uint
 // ---- kernel 1: chunk partials of the row max / row sum ------------------------------------------
 __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_stats_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
-    int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, int n_chunks,
+    int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, int n_chunks, int tiles_per_wg,
     float2* __restrict__ partial /* [hq][n_chunks][128] */) {
   const int h = blockIdx.y;
   const int chunk = blockIdx.x;
@@ -148,22 +153,22 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_stats_kernel(
   float m[16], l[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    m[r] = -INFINITY;
+    m[r] = LQ_NO_MAX;
     l[r] = 0.f;
   }
   __shared__ sp_bf16 Ks[LQ_TILE * LQ_KPITCH];
   const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
-  const int64_t tile0 = (int64_t)chunk * LQ_STAT_TILES;
+  const int64_t tile0 = (int64_t)chunk * tiles_per_wg;
   LqKRegs kr;
   if (tile0 < n_tiles) lq_fetch_k(kh, n, sk_n, tile0 * LQ_TILE, threadIdx.x, kr);
-  for (int t = 0; t < LQ_STAT_TILES; ++t) {
+  for (int t = 0; t < tiles_per_wg; ++t) {
     const int64_t tile = tile0 + t;
     if (tile >= n_tiles) break;
     const int64_t kb = tile * LQ_TILE;
     __syncthreads();  // the previous tile's operand reads are done
     lq_store_k(Ks, threadIdx.x, kr);
     __syncthreads();
-    if (t + 1 < LQ_STAT_TILES && tile + 1 < n_tiles) lq_fetch_k(kh, n, sk_n, kb + LQ_TILE, threadIdx.x, kr);
+    if (t + 1 < tiles_per_wg && tile + 1 < n_tiles) lq_fetch_k(kh, n, sk_n, kb + LQ_TILE, threadIdx.x, kr);
     floatx16 acc[4];
     lq_tile_logits(Ks, lane, qa, acc);
     if (kb + LQ_TILE <= n - LQ_ROWS)
@@ -173,14 +178,12 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_stats_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const float tmax = fmaxf(fmaxf(acc[0][r], acc[1][r]), fmaxf(acc[2][r], acc[3][r]));
-      if (tmax > -INFINITY) {
-        const float mn = fmaxf(m[r], tmax);
-        float add = 0.f;
+      const float mn = fmaxf(m[r], tmax * LQ_LOG2E);
+      float add = 0.f;
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt) add += __expf(acc[nt][r] - mn);
-        l[r] = l[r] * __expf(m[r] - mn) + add;
-        m[r] = mn;
-      }
+      for (int nt = 0; nt < 4; ++nt) add += __builtin_amdgcn_exp2f(__builtin_fmaf(acc[nt][r], LQ_LOG2E, -mn));
+      l[r] = __builtin_fmaf(l[r], __builtin_amdgcn_exp2f(m[r] - mn), add);
+      m[r] = mn;
     }
   }
   // merge the 32 lanes that share a row (fixed xor tree)
@@ -192,9 +195,7 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_stats_kernel(
       const float m2 = __shfl_xor(mm, o, SP_WAVE);
       const float l2 = __shfl_xor(ll, o, SP_WAVE);
       const float mn = fmaxf(mm, m2);
-      if (mn > -INFINITY) {
-        ll = ll * __expf(mm - mn) + l2 * __expf(m2 - mn);
-      }
+      ll = ll * __builtin_amdgcn_exp2f(mm - mn) + l2 * __builtin_amdgcn_exp2f(m2 - mn);
       mm = mn;
     }
     if ((lane & 31) == 0) {
@@ -212,7 +213,7 @@ __global__ __launch_bounds__(LQ_ROWS * LQ_COMBINE_GROUPS) void sp_lastq_combine_
   __shared__ float gm[LQ_COMBINE_GROUPS][LQ_ROWS], gl[LQ_COMBINE_GROUPS][LQ_ROWS];
   const int h = blockIdx.x, row = threadIdx.x % LQ_ROWS, grp = threadIdx.x / LQ_ROWS;
   const float2* p = partial + (int64_t)h * n_chunks * LQ_ROWS + row;
-  float m = -INFINITY;
+  float m = LQ_NO_MAX;
   for (int c = grp; c < n_chunks; c += LQ_COMBINE_GROUPS) m = fmaxf(m, p[(int64_t)c * LQ_ROWS].x);
   gm[grp][row] = m;
   __syncthreads();
@@ -222,7 +223,7 @@ __global__ __launch_bounds__(LQ_ROWS * LQ_COMBINE_GROUPS) void sp_lastq_combine_
   float l = 0.f;
   for (int c = grp; c < n_chunks; c += LQ_COMBINE_GROUPS) {
     const float2 v = p[(int64_t)c * LQ_ROWS];
-    if (v.x > -INFINITY) l += v.y * __expf(v.x - m);
+    l += v.y * __builtin_amdgcn_exp2f(v.x - m);
   }
   gl[grp][row] = l;
   __syncthreads();
@@ -237,7 +238,7 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
     int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, const float2* __restrict__ rowstat,
     float* __restrict__ vert_tok, float* __restrict__ slash_tok, float* __restrict__ vert_blk,
-    float* __restrict__ slash_blk, int64_t nb) {
+    float* __restrict__ slash_blk, int64_t nb, int tiles_per_wg) {
   extern __shared__ float lds[];
   float* P = lds;                           // [128][LQ_PITCH]
   float* red = lds + LQ_ROWS * LQ_PITCH;    // [4] wave partials of the block sums
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
     rinv[r] = st.y;
   }
   const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
-  const int64_t first = (int64_t)blockIdx.x * LQ_PROB_TILES;
+  const int64_t first = (int64_t)blockIdx.x * tiles_per_wg;
   const float inv_rows = 1.0f / (float)LQ_ROWS;
   float carry = 0.f;  // upper anti-diagonal part handed from the previous tile to bin (u) of this one
   const int u = threadIdx.x & 127;
@@ -263,7 +264,7 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
   // the K tile is staged in the same LDS region the probability tile is written to afterwards
   sp_bf16* Ks = reinterpret_cast<sp_bf16*>(lds);
   const int64_t t_begin = first > 0 ? first - 1 : 0;
-  const int64_t t_end = first + LQ_PROB_TILES < n_tiles ? first + LQ_PROB_TILES : n_tiles;
+  const int64_t t_end = first + tiles_per_wg < n_tiles ? first + tiles_per_wg : n_tiles;
   LqKRegs kr;
   if (t_begin < t_end) lq_fetch_k(kh, n, sk_n, t_begin * LQ_TILE, threadIdx.x, kr);
   for (int64_t tile = t_begin; tile < t_end; ++tile) {
@@ -283,7 +284,8 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
       const int row = lq_row_of(wave, lane, r);
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)  // exp(-inf) = 0 for the masked entries
-        P[row * LQ_PITCH + 32 * nt + (lane & 31)] = __expf(acc[nt][r] - rm[r]) * rinv[r];
+        P[row * LQ_PITCH + 32 * nt + (lane & 31)] =
+            __builtin_amdgcn_exp2f(__builtin_fmaf(acc[nt][r], LQ_LOG2E, -rm[r])) * rinv[r];
     }
     __syncthreads();
     const bool emit = tile >= first;
@@ -322,7 +324,14 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
 }
 
 // ---- host -------------------------------------------------------------------------------------------------
-static inline int lq_chunks(int64_t n) { return (int)sp_ceil_div(sp_ceil_div(n, LQ_TILE), LQ_STAT_TILES); }
+static inline int lq_tiles_per_wg(int64_t n, int32_t hq) {
+  const int64_t work = sp_ceil_div(n, LQ_TILE) * hq;  // (head, key tile) pairs
+  int tiles = LQ_MIN_TILES;
+  while (tiles < LQ_MAX_TILES && work / (2 * tiles) >= 1024) tiles *= 2;
+  return tiles;
+}
+// upper bound of the chunk count (the workspace is sized for it whatever the launch picks)
+static inline int lq_chunks(int64_t n) { return (int)sp_ceil_div(sp_ceil_div(n, LQ_TILE), LQ_MIN_TILES); }
 
 extern "C" size_t sp_lastq_scores_workspace_bytes(int64_t n, int32_t hq, int32_t bs) {
   (void)bs;
@@ -350,16 +359,17 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
              SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: q/k must be 16-byte aligned with strides multiple of 8");
   SP_REQUIRE(workspace_bytes >= sp_lastq_scores_workspace_bytes(n, hq, bs), SP_ERR_WORKSPACE,
              "sp_lastq_scores_bf16: workspace too small");
-  const int n_chunks = lq_chunks(n);
+  const int tiles_per_wg = lq_tiles_per_wg(n, hq);
+  const int n_chunks = (int)sp_ceil_div(sp_ceil_div(n, LQ_TILE), tiles_per_wg);
   const int64_t nb = sp_ceil_div(n, bs);
   float2* partial = (float2*)workspace;
-  float2* rowstat = partial + (size_t)hq * n_chunks * LQ_ROWS;
+  float2* rowstat = partial + (size_t)hq * lq_chunks(n) * LQ_ROWS;
   const float inv_sqrt_d = 1.0f / sqrtf((float)d);
   const int group = hq / hkv;
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(sp_lastq_stats_kernel, dim3(n_chunks, hq), dim3(LQ_THREADS), 0, s, (const sp_bf16*)q,
                      (const sp_bf16*)k, n, hkv, group, q_stride_n, q_stride_h, k_stride_n, k_stride_h, inv_sqrt_d,
-                     flags, n_chunks, partial);
+                     flags, n_chunks, tiles_per_wg, partial);
   SP_LAUNCH_CHECK();
   hipLaunchKernelGGL(sp_lastq_combine_kernel, dim3(hq), dim3(LQ_ROWS * LQ_COMBINE_GROUPS), 0, s, partial, n_chunks,
                      rowstat);
@@ -374,10 +384,10 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
                                (int)lds_bytes));
     attr_set[dev] = true;
   }
-  const int grid_x = (int)sp_ceil_div(nb, LQ_PROB_TILES);
+  const int grid_x = (int)sp_ceil_div(nb, tiles_per_wg);
   hipLaunchKernelGGL(sp_lastq_probs_kernel, dim3(grid_x, hq), dim3(LQ_THREADS), lds_bytes, s, (const sp_bf16*)q,
                      (const sp_bf16*)k, n, hkv, group, q_stride_n, q_stride_h, k_stride_n, k_stride_h, inv_sqrt_d,
-                     flags, rowstat, vert_tok, slash_tok, vert_blk, slash_blk, nb);
+                     flags, rowstat, vert_tok, slash_tok, vert_blk, slash_blk, nb, tiles_per_wg);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
