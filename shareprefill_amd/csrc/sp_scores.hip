@@ -7,11 +7,11 @@
 // Three kernels:
 //   stats   : per (head, key chunk) the running row max / row sum of the logits (bf16 MFMA);
 //   combine : folds the chunk partials into one (max, 1/sum) per query row, in chunk order;
-//   probs   : recomputes the logits tile by tile, writes the probabilities of one 128x128 tile to
-//             LDS, and lets 128 threads sum columns (vertical) while the other 128 sum the tile's
-//             anti-diagonals (slash).  A slash bin receives its upper part from the previous key tile;
-//             that part is carried in a register, and each workgroup recomputes one leading tile so
-//             that no cross-workgroup accumulation (and no float atomic) is needed.
+//   probs   : recomputes the logits tile by tile; the column sums (vertical) start in registers and meet in LDS,
+//             the probabilities of one 128x128 tile go to LDS and all four waves sum its anti-diagonals (slash).
+//             A slash bin receives its upper part from the previous key tile; that part is carried in registers,
+//             and each workgroup recomputes one leading tile so that no cross-workgroup accumulation (and no
+//             float atomic) is needed.
 // Every sum runs in a fixed order, so results are reproducible run to run.
 #include "sp_common.h"
 
@@ -240,8 +240,9 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
     float* __restrict__ vert_tok, float* __restrict__ slash_tok, float* __restrict__ vert_blk,
     float* __restrict__ slash_blk, int64_t nb, int tiles_per_wg) {
   extern __shared__ float lds[];
-  float* P = lds;                           // [128][LQ_PITCH]
-  float* red = lds + LQ_ROWS * LQ_PITCH;    // [4] wave partials of the block sums
+  float* P = lds;                            // [128][LQ_PITCH] probability tile (the K tile is staged here first)
+  float* vpart = lds + LQ_ROWS * LQ_PITCH;   // [8][128] column sums per (wave, lane half)
+  float* spart = vpart + 8 * LQ_TILE;        // [6][128] lower / upper anti-diagonal and column sums per row half
   const int h = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const sp_bf16* qh = q + (int64_t)h * sq_h;
@@ -258,8 +259,7 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
   const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
   const int64_t first = (int64_t)blockIdx.x * tiles_per_wg;
   const float inv_rows = 1.0f / (float)LQ_ROWS;
-  float carry = 0.f;  // upper anti-diagonal part handed from the previous tile to bin (u) of this one
-  const int u = threadIdx.x & 127;
+  float carry[2] = {0.f, 0.f};  // wave 0: upper anti-diagonal parts handed from the previous tile to its two bins
 
   // the K tile is staged in the same LDS region the probability tile is written to afterwards
   sp_bf16* Ks = reinterpret_cast<sp_bf16*>(lds);
@@ -279,47 +279,79 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
       lq_finish_logits<false>(acc, flags, kb, n, wave, lane);
     else
       lq_finish_logits<true>(acc, flags, kb, n, wave, lane);
+    // probabilities (exp2(-inf) = 0 for the masked entries): the tile goes to LDS for the anti-diagonal sums, the
+    // column sums start in registers (a lane holds 16 rows of each of its 4 columns)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = lq_row_of(wave, lane, r);
+    for (int nt = 0; nt < 4; ++nt) {
+      float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt)  // exp(-inf) = 0 for the masked entries
-        P[row * LQ_PITCH + 32 * nt + (lane & 31)] =
-            __builtin_amdgcn_exp2f(__builtin_fmaf(acc[nt][r], LQ_LOG2E, -rm[r])) * rinv[r];
-    }
-    __syncthreads();
-    const bool emit = tile >= first;
-    float val;
-    if (threadIdx.x < 128) {
-      // anti-diagonals: element (i, c) belongs to bin kb + c - i + 127; thread u reads P[i][(u+1+i) mod 128]
-      float low = carry, high = 0.f;
-#pragma unroll 8
-      for (int i = 0; i < LQ_ROWS; ++i) {
-        const float p = P[i * LQ_PITCH + ((u + 1 + i) & 127)];
-        if (i <= 126 - u)
-          high += p;  // c = u+1+i > i : bin kb + 128 + u (next tile)
-        else
-          low += p;   // c = u+1+i-128 <= i : bin kb + u
+      for (int r = 0; r < 16; ++r) {
+        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[nt][r], LQ_LOG2E, -rm[r])) * rinv[r];
+        P[lq_row_of(wave, lane, r) * LQ_PITCH + 32 * nt + (lane & 31)] = pv;
+        part[r & 3] += pv;
       }
-      carry = high;
-      val = low * inv_rows;
-      if (emit && kb + u < n) slash_tok[(int64_t)h * n + kb + u] = val;
-    } else {
-      float s = 0.f;
-#pragma unroll 8
-      for (int i = 0; i < LQ_ROWS; ++i) s += P[i * LQ_PITCH + u];
-      val = s * inv_rows;
-      if (emit && kb + u < n) vert_tok[(int64_t)h * n + kb + u] = val;
+      vpart[(2 * wave + (lane >> 5)) * LQ_TILE + 32 * nt + (lane & 31)] = (part[0] + part[1]) + (part[2] + part[3]);
     }
-    // block sums (the tile is one 128-token block): wave tree, then two waves per vector in fixed order
-    if (kb + u >= n) val = 0.f;
-    const float ws = sp_wave_sum(val);
-    if (lane == 0) red[wave] = ws;
     __syncthreads();
-    if (emit && threadIdx.x == 0) slash_blk[(int64_t)h * nb + tile] = red[0] + red[1];
-    if (emit && threadIdx.x == 128) vert_blk[(int64_t)h * nb + tile] = red[2] + red[3];
-    // the next iteration's P writes are ordered after these reads by the barrier above plus the one below
-    __syncthreads();
+    {
+      // anti-diagonals: element (i, c) belongs to bin kb + c - i + 127.  Thread (u, hv) walks rows 64 hv .. 64 hv + 63
+      // of the wrapped diagonal u, P[i][(u + 1 + i) mod 128]; rows i <= 126 - u lie above the tile's main diagonal
+      // and belong to bin kb + 128 + u (next tile), the others to bin kb + u.  Which of the two a row feeds is the
+      // same for all rows of wave 0 (upper) and wave 3 (lower); four independent partial sums per kind.
+      int tid = threadIdx.x;
+      asm volatile("" : "+v"(tid));  // recompute the walk's addresses per tile: hoisted out of the loop they spill
+      const int u = tid & 127, hv = tid >> 7;
+      const float* col = P + (64 * hv) * LQ_PITCH;
+      float lo[4] = {0.f, 0.f, 0.f, 0.f}, hi[4] = {0.f, 0.f, 0.f, 0.f};
+      if (wave == 0) {
+#pragma unroll 8
+        for (int j = 0; j < 64; ++j) hi[j & 3] += col[j * LQ_PITCH + ((u + 1 + j) & 127)];
+      } else if (wave == 3) {
+#pragma unroll 8
+        for (int j = 0; j < 64; ++j) lo[j & 3] += col[j * LQ_PITCH + ((u + 1 + 64 + j) & 127)];
+      } else {
+        const int split = 126 - u - 64 * hv;  // rows j <= split of this half are upper rows
+#pragma unroll 8
+        for (int j = 0; j < 64; ++j) {
+          const float pv = col[j * LQ_PITCH + ((u + 1 + 64 * hv + j) & 127)];
+          hi[j & 3] += j <= split ? pv : 0.f;
+          lo[j & 3] += j <= split ? 0.f : pv;
+        }
+      }
+      spart[(0 + hv) * LQ_TILE + u] = (lo[0] + lo[1]) + (lo[2] + lo[3]);
+      spart[(2 + hv) * LQ_TILE + u] = (hi[0] + hi[1]) + (hi[2] + hi[3]);
+      // columns: fold the 8 (wave, lane half) partials, four per thread
+      const float* vp = vpart + (4 * hv) * LQ_TILE + u;
+      spart[(4 + hv) * LQ_TILE + u] = (vp[0] + vp[LQ_TILE]) + (vp[2 * LQ_TILE] + vp[3 * LQ_TILE]);
+    }
+    __syncthreads();  // also: every wave is done with the tile, the next K tile may overwrite it
+    // Final sums, token stores and block sums: wave 0 the anti-diagonals, wave 2 the columns, two bins per lane
+    // (the tile is one 128-token block, so a wave's total is the block sum and needs no further exchange).
+    if ((wave & 1) == 0) {
+      const bool emit = tile >= first;
+      int ln = lane;
+      asm volatile("" : "+v"(ln));
+      const int u0 = 2 * ln;
+      float val[2];
+      if (wave == 0) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          val[e] = (carry[e] + (spart[u0 + e] + spart[LQ_TILE + u0 + e])) * inv_rows;
+          carry[e] = spart[2 * LQ_TILE + u0 + e] + spart[3 * LQ_TILE + u0 + e];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) val[e] = (spart[4 * LQ_TILE + u0 + e] + spart[5 * LQ_TILE + u0 + e]) * inv_rows;
+      }
+      float* tok = (wave == 0 ? slash_tok : vert_tok) + (int64_t)h * n + kb;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        if (kb + u0 + e >= n) val[e] = 0.f;
+        else if (emit) tok[u0 + e] = val[e];
+      }
+      const float bsum = sp_wave_sum(val[0] + val[1]);
+      if (emit && lane == 0) (wave == 0 ? slash_blk : vert_blk)[(int64_t)h * nb + tile] = bsum;
+    }
   }
 }
 
@@ -374,7 +406,7 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
   hipLaunchKernelGGL(sp_lastq_combine_kernel, dim3(hq), dim3(LQ_ROWS * LQ_COMBINE_GROUPS), 0, s, partial, n_chunks,
                      rowstat);
   SP_LAUNCH_CHECK();
-  const size_t lds_bytes = (LQ_ROWS * LQ_PITCH + 4) * sizeof(float);
+  const size_t lds_bytes = (LQ_ROWS * LQ_PITCH + 14 * LQ_TILE) * sizeof(float);
   static bool attr_set[64] = {false};  // per device, once (idempotent)
   int dev = 0;
   SP_HIP(hipGetDevice(&dev));
