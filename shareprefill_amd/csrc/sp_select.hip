@@ -700,76 +700,78 @@ __device__ static void vs_sets(const float* __restrict__ vert, const float* __re
 }
 
 // ------------------------------------------------------------------------------------------------
-// pivot election / share test (attention_sharing.py:204-301), single workgroup
+// pivot election / share test (attention_sharing.py:204-301): three launches.
+//   similarity : one workgroup per head, its sqrt-JS against the cluster's stored pivot (one wave per vector);
+//   decide     : one thread walks the heads in ascending order (the election is sequential by definition);
+//   keep       : one workgroup per head; the newly elected pivots store their pooled vectors and their own
+//                vertical-slash sets.
 // ------------------------------------------------------------------------------------------------
 #define DEC_THREADS 256
 #define DEC_MAX_HEADS 256
-__global__ __launch_bounds__(DEC_THREADS) void sp_share_decide_kernel(
-    sp_cluster_state st, const int32_t* __restrict__ head_cluster, int layer_idx, int hq,
-    const float* __restrict__ vert_blk, const float* __restrict__ slash_blk, const int32_t* __restrict__ use_qa,
-    const int32_t* __restrict__ nv, const int32_t* __restrict__ ns, int minb, float sim_thr, double fb_thr,
-    int32_t* __restrict__ decision, float* __restrict__ js_v, float* __restrict__ js_s, int32_t* __restrict__ nv_f,
-    int32_t* __restrict__ ns_f) {
-  __shared__ float s_jv[DEC_MAX_HEADS], s_js[DEC_MAX_HEADS];
-  __shared__ int32_t s_new[DEC_MAX_HEADS];
-  __shared__ __attribute__((aligned(16))) uint32_t s_keys[RS_MAX];
+// similarity of every candidate head against its cluster's stored pivot (pivots of EARLIER layers only: this
+// launch precedes the layer's election)
+__global__ __launch_bounds__(2 * SP_WAVE) void sp_share_similarity_kernel(
+    sp_cluster_state st, const int32_t* __restrict__ head_cluster, const float* __restrict__ vert_blk,
+    const float* __restrict__ slash_blk, const int32_t* __restrict__ use_qa, float* __restrict__ js_v,
+    float* __restrict__ js_s) {
   const int nb = st.nb;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  // similarity of every candidate head against its cluster's stored pivot (pivots of EARLIER layers only)
-  for (int h = wave; h < hq; h += DEC_THREADS / SP_WAVE) {
-    float jv = NAN, js = NAN;
-    const int c = head_cluster[h];
-    if (c >= 0 && !use_qa[h] && st.info[c * 8 + 0] >= 0 && st.info[c * 8 + 1] != 0) {
-      jv = wave_sqrt_js(st.vert + (int64_t)c * nb, vert_blk + (int64_t)h * nb, nb, lane);
-      js = wave_sqrt_js(st.slash + (int64_t)c * nb, slash_blk + (int64_t)h * nb, nb, lane);
-    }
-    if (lane == 0) {
-      s_jv[h] = jv;
-      s_js[h] = js;
-      js_v[h] = jv;
-      js_s[h] = js;
-    }
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int h = 0; h < hq; ++h) {
-      int dec = SP_DEC_VS;
-      s_new[h] = 0;
-      if (use_qa[h]) {
-        dec = SP_DEC_QA;
-      } else {
-        const int c = head_cluster[h];
-        if (c >= 0) {
-          if (st.info[c * 8 + 0] < 0) {
-            st.info[c * 8 + 0] = h;
-            st.info[c * 8 + 2] = nv[h];
-            st.info[c * 8 + 3] = ns[h];
-            st.info[c * 8 + 4] = layer_idx;
-            dec = SP_DEC_DENSE;
-            s_new[h] = 1;
-          } else if (st.info[c * 8 + 1] != 0) {
-            if (s_jv[h] < sim_thr && s_js[h] < sim_thr && st.ratio[c] < fb_thr) dec = SP_DEC_SHARE;
-          }
+  const int h = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = head_cluster[h];
+  float js = NAN;
+  if (c >= 0 && !use_qa[h] && st.info[c * 8 + 0] >= 0 && st.info[c * 8 + 1] != 0)
+    js = wave == 0 ? wave_sqrt_js(st.vert + (int64_t)c * nb, vert_blk + (int64_t)h * nb, nb, lane)
+                   : wave_sqrt_js(st.slash + (int64_t)c * nb, slash_blk + (int64_t)h * nb, nb, lane);
+  if (lane == 0) (wave == 0 ? js_v : js_s)[h] = js;
+}
+
+__global__ __launch_bounds__(SP_WAVE) void sp_share_decide_kernel(
+    sp_cluster_state st, const int32_t* __restrict__ head_cluster, int layer_idx, int hq,
+    const int32_t* __restrict__ use_qa, const int32_t* __restrict__ nv, const int32_t* __restrict__ ns, int minb,
+    float sim_thr, double fb_thr, int32_t* __restrict__ decision, const float* __restrict__ js_v,
+    const float* __restrict__ js_s, int32_t* __restrict__ nv_f, int32_t* __restrict__ ns_f) {
+  if (threadIdx.x != 0) return;
+  for (int h = 0; h < hq; ++h) {
+    int dec = SP_DEC_VS;
+    if (use_qa[h]) {
+      dec = SP_DEC_QA;
+    } else {
+      const int c = head_cluster[h];
+      if (c >= 0) {
+        if (st.info[c * 8 + 0] < 0) {
+          st.info[c * 8 + 0] = h;
+          st.info[c * 8 + 2] = nv[h];
+          st.info[c * 8 + 3] = ns[h];
+          st.info[c * 8 + 4] = layer_idx;
+          dec = SP_DEC_DENSE;
+        } else if (st.info[c * 8 + 1] != 0) {
+          if (js_v[h] < sim_thr && js_s[h] < sim_thr && st.ratio[c] < fb_thr) dec = SP_DEC_SHARE;
         }
       }
-      decision[h] = dec;
-      const bool reset = (dec == SP_DEC_QA || dec == SP_DEC_SHARE);
-      nv_f[h] = reset ? minb : nv[h];
-      ns_f[h] = reset ? minb : ns[h];
     }
+    decision[h] = dec;
+    const bool reset = (dec == SP_DEC_QA || dec == SP_DEC_SHARE);
+    nv_f[h] = reset ? minb : nv[h];
+    ns_f[h] = reset ? minb : ns[h];
   }
-  __syncthreads();
-  // newly elected pivots keep their pooled vectors and their own vertical-slash sets (:223-263)
-  for (int h = 0; h < hq; ++h) {
-    if (!s_new[h]) continue;
-    const int c = head_cluster[h];
-    for (int i = threadIdx.x; i < nb; i += DEC_THREADS) {
-      st.vert[(int64_t)c * nb + i] = vert_blk[(int64_t)h * nb + i];
-      st.slash[(int64_t)c * nb + i] = slash_blk[(int64_t)h * nb + i];
-    }
-    vs_sets(vert_blk + (int64_t)h * nb, slash_blk + (int64_t)h * nb, nb, nv[h], ns[h], s_keys,
-            st.cols + (int64_t)c * nb, st.dists + (int64_t)c * nb, DEC_THREADS);
+}
+
+// newly elected pivots (the cluster's pivot is this head, elected in this layer) keep their pooled vectors and
+// their own vertical-slash sets (:223-263)
+__global__ __launch_bounds__(DEC_THREADS) void sp_share_keep_kernel(
+    sp_cluster_state st, const int32_t* __restrict__ head_cluster, int layer_idx,
+    const float* __restrict__ vert_blk, const float* __restrict__ slash_blk, const int32_t* __restrict__ decision,
+    const int32_t* __restrict__ nv, const int32_t* __restrict__ ns) {
+  __shared__ __attribute__((aligned(16))) uint32_t s_keys[RS_MAX];
+  const int nb = st.nb;
+  const int h = blockIdx.x;
+  const int c = head_cluster[h];
+  if (c < 0 || decision[h] != SP_DEC_DENSE || st.info[c * 8 + 0] != h || st.info[c * 8 + 4] != layer_idx) return;
+  for (int i = threadIdx.x; i < nb; i += DEC_THREADS) {
+    st.vert[(int64_t)c * nb + i] = vert_blk[(int64_t)h * nb + i];
+    st.slash[(int64_t)c * nb + i] = slash_blk[(int64_t)h * nb + i];
   }
+  vs_sets(vert_blk + (int64_t)h * nb, slash_blk + (int64_t)h * nb, nb, nv[h], ns[h], s_keys,
+          st.cols + (int64_t)c * nb, st.dists + (int64_t)c * nb, DEC_THREADS);
 }
 
 static int check_state(const sp_cluster_state* st, int nb, const char* who) {
@@ -797,9 +799,16 @@ extern "C" int sp_share_decide(const sp_cluster_state* state, const int32_t* hea
   SP_REQUIRE(hq > 0 && hq <= DEC_MAX_HEADS, SP_ERR_UNSUPPORTED, "sp_share_decide: hq=%d unsupported (max %d)", hq,
              DEC_MAX_HEADS);
   SP_REQUIRE(state->nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_share_decide: nb=%d exceeds %d", state->nb, RS_MAX);
-  hipLaunchKernelGGL(sp_share_decide_kernel, dim3(1), dim3(DEC_THREADS), 0, (hipStream_t)stream, *state, head_cluster,
-                     layer_idx, hq, vert_blk, slash_blk, use_qa, nv, ns, min_blocks, similarity_threshold,
-                     fallback_threshold, decision, js_v, js_s, nv_final, ns_final);
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(sp_share_similarity_kernel, dim3(hq), dim3(2 * SP_WAVE), 0, s, *state, head_cluster, vert_blk,
+                     slash_blk, use_qa, js_v, js_s);
+  SP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sp_share_decide_kernel, dim3(1), dim3(SP_WAVE), 0, s, *state, head_cluster, layer_idx, hq, use_qa,
+                     nv, ns, min_blocks, similarity_threshold, fallback_threshold, decision, js_v, js_s, nv_final,
+                     ns_final);
+  SP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sp_share_keep_kernel, dim3(hq), dim3(DEC_THREADS), 0, s, *state, head_cluster, layer_idx, vert_blk,
+                     slash_blk, decision, nv, ns);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
