@@ -72,10 +72,14 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 }
 
 // ---- work distribution ----------------------------------------------------------------------------------
-// The kernel is persistent, one workgroup of 8 waves per CU.  A work item is a PAIR of adjacent query blocks
-// (rows 2p, 2p+1) of one head: waves 0-3 own the even row, waves 4-7 the odd row, and both consume the same
-// K / V^T tiles from LDS (the union of the two rows' masks), which halves the L2->LDS traffic wherever
-// neighbouring rows keep the same columns.  Items are grouped in gangs of AT_GANG consecutive pairs of ONE
+// The kernel is persistent, one workgroup of 8 waves per CU.  A work item is a PAIR of query blocks that read the
+// same K / V: waves 0-3 own one, waves 4-7 the other, and both consume the same K / V^T tiles from LDS (the union
+// of the two rows' masks), which halves the L2->LDS traffic wherever the two keep the same columns -- and wherever
+// they do not, the row that does not keep a column idles while the other computes.  Two pairings exist, chosen per
+// two adjacent heads (2i, 2i+1) of a kv group by sp_attn_pairing_kernel, whichever gives the smaller unions:
+//   rows  : item (h, p) = rows 2p and 2p+1 of head h (verticals are shared, slashes shift by one block);
+//   heads : item (h, p) = row 2p + (h & 1) of heads 2i and 2i+1 (heads that share a pattern keep the same columns).
+// Items are grouped in gangs of AT_GANG consecutive pairs of ONE
 // head.  Gangs are dealt statically to the 8 XCDs (queue x = gang position % 8; workgroup b serves queue b % 8
 // first -- workgroups are placed on XCDs round-robin), so the 32 workgroups of an XCD start a gang together at
 // column 0 and sweep the key blocks nearly in lock-step: every K / V^T tile one of them pulls into the XCD's
@@ -86,10 +90,12 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 #define AT_GANG 32
 // The 1 KiB scheduler area (int indices): 0..127 eight queue tickets (one per 64 bytes), 128..191 the pivot slot of
 // every head (one byte each, AT_NO_SLOT = its block sums are not kept), 192..195 {shader cycles, 100 MHz ticks} of
-// workgroup 0, 196 the number of pivot slots in use.
+// workgroup 0, 196 the number of pivot slots in use, 200..231 the pairing of every two adjacent heads (one byte each,
+// see sp_attn_pairing_kernel).
 #define AT_SLOT_TABLE 128
 #define AT_CLOCK_SLOT 192
 #define AT_NPIV_SLOT 196
+#define AT_PAIR_TABLE 200
 #define AT_NO_SLOT 255
 #define AT_MAX_HEADS 256
 #define AT_FWD_THREADS 512
@@ -605,6 +611,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
   __shared__ int s_queue, s_ticket;
   if (PIVOT && sched[AT_NPIV_SLOT] == 0) return;  // no pivot in this layer
   const uint8_t* const slots = reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE);
+  const uint8_t* const pair_table = reinterpret_cast<const uint8_t*>(sched + AT_PAIR_TABLE);
 
   const long long clk0 = clock64(), tick0 = wall_clock64();  // see sp_attn_last_launch_clocks
   AtGeom gm;
@@ -667,28 +674,34 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       break;
     }
     const int ticket = __builtin_amdgcn_readfirstlane(s_ticket);
-    int h, pair;
-    if (!at_item(gm, queue, ticket, h, pair)) continue;
-    const int slot = slots[h];
+    int h_item, pair;
+    if (!at_item(gm, queue, ticket, h_item, pair)) continue;
+    const int slot = slots[h_item];
     if (PIVOT ? slot == AT_NO_SLOT : (skip_slotted && slot != AT_NO_SLOT)) continue;  // the other launch's head
-    const int r0 = 2 * pair;
-    const bool has_b = r0 + 1 < nb;
-    const int r = r0 + grp;  // this wave's row
+    // the item's two (head, row): A for waves 0-3, B for waves 4-7
+    const bool by_heads = !PIVOT && pair_table[h_item >> 1] != 0;
+    const int h_a = by_heads ? (h_item & ~1) : h_item, h_b = by_heads ? (h_item | 1) : h_item;
+    const int r_a = by_heads ? 2 * pair + (h_item & 1) : 2 * pair, r_b = by_heads ? r_a : r_a + 1;
+    if (r_a >= nb) continue;  // (heads pairing, odd nb: the odd head's last item has no row)
+    const bool has_b = r_b < nb;
+    const int h = grp ? h_b : h_a;  // this wave's head
+    const int r = grp ? r_b : r_a;  // this wave's row
     const bool row_ok = grp == 0 || has_b;
-    const int kvh = h / gm.group;
+    const int kvh = h_a / gm.group;
     const sp_bf16* kh = k + (int64_t)kvh * sk_h;
     const char* vth = reinterpret_cast<const char*>(vt + (int64_t)kvh * nb * AT_D * AT_BS);
-    const uint64_t* mrow = mask + ((int64_t)h * nb + r0) * nbw;
+    const uint64_t* mrow_a = mask + ((int64_t)h_a * nb + r_a) * nbw;
+    const uint64_t* mrow_b = mask + ((int64_t)h_b * nb + (has_b ? r_b : r_a)) * nbw;
 
     // ---- the pair's block list: every column kept by either row, ascending, with membership flags ----
     // All waves walk the (uniform) mask words and keep a running count; wave w compacts words w, w+8, ...
     int n_blk = 0;
     {
-      const int wmax = (has_b ? r0 + 1 : r0) >> 6;
+      const int wmax = (has_b ? r_b : r_a) >> 6;
       const int lane = t & 63;
       for (int wi = 0; wi <= wmax; ++wi) {
-        const uint64_t wa = at_trim(mrow[wi], wi, r0);
-        const uint64_t wb = has_b ? at_trim(mrow[nbw + wi], wi, r0 + 1) : 0ull;
+        const uint64_t wa = at_trim(mrow_a[wi], wi, r_a);
+        const uint64_t wb = has_b ? at_trim(mrow_b[wi], wi, r_b) : 0ull;
         const uint64_t wu = wa | wb;
         if ((wi & 7) == wave && ((wu >> lane) & 1ull)) {
           const int pos = n_blk + __builtin_popcountll(wu & ((1ull << lane) - 1ull));
@@ -956,6 +969,43 @@ __global__ void sp_attn_prep_kernel(int* __restrict__ sched, const int32_t* __re
   }
 }
 
+// After sp_attn_prep_kernel: chooses, for every two adjacent heads (2i, 2i+1), how the forward kernel pairs query
+// blocks into work items.  One workgroup per head pair sums the union sizes both ways over all rows,
+//   rows : |row 2p  |  row 2p+1| of each head,      heads : |row r of head 2i  |  row r of head 2i+1|,
+// and writes 1 (pair by heads) when that union is strictly smaller and the two heads may share an item: same kv
+// head, and neither runs in the pivot launch.  Integer sums: the choice does not depend on the order of anything.
+__global__ __launch_bounds__(256) void sp_attn_pairing_kernel(int* __restrict__ sched, const uint64_t* __restrict__ mask,
+                                                              int hq, int group, int nb, int nbw, int skip_slotted) {
+  __shared__ unsigned long long tot[2];
+  const int i = blockIdx.x, h0 = 2 * i, h1 = 2 * i + 1;
+  uint8_t* table = reinterpret_cast<uint8_t*>(sched + AT_PAIR_TABLE);
+  const uint8_t* slots = reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE);
+  const bool eligible = h1 < hq && h0 / group == h1 / group &&
+                        !(skip_slotted && (slots[h0] != AT_NO_SLOT || slots[h1] != AT_NO_SLOT));
+  if (!eligible) {  // (uniform)
+    if (threadIdx.x == 0) table[i] = 0;
+    return;
+  }
+  if (threadIdx.x < 2) tot[threadIdx.x] = 0ull;
+  __syncthreads();
+  const uint64_t* m0 = mask + (int64_t)h0 * nb * nbw;
+  const uint64_t* m1 = mask + (int64_t)h1 * nb * nbw;
+  unsigned long long by_rows = 0ull, by_heads = 0ull;
+  for (int p = threadIdx.x; 2 * p < nb; p += blockDim.x) {
+    const int ra = 2 * p, rb = 2 * p + 1 < nb ? 2 * p + 1 : 2 * p;
+    for (int w = 0; w <= (rb >> 6); ++w) {
+      const uint64_t a0 = m0[(int64_t)ra * nbw + w], b0 = m0[(int64_t)rb * nbw + w];
+      const uint64_t a1 = m1[(int64_t)ra * nbw + w], b1 = m1[(int64_t)rb * nbw + w];
+      by_rows += __builtin_popcountll(a0 | b0) + __builtin_popcountll(a1 | b1);
+      by_heads += __builtin_popcountll(a0 | a1) + (rb != ra ? __builtin_popcountll(b0 | b1) : 0);
+    }
+  }
+  atomicAdd(&tot[0], by_rows);
+  atomicAdd(&tot[1], by_heads);
+  __syncthreads();
+  if (threadIdx.x == 0) table[i] = tot[1] < tot[0] ? 1 : 0;
+}
+
 // ---- pivot heads with a slot: block-averaged attention map from the block sums the forward kernel kept ----
 // avg[h][r][c] = mean over the valid queries of block r of  exp2(u[q][c] - m[q]) / l[q]  (m, l: the query's final
 // softmax statistics).  One workgroup per (query block, head); a wave takes every fourth kept block.
@@ -1190,6 +1240,9 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   }
   float* pivot_u = reinterpret_cast<float*>(ws + base_aligned);
   hipLaunchKernelGGL(sp_attn_prep_kernel, dim3(1), dim3(128), 0, s, counter, decision, (int)hq, max_pivots);
+  SP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sp_attn_pairing_kernel, dim3((unsigned)((hq + 1) / 2)), dim3(256), 0, s, counter, mask, (int)hq,
+                     (int)(hq / hkv), (int)nb, (int)((nb + 63) / 64), max_pivots > 0 ? 1 : 0);
   SP_LAUNCH_CHECK();
   const size_t lds_bytes = AT_LDS_BYTES;
   // per device, once: the kernels' LDS allowance and the CU count (idempotent, so a race between two host threads
