@@ -188,6 +188,13 @@ size_t sp_attn_pivot_scratch_bytes(int64_t n, int32_t bs);
  * stream. */
 int sp_attn_last_launch_clocks(const void* workspace, int64_t n, int32_t hkv, int32_t d, int32_t bs,
                                int64_t* cycles_and_ticks, sp_stream_t stream);
+/* Test / measurement aid (no counterpart in the reference): how the LAST sp_block_sparse_attn_fwd_bf16 launch on
+ * this workspace paired query blocks into work items, one byte per two adjacent heads (2i, 2i+1): 0 = rows 2p and
+ * 2p+1 of each head share an item, 1 = the same row of the two heads does (chosen when it makes the unions of the
+ * paired masks smaller; only inside a kv group).  Copies (hq + 1) / 2 bytes to host memory after synchronising the
+ * stream.  The pairing changes how the work is scheduled, never the result. */
+int sp_attn_last_launch_pairing(const void* workspace, int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs,
+                                uint8_t* by_heads, sp_stream_t stream);
 int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n, int64_t v_stride_h,
                           int32_t bs, void* workspace, size_t workspace_bytes, sp_stream_t stream);
 int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,

@@ -55,6 +55,7 @@ SIGNATURES = {
     "sp_attn_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _I32]),
     "sp_attn_pivot_scratch_bytes": (_SZ, [_I64, _I32]),
     "sp_attn_last_launch_clocks": (_I32, [_P, _I64, _I32, _I32, _I32, _P, _P]),
+    "sp_attn_last_launch_pairing": (_I32, [_P, _I64, _I32, _I32, _I32, _I32, _P, _P]),
     "sp_attn_repack_v_bf16": (_I32, [_P, _I64, _I32, _I32, _I64, _I64, _I32, _P, _SZ, _P]),
     "sp_block_sparse_attn_fwd_bf16": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I64, _I64,
                                              _I32, _F, _P, _P, _P, _P, _P, _SZ, _U32, _P]),

@@ -1169,6 +1169,16 @@ extern "C" int sp_attn_last_launch_clocks(const void* workspace, int64_t n, int3
   return SP_OK;
 }
 
+extern "C" int sp_attn_last_launch_pairing(const void* workspace, int64_t n, int32_t hq, int32_t hkv, int32_t d,
+                                           int32_t bs, uint8_t* by_heads, sp_stream_t stream) {
+  SP_REQUIRE(workspace && by_heads && n > 0 && hq > 0 && hq <= AT_MAX_HEADS && hkv > 0 && d > 0 && bs > 0,
+             SP_ERR_INVALID_ARGUMENT, "sp_attn_last_launch_pairing: bad arguments");
+  SP_HIP(hipStreamSynchronize((hipStream_t)stream));
+  SP_HIP(hipMemcpy(by_heads, (const char*)workspace + at_vt_bytes(n, hkv, d, bs) + AT_PAIR_TABLE * sizeof(int),
+                   (size_t)((hq + 1) / 2), hipMemcpyDeviceToHost));
+  return SP_OK;
+}
+
 extern "C" int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n,
                                      int64_t v_stride_h, int32_t bs, void* workspace, size_t workspace_bytes,
                                      sp_stream_t stream) {

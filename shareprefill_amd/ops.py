@@ -325,6 +325,22 @@ def attention_clock_mhz(n: int, hkv: int, d: int, block_size: int, device) -> fl
     return float(buf[0]) / (float(buf[1]) / 100.0) if buf[1] > 0 else float("nan")
 
 
+def attention_pairing(n: int, hq: int, hkv: int, d: int, block_size: int, device) -> list:
+    """How the last block_sparse_attention launch on this device paired query blocks into work items: one entry per
+    two adjacent heads, False = two rows of a head, True = one row of both heads (test / measurement aid;
+    synchronises the current stream)."""
+    import ctypes
+    lib = _lib.load()
+    ws = _workspaces.get(("attn_vt", str(device)))
+    if ws is None:
+        raise RuntimeError("no attention launch on this device yet")
+    buf = (ctypes.c_uint8 * ((hq + 1) // 2))()
+    st = lib.sp_attn_last_launch_pairing(_ptr(ws), n, hq, hkv, d, block_size, ctypes.cast(buf, ctypes.c_void_p),
+                                         _stream())
+    _lib.check(st, "sp_attn_last_launch_pairing")
+    return [bool(x) for x in buf]
+
+
 def mfma_probe_tflops(random_operands, iters: int = 1500000, reps: int = 2) -> float:
     """Sustained bf16 MFMA rate of back-to-back 32x32x16 MFMAs on every CU (measurement aid).  The default runs
     about 0.2 s per repetition, long enough for the clocks to settle under the load; the last repetition counts."""

@@ -86,6 +86,43 @@ def test_row_pairs_with_unequal_masks(gpu_device):
     _check(out.transpose(0, 1), ref)
 
 
+@pytest.mark.parametrize("n", [2048, 2048 + 40])  # 16 blocks; 17 blocks, the last one ragged
+def test_items_pair_rows_or_heads_whichever_overlaps_more(gpu_device, n):
+    """Heads 0/1 keep the same scattered columns (pairing the same row of both heads gives unions no larger than a
+    row), heads 2/3 keep disjoint columns but every head's neighbouring rows agree (pairing rows wins), heads 4/5
+    lie in different kv groups (never paired by heads), heads 6/7: one of them is a pivot with its own launch when
+    block sums are kept (then never paired by heads).  Whatever the pairing, the result is the oracle's."""
+    from shareprefill_amd import ops
+
+    hq, hkv = 10, 2  # kv groups {0..4}, {5..9}
+    nb = -(-n // 128)
+    q, k, v = _qkv(hq, hkv, n, 4242 + n)
+    rng = np.random.default_rng(5)
+    r = np.arange(nb)
+    m = np.zeros((hq, nb, nb), dtype=bool)
+    m[0] = m[1] = np.tril(rng.random((nb, nb)) < 0.35)               # same scattered blocks, rows independent
+    for h, par in ((2, 0), (3, 1)):                                    # columns of one parity, same in every row
+        m[h] = np.tril(np.broadcast_to((r % 2 == par)[None, :], (nb, nb)))
+    m[4] = np.tril(rng.random((nb, nb)) < 0.35)
+    m[5] = m[4]                                                        # same blocks, but another kv head
+    m[6] = m[7] = np.tril(rng.random((nb, nb)) < 0.5)
+    m[8] = np.tril(np.ones((nb, nb), dtype=bool))                      # dense next to diagonal-only
+    m[:, r, r] = True
+    m[:, :, 0] = True
+    scale = 1.0 / math.sqrt(128)
+    dec = torch.tensor([O.DEC_VS] * 6 + [O.DEC_DENSE] + [O.DEC_VS] * 3, dtype=torch.int32)
+    ref, avg_ref = O.masked_attention(q, k, v, m, 128, scale, want_avg=(dec == O.DEC_DENSE).numpy())
+    mg = ops.bool_to_mask(torch.from_numpy(m)).to(gpu_device)
+    qg, kg, vg = q.to(gpu_device), k.to(gpu_device), v.to(gpu_device)
+    for max_pivots, want_67 in ((0, True), (1, False)):
+        avg = torch.zeros(hq, nb, nb, dtype=torch.float32, device=gpu_device)
+        out = ops.block_sparse_attention(qg, kg, vg, mg, 128, scale, decision=dec.to(gpu_device), avg_attn=avg,
+                                         max_pivots=max_pivots).cpu()
+        assert ops.attention_pairing(n, hq, hkv, 128, 128, gpu_device) == [True, False, False, want_67, False]
+        _check(out.transpose(0, 1), ref)
+        assert (avg.cpu() - avg_ref).abs().max().item() <= 1e-3
+
+
 def test_measurement_aids(gpu_device):
     from shareprefill_amd import ops
 
