@@ -42,7 +42,8 @@ def _random_mask(hq, nb, seed, density=0.4):
     return m
 
 
-@pytest.mark.parametrize("hq,hkv,n", [(4, 2, 1024), (8, 2, 2048), (2, 1, 128), (4, 4, 640), (4, 1, 1000), (7, 1, 8320)])
+@pytest.mark.parametrize("hq,hkv,n", [(4, 2, 1024), (8, 2, 2048), (2, 1, 128), (4, 4, 640), (4, 1, 1000), (7, 1, 8320),
+                                       (256, 32, 384)])  # the last: the largest supported head count
 def test_block_sparse_attention_matches_oracle(gpu_device, hq, hkv, n):
     from shareprefill_amd import ops
 
@@ -233,3 +234,6 @@ def test_attention_rejects_unsupported(gpu_device):
         ops.block_sparse_attention(q, q, q, m, 64, 1.0)
     with pytest.raises(AssertionError):
         ops.block_sparse_attention(q.float(), q, q, m, 128, 1.0)
+    q = torch.zeros(257, 128, 128, dtype=torch.bfloat16, device=gpu_device)  # one query head too many
+    with pytest.raises(NotImplementedError):
+        ops.block_sparse_attention(q, q, q, torch.ones(257, 1, 1, dtype=torch.int64, device=gpu_device), 128, 1.0)

@@ -152,3 +152,39 @@ def test_attention_is_linear_in_v_and_reproducible(c3):
     assert ((lhs - rhs).abs() <= 2.0 ** -7 * scale_of + 5e-2).all()
     assert ((lhs - rhs).abs().mean() / rhs.abs().mean()).item() <= 1e-2
     assert torch.equal(o1, c3.outs[1][0])  # the layer call produced exactly this
+
+
+def test_maximum_supported_length_selection_bit_exact_and_rows_within_tolerance(gpu_device, tmp_path):
+    """524288 tokens = 4096 key blocks, the longest sequence the block lists and rank tables are sized for (two query
+    heads on one kv head, one shared cluster, two layers): budgets, decisions, masks and the pivot's pattern
+    identical to the oracle's integer logic on the GPU's own scores, and single query blocks of both layers -- the
+    dense pivot of layer 0 included -- against the plain fp32 torch evaluation."""
+    import importlib.util
+    import os
+
+    from shareprefill_amd import ops
+
+    spec = importlib.util.spec_from_file_location(
+        "layer_helpers_max", os.path.join(os.path.dirname(__file__), "test_gpu_layer.py"))
+    helpers = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(helpers)
+    n, hq, hkv = 4096 * 128, 2, 1
+    run = helpers.run_layers(gpu_device, tmp_path, hq=hq, hkv=hkv, n=n, seed=91, n_clusters=1, with_free=False)
+    helpers.check_forced(run)
+    assert run["nb"] == 4096
+    assert (run["layers"][0]["dec"] == 1).sum() == 1  # the cluster's pivot runs dense
+    q, k, v = (run[x][None].to(gpu_device) for x in ("q", "k", "v"))
+    scale = 1.0 / math.sqrt(128)
+    for L in run["layers"]:
+        mb = torch.from_numpy(L["mask"]).to(gpu_device)
+        out = L["out"][0].to(gpu_device)  # [N, Hq, D]
+        for h, r in ((0, 4095), (1, 4095), (0, 2048), (1, 4094), (0, 0), (1, 63)):
+            ref = _rows_reference(q, k, v, mb[h, r], h, r, hq // hkv, scale)
+            got = out[r * 128:(r + 1) * 128, h].float()
+            assert (got - ref).abs().max().item() <= MAX_ABS
+            assert ((got - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL
+    # one more key block is refused, not mangled
+    with pytest.raises(NotImplementedError):
+        qq = torch.zeros(1, 4097 * 128, 128, dtype=torch.bfloat16, device=gpu_device)
+        mm = torch.zeros(1, 4097, 65, dtype=torch.int64, device=gpu_device)
+        ops.block_sparse_attention(qq, qq, qq, mm, 128, scale)
