@@ -257,13 +257,13 @@ __device__ static inline uint64_t at_trim(uint64_t x, int wi, int r) {
 // to bf16 in place.
 // Keys are consumed in half-tiles of 32.  For half-tile j the wave issues, in ONE instruction stream,
 //     S(j+1) = K(j+1) . Q^T        16 MFMAs  (matrix core)
-//     O     += V^T(j-1) . P(j-1)   16 MFMAs  (matrix core)
-//     P(j)   = exp2(S(j)*scale - m), row sums, bf16 packing     ~60 vector instructions
-// interleaved one LDS operand read : two MFMAs : three or four vector instructions.  A wave issues in order but
+//     O     += V^T(j-1) . P(j-1)   16 MFMAs  (matrix core), + 2 for the row sums  ones . P(j-1)
+//     P(j)   = exp2(S(j)*scale - m), bf16 packing               ~45 vector instructions
+// interleaved one LDS operand read : two MFMAs : two or three vector instructions.  A wave issues in order but
 // an MFMA executes for 16 cycles after it is issued, so the vector work of half-tile j runs in the shadow of the
-// matrix work of its neighbours; scheduling barriers pin that order.  The running max is taken before the fused
-// stage; when it moves (rare after the first tiles) the pending P(j-1) is flushed into O first, O and the row
-// sums are rescaled, and the stage runs with an empty P.
+// matrix work of its neighbours; scheduling barriers pin that order.  The running max m is lazy (see at_commit):
+// it moves only when some probability came out at 2 or more, and then O and the row sums are rescaled and that
+// half-tile's probabilities are formed again before they are used.
 typedef uint32_t at_u32x4 __attribute__((ext_vector_type(4)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -316,11 +316,11 @@ __device__ __forceinline__ void at_mfma_acc(floatx4& d, bf16x8 a, bf16x8 b) {  /
 __device__ __forceinline__ void at_settle_s(floatx4 (&s)[2][2]) {
   asm volatile("s_nop 15" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]));
 }
-__device__ __forceinline__ void at_settle_o(floatx4 (&o)[8][2]) {
+__device__ __forceinline__ void at_settle_o(floatx4 (&o)[9][2]) {
   asm volatile("s_nop 15"
                : "+v"(o[0][0]), "+v"(o[0][1]), "+v"(o[1][0]), "+v"(o[1][1]), "+v"(o[2][0]), "+v"(o[2][1]),
                  "+v"(o[3][0]), "+v"(o[3][1]), "+v"(o[4][0]), "+v"(o[4][1]), "+v"(o[5][0]), "+v"(o[5][1]),
-                 "+v"(o[6][0]), "+v"(o[6][1]), "+v"(o[7][0]), "+v"(o[7][1]));
+                 "+v"(o[6][0]), "+v"(o[6][1]), "+v"(o[7][0]), "+v"(o[7][1]), "+v"(o[8][0]), "+v"(o[8][1]));
 }
 
 // LDS addresses of a block's operands, one XOR each, made once per block: K channel step ks of sub-tile 2b at
@@ -364,22 +364,19 @@ __device__ __forceinline__ float at_max2(float a, float b) {
 // KQ: which 32-key quarter (0..3) of the block's two K buffers S_out is computed from; VB / KT: which V^T buffer
 // (0: sub-tile 2b-1, 1: sub-tile 2b) and which half of it P_prev belongs to.
 // Slot order: the 8 operand slots of S_out first (channel step outermost, so that the four accumulators take turns),
-// then the 8 of O (one channel tile each), so that S_out is complete early enough for its in-lane maxima (mx_out)
-// to be taken in the shadow of the last slots.
+// then the 8 of O (one channel tile each) and the two row-sum MFMAs; det receives the OR of P_out's packed words.
 template <bool DO_QK, bool DO_PV, int KQ, int VB, int KT>
 __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2],
                                          const floatx4 (&s_in)[2][2], const bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
-                                         floatx4 (&o)[8][2], float sc, const float (&neg_m)[2], float (&l_lane)[2],
-                                         float (&mx_out)[2]) {
+                                         floatx4 (&o)[9][2], float sc, const float (&neg_m)[2], uint32_t (&det)[2],
+                                         const bf16x8& ones) {
   constexpr int NP = (DO_QK ? 8 : 0) + (DO_PV ? 8 : 0);  // operand slots; each holds one MFMA per query tile
   static_assert(NP == 8 || NP == 16, "a fused stage has 8 or 16 operand slots");
   constexpr int EPS = 16 / NP;  // softmax elements handled per operand slot
   constexpr int AHEAD = 2;      // LDS operands are fetched this many slots before their MFMAs
-  constexpr int MX0 = 11;       // first slot that takes part in the maxima of S_out (16-slot stages)
   bf16x8 opnd[NP];
   float x[16], e[16];
   uint32_t pk[8];
-  float mx[2] = {-INFINITY, -INFINITY};
   auto fetch = [&](auto kc) {
     constexpr int k = decltype(kc)::value;
     constexpr bool qk = DO_QK && k < 8;
@@ -424,39 +421,31 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
       if (idx >= 3 && ((idx - 3) & 1) == 0) {
         const int m = (idx - 3) >> 1;
         pk[m] = at_pack2(e[idx - 3], e[idx - 2]);
-        l_lane[(idx - 3) >> 3] += e[idx - 3];
-        l_lane[(idx - 3) >> 3] += e[idx - 2];
+        // OR of the packed probabilities: any exponent >= 128 (P >= 2, inf, NaN) shows in bit 14 or 30
+        if (((idx - 3) & 7) == 0)
+          det[(idx - 3) >> 3] = pk[m];
+        else
+          det[(idx - 3) >> 3] |= pk[m];
       }
       // ... and the results to the slot they were produced in (instruction selection lets pure arithmetic float)
       asm volatile("" : "+v"(x[idx]));
       if (idx >= 1) asm volatile("" : "+v"(e[idx - 1]));
-      if (idx >= 3 && ((idx - 3) & 1) == 0) asm volatile("" : "+v"(pk[(idx - 3) >> 1]), "+v"(l_lane[(idx - 3) >> 3]));
+      if (idx >= 3 && ((idx - 3) & 1) == 0) asm volatile("" : "+v"(pk[(idx - 3) >> 1]), "+v"(det[(idx - 3) >> 3]));
     }
     AT_PIN();
     mfma(std::integral_constant<int, 1>{});
-    if constexpr (DO_QK && DO_PV && k >= MX0 && k < MX0 + 4) {  // two elements of S_out per query tile and slot
-      constexpr int j0 = (k - MX0) * 2;
-      mx[0] = at_max3(mx[0], AT_SVAL(s_out, j0), AT_SVAL(s_out, j0 + 1));
-      mx[1] = at_max3(mx[1], AT_SVAL(s_out, 8 + j0), AT_SVAL(s_out, 8 + j0 + 1));
-      static_assert(MX0 + 4 <= NP, "the maxima must cover all 16 elements");
-      asm volatile("" : "+v"(mx[0]), "+v"(mx[1]));
+    if constexpr (DO_PV && k == NP - 1) {  // row sums of P(j-1) as rounded for the P.V product: ones . P
+      at_mfma_acc(o[8][0], ones, p_prev[0]);
+      at_mfma_acc(o[8][1], ones, p_prev[1]);
     }
     AT_PIN();
   });
   e[15] = __builtin_amdgcn_exp2f(x[15]);
   pk[7] = at_pack2(e[14], e[15]);
-  l_lane[1] += e[14];
-  l_lane[1] += e[15];
-  if constexpr (DO_QK && !DO_PV) {  // start of a run: nothing to hide the maxima behind
-    at_settle_s(s_out);
-#pragma unroll
-    for (int j = 0; j < 8; j += 2) {
-      mx[0] = at_max3(mx[0], AT_SVAL(s_out, j), AT_SVAL(s_out, j + 1));
-      mx[1] = at_max3(mx[1], AT_SVAL(s_out, 8 + j), AT_SVAL(s_out, 8 + j + 1));
-    }
-  }
-  mx_out[0] = mx[0];
-  mx_out[1] = mx[1];
+  det[1] |= pk[7];
+  // start of a run: S_out's last accumulation is only a few cycles old and the next stage reads it with vector
+  // instructions right away
+  if constexpr (DO_QK && !DO_PV) at_settle_s(s_out);
   at_u32x4 w0, w1;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -467,7 +456,7 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
   p_out[1] = __builtin_bit_cast(bf16x8, w1);
 }
 
-// MFMA-only stages (no vector work to hide): first S of a row, flush of a pending P, last P.V of a row
+// MFMA-only stages (no vector work to hide): first S of a run, last P.V of a run
 template <int KH>
 __device__ __forceinline__ void at_qk_only(const char* kb, int koff, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2]) {
   bf16x8 a[8];  // slot i: channel step i / 2, key tile i % 2
@@ -490,7 +479,8 @@ __device__ __forceinline__ void at_qk_only(const char* kb, int koff, const bf16x
 }
 
 template <int KT>
-__device__ __forceinline__ void at_pv_only(const char* vb, int voff, const bf16x8 (&p)[2], floatx4 (&o)[8][2]) {
+__device__ __forceinline__ void at_pv_only(const char* vb, int voff, const bf16x8 (&p)[2], floatx4 (&o)[9][2],
+                                           const bf16x8& ones) {
   bf16x8 a[8];  // slot i: channel tile i
 #pragma unroll
   for (int i = 0; i < 4; ++i) a[i] = at_lds128(vb + (voff ^ (KT << 6)) + i * 16 * 128);
@@ -502,6 +492,8 @@ __device__ __forceinline__ void at_pv_only(const char* vb, int voff, const bf16x
     for (int qt = 0; qt < 2; ++qt) at_mfma_acc(o[i][qt], a[i], p[qt]);
     AT_PIN();
   }
+  at_mfma_acc(o[8][0], ones, p[0]);
+  at_mfma_acc(o[8][1], ones, p[1]);
 }
 
 // causal predicate inside the diagonal block; key_base = offset of the half-tile's first key inside the block
@@ -538,62 +530,73 @@ __device__ __forceinline__ float at_groupmax(float mx) {
   const auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // (own, lane ^ 32) in some order
   return at_max2(__builtin_bit_cast(float, (uint32_t)b[0]), __builtin_bit_cast(float, (uint32_t)b[1]));
 }
-__device__ __forceinline__ float at_groupsum(float x) {
-  uint32_t u = __builtin_bit_cast(uint32_t, x);
-  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  const float s1 = __builtin_bit_cast(float, (uint32_t)a[0]) + __builtin_bit_cast(float, (uint32_t)a[1]);
-  u = __builtin_bit_cast(uint32_t, s1);
-  const auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return __builtin_bit_cast(float, (uint32_t)b[0]) + __builtin_bit_cast(float, (uint32_t)b[1]);
-}
 
-// One pipeline step.  s_in = S(j) (complete) with in-lane maxima mx_carry, p_prev = P(j-1) not yet applied to O
-// (HAVE_PREV); on return mx_carry holds the in-lane maxima of s_out.
-// When some query's running max moves, the pending P(j-1) -- computed against the old max -- is flushed into O
-// first, O and the row sums are rescaled, and P(j-1) is cleared so that the fused stage's P.V part adds nothing.
-// The fused stage itself exists once per step: O never lives in two register sets that would have to be merged.
+// ---- the running max of a query is lazy, its row sum comes off the matrix core ----
+// Probabilities are formed against the max as it stood, m_run, which is only ever a lower bound of the true running
+// max: they can exceed 1, which costs nothing as long as they stay far from the range limit.  The row sums are taken
+// from the probabilities as rounded to bf16 for P.V -- two more MFMAs per step against an all-ones operand,
+// accumulated in o[8] -- so numerator and denominator of the softmax see the same values and the result does not
+// depend on the largest probability being exactly 1.  No maximum per half-tile: the packed probabilities are OR-ed
+// (three instructions per step) and one test of the top exponent bit per step says whether some P(j-1) >= 2, is inf
+// or NaN (the first keys of a row, m_run = AT_NO_MAX; a logit more than one octave above the max).  Only then is the
+// max taken from S(j-1) -- still intact in the registers the next stage overwrites -- O and the sums are rescaled and
+// P(j-1) is formed again; P(j-1) enters O only after this test.
+#define AT_NO_MAX (-1.0e30f)          // "no key seen yet": finite, so exp2(S * scale - m) is +inf or 0, never NaN
+#define AT_P_TOO_LARGE 0x40004000u    // bf16 pair: exponent >= 128 in either half
+
+// s_prev = S(j-1) (causal predicate applied), p = P(j-1), det = OR of its packed words.  On return p is safe to use.
 // PIVOT: l_mark (the row sums at the start of the current key block, see the block sums of pivot heads in the
 // kernel) follows every rescale.
-template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT, bool PIVOT>
-__device__ __forceinline__ void at_step(const AtAddr& ad, const char* vbuf, int voff, const bf16x8 (&qb)[2][4],
-                                        floatx4 (&s_out)[2][2], floatx4 (&s_in)[2][2], bf16x8 (&p_prev)[2],
-                                        bf16x8 (&p_out)[2], floatx4 (&o)[8][2], float scale_log2, float (&m_run)[2],
-                                        float (&l_lane)[2], float (&mx_carry)[2], bool diag, int key_base, int t,
-                                        float (&l_mark)[2]) {
-  if (diag) {  // the causal predicate changes the maxima: take them again
-    at_causal(s_in, key_base, t);
-    at_lanemax(s_in, mx_carry);
-  }
-  // A row's max moves only if one of its four lanes saw a logit above it: one comparison per lane and a ballot
-  // decide; the exchange between the lanes runs only then.
-  const float c0 = mx_carry[0] * scale_log2, c1 = mx_carry[1] * scale_log2;
-  if (__builtin_amdgcn_ballot_w64(c0 > m_run[0] || c1 > m_run[1]) != 0ull) {  // some row's max moved
-    const float m_new0 = at_max2(m_run[0], at_groupmax(c0));
-    const float m_new1 = at_max2(m_run[1], at_groupmax(c1));
-    if (HAVE_PREV) {
-      at_pv_only<KT>(vbuf, voff, p_prev, o);
-      p_prev[0] = __builtin_bit_cast(bf16x8, (at_u32x4){0, 0, 0, 0});
-      p_prev[1] = p_prev[0];
-    }
+template <bool PIVOT>
+__device__ __forceinline__ void at_commit(floatx4 (&s_prev)[2][2], bf16x8 (&p)[2], uint32_t (&det)[2],
+                                          floatx4 (&o)[9][2], float scale_log2, float (&m_run)[2],
+                                          float (&l_mark)[2]) {
+  if (__builtin_amdgcn_ballot_w64(((det[0] | det[1]) & AT_P_TOO_LARGE) != 0u) != 0ull) {
+    at_settle_s(s_prev);
+    float mx[2];
+    at_lanemax(s_prev, mx);
+    const float m_new[2] = {at_max2(m_run[0], at_groupmax(mx[0] * scale_log2)),
+                            at_max2(m_run[1], at_groupmax(mx[1] * scale_log2))};
     at_settle_o(o);
-    // m_run = -inf on a row's first keys: alpha = 0
-    const float alpha[2] = {__builtin_amdgcn_exp2f(m_run[0] - m_new0), __builtin_amdgcn_exp2f(m_run[1] - m_new1)};
+    // m_run = AT_NO_MAX on a row's first keys: alpha = 0 (O and the sums are still zero then)
+    const float alpha[2] = {__builtin_amdgcn_exp2f(m_run[0] - m_new[0]), __builtin_amdgcn_exp2f(m_run[1] - m_new[1])};
+    uint32_t pk[8];
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
-      l_lane[qt] *= alpha[qt];
       if constexpr (PIVOT) l_mark[qt] *= alpha[qt];
 #pragma unroll
-      for (int dt = 0; dt < 8; ++dt)
+      for (int dt = 0; dt < 9; ++dt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) o[dt][qt][j] *= alpha[qt];
+      float e[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        e[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(AT_SVAL(s_prev, 8 * qt + j), scale_log2, -m_new[qt]));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pk[4 * qt + j] = at_pack2(e[2 * j], e[2 * j + 1]);
+      m_run[qt] = m_new[qt];
     }
     at_settle_o(o);
-    m_run[0] = m_new0;
-    m_run[1] = m_new1;
+    p[0] = __builtin_bit_cast(bf16x8, (at_u32x4){pk[0], pk[1], pk[2], pk[3]});
+    p[1] = __builtin_bit_cast(bf16x8, (at_u32x4){pk[4], pk[5], pk[6], pk[7]});
+    asm volatile("s_nop 4" : "+v"(p[0]), "+v"(p[1]));  // vector writes of P are complete before an MFMA reads them
   }
-  // a query with nothing unmasked so far keeps m_run = -inf; exp2(-inf - (-inf)) must not be evaluated
-  const float neg_m[2] = {(m_run[0] == -INFINITY) ? 0.f : -m_run[0], (m_run[1] == -INFINITY) ? 0.f : -m_run[1]};
-  at_fused<DO_QK, HAVE_PREV, KQ, VB, KT>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, l_lane, mx_carry);
+  det[0] = 0u;
+  det[1] = 0u;
+}
+
+// One pipeline step.  s_in = S(j) (complete), p_prev = P(j-1) not yet applied to O (HAVE_PREV), det the OR of its
+// packed words; s_out still holds S(j-1) on entry and S(j+1) on return, p_out = P(j) with its OR in det.
+// The fused stage exists once per step: O never lives in two register sets that would have to be merged.
+template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT, bool PIVOT>
+__device__ __forceinline__ void at_step(const AtAddr& ad, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2],
+                                        floatx4 (&s_in)[2][2], bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
+                                        floatx4 (&o)[9][2], float scale_log2, float (&m_run)[2], uint32_t (&det)[2],
+                                        const bf16x8& ones, bool diag, int key_base, int t, float (&l_mark)[2]) {
+  if (HAVE_PREV) at_commit<PIVOT>(s_out, p_prev, det, o, scale_log2, m_run, l_mark);
+  if (diag) at_causal(s_in, key_base, t);
+  const float neg_m[2] = {-m_run[0], -m_run[1]};
+  at_fused<DO_QK, HAVE_PREV, KQ, VB, KT>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, det, ones);
 }
 
 // PIVOT = false: every head except the pivots that have a slot in the scheduler area's table (when skip_slotted).
@@ -729,26 +732,30 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       }
     }
 
-    floatx4 o[8][2];  // [channel tile][query tile]
+    floatx4 o[9][2];  // [channel tile][query tile]; o[8]: the row sums (ones . P)
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt)
+    for (int dt = 0; dt < 9; ++dt)
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt) o[dt][qt] = (floatx4){0, 0, 0, 0};
-    float m_run[2] = {-INFINITY, -INFINITY}, l_lane[2] = {0.f, 0.f};
-    // Pivot heads: block sums.  l_lane - l_mark is the lane's share of the softmax mass of the key block whose
-    // last half-tile has just gone through the softmax, relative to the current running max (both follow every
-    // rescale); the four lanes of a query are added and the value is kept as u = log2(sum) + m_run.
+    float m_run[2] = {AT_NO_MAX, AT_NO_MAX};
+    uint32_t det[2] = {0u, 0u};
+    bf16x8 ones = __builtin_bit_cast(bf16x8, (at_u32x4){0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
+    asm volatile("" : "+v"(ones));  // one register set for the whole row
+    // Pivot heads: block sums.  o[8] - l_mark is the softmax mass of the key block whose last half-tile has just been
+    // applied to O, relative to the current running max (both follow every rescale; every lane of a query's group
+    // holds the whole sum); it is kept as u = log2(sum) + m_run.
     float l_mark[2] = {0.f, 0.f};
     const int64_t tri_row = (int64_t)slot * ((int64_t)nb * (nb + 1) / 2) + (int64_t)r * (r + 1) / 2;
     float* const pu = PIVOT ? pivot_u + tri_row * AT_BS : nullptr;
     auto emit = [&](int c) {
       if constexpr (PIVOT) {
+        asm volatile("s_nop 15" : "+v"(o[8][0]), "+v"(o[8][1]));  // the sums' last MFMAs have written
         AT_LANE_VIEW(tq);
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
-          const float tl = l_lane[qt] - l_mark[qt];
-          l_mark[qt] = l_lane[qt];
-          const float u = __builtin_amdgcn_logf(at_groupsum(tl)) + m_run[qt];
+          const float tl = o[8][qt][0] - l_mark[qt];
+          l_mark[qt] = o[8][qt][0];
+          const float u = __builtin_amdgcn_logf(tl) + m_run[qt];
           if (g == 0) pu[(int64_t)c * AT_BS + q_off + qt * 16] = u;
         }
       }
@@ -842,19 +849,17 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       }
       floatx4 sa[2][2], sb[2][2];  // [key tile][query tile]
       bf16x8 pa[2], pb[2];         // [query tile]
-      float mx_carry[2];
       // ---- start of a run: S of the first half-tile, nothing to overlap with yet ----
       feed(0);
       at_qk_only<0>(kb, koff, qb, sa);
-      at_lanemax(sa, mx_carry);
       feed(1);
-      at_step<true, false, 1, 0, 0, PIVOT>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+      at_step<true, false, 1, 0, 0, PIVOT>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
                                            c_cur == r, 0, tq, l_mark);
       feed(2);
-      at_step<true, true, 2, 1, 0, PIVOT>(ad, vb1, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+      at_step<true, true, 2, 1, 0, PIVOT>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                           c_cur == r, 32, tq, l_mark);
       feed(3);
-      at_step<true, true, 3, 1, 1, PIVOT>(ad, vb1, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+      at_step<true, true, 3, 1, 1, PIVOT>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
                                           c_cur == r, AT_SUB, tq, l_mark);
       int c_prev = c_cur;
       step_walk();
@@ -867,18 +872,18 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         if (grp) __builtin_amdgcn_s_setprio(1);
         feed(0);
         // S(previous block, keys 96..127) -> P;  S(keys 0..31) on the matrix core;  O += V^T(2b-1, keys 0..31) . P
-        at_step<true, true, 0, 0, 0, PIVOT>(ad, vb, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+        at_step<true, true, 0, 0, 0, PIVOT>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                             c_prev == r, AT_SUB + 32, tq, l_mark);
-        emit(c_prev);
         feed(1);
-        at_step<true, true, 1, 0, 1, PIVOT>(ad, vb, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+        at_step<true, true, 1, 0, 1, PIVOT>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
                                             c_cur == r, 0, tq, l_mark);
+        emit(c_prev);  // the previous block's last half-tile went into O (and the sums) in this step
         if (grp) __builtin_amdgcn_s_setprio(0);
         feed(2);
-        at_step<true, true, 2, 1, 0, PIVOT>(ad, vb1, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+        at_step<true, true, 2, 1, 0, PIVOT>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                             c_cur == r, 32, tq, l_mark);
         feed(3);
-        at_step<true, true, 3, 1, 1, PIVOT>(ad, vb1, voff, qb, sb, sa, pb, pa, o, scale_log2, m_run, l_lane, mx_carry,
+        at_step<true, true, 3, 1, 1, PIVOT>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
                                             c_cur == r, AT_SUB, tq, l_mark);
         c_prev = c_cur;
         step_walk();
@@ -895,17 +900,19 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         vb = vring + ((2 * b + 3) & 3) * AT_VBUF_BYTES;
         at_block_addr(ad, kb, vb, vb, koff, voff);
       }
-      at_step<false, true, 0, 0, 0, PIVOT>(ad, vb, voff, qb, sa, sb, pa, pb, o, scale_log2, m_run, l_lane, mx_carry,
+      at_step<false, true, 0, 0, 0, PIVOT>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                            c_prev == r, AT_SUB + 32, tq, l_mark);
+      at_commit<PIVOT>(sb, pb, det, o, scale_log2, m_run, l_mark);
+      at_pv_only<1>(vb, voff, pb, o, ones);
       emit(c_prev);
-      at_pv_only<1>(vb, voff, pb, o);
     }
     if (!finished) {
       AT_WAIT_VMCNT0();
       __syncthreads();
     }
     at_settle_o(o);
-    const float l_tot[2] = {at_groupsum(l_lane[0]), at_groupsum(l_lane[1])};
+    // every lane of a query's group holds the whole row sum (all rows of the ones . P tile are equal)
+    const float l_tot[2] = {o[8][0][0], o[8][1][0]};
     AT_LANE_VIEW(tq);
 
     // pivot heads: keep the softmax statistics of every query row for the block-average pass

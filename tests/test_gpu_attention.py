@@ -164,7 +164,7 @@ def test_full_mask_equals_sdpa_and_avg_map(gpu_device):
 def test_pivot_maps_from_kept_block_sums_equal_the_recomputing_pass(gpu_device, n, max_pivots):
     """With workspace for their block sums, pivot heads run in a launch of their own and their block-average
     maps come from those sums; without it (or for pivots beyond the room) the maps are recomputed from Q.K^T.
-    Same outputs bit for bit, same maps to rounding, whatever the split; also with a pivot whose mask is not
+    Same outputs bit for bit, same maps to the rounding of the probabilities, whatever the split; also with a pivot whose mask is not
     the full triangle and with a ragged last block."""
     from shareprefill_amd import ops
 
@@ -182,7 +182,9 @@ def test_pivot_maps_from_kept_block_sums_equal_the_recomputing_pass(gpu_device, 
     avg_b = torch.zeros(hq, nb, nb, dtype=torch.float32, device=gpu_device)
     out_b = ops.block_sparse_attention(*args, decision=dec.to(gpu_device), avg_attn=avg_b, max_pivots=max_pivots)
     assert torch.equal(out_a, out_b)
-    assert torch.allclose(avg_a, avg_b, rtol=1e-4, atol=1e-7)
+    # kept block sums add the probabilities as rounded to bf16 for the P.V product (2^-9 relative each), the
+    # recomputing pass adds fp32 probabilities: blocks of a few keys show the difference undiminished
+    assert torch.allclose(avg_a, avg_b, rtol=2.0 ** -8, atol=1e-7)
     _, avg_ref = O.masked_attention(q, k, v, mask, 128, 0.09, want_avg=(dec == O.DEC_DENSE).numpy())
     for h in (0, 2, 4):
         assert torch.allclose(avg_b[h].cpu(), avg_ref[h], rtol=2e-2, atol=1e-5)
