@@ -414,9 +414,11 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
       // The softmax arithmetic depends only on values known before the stage starts, and the optimiser would
       // otherwise move all of it in front of the stage (out of the MFMAs' shadow): the empty asm ties each
       // element to its slot.
-      float sv = AT_SVAL(s_in, idx);
-      asm volatile("" : "+v"(sv));
-      x[idx] = __builtin_fmaf(sv, sc, neg_m[idx >> 3]);
+      // (the tie goes through a scalar copy of the scale: S(j) itself must stay where it is, the next step may
+      // need it again)
+      float sc_here = sc;
+      asm volatile("" : "+s"(sc_here));
+      x[idx] = __builtin_fmaf(AT_SVAL(s_in, idx), sc_here, neg_m[idx >> 3]);
       if (idx >= 1) e[idx - 1] = __builtin_amdgcn_exp2f(x[idx - 1]);
       if (idx >= 3 && ((idx - 3) & 1) == 0) {
         const int m = (idx - 3) >> 1;
@@ -548,12 +550,11 @@ __device__ __forceinline__ float at_groupmax(float mx) {
 // PIVOT: l_mark (the row sums at the start of the current key block, see the block sums of pivot heads in the
 // kernel) follows every rescale.
 template <bool PIVOT>
-__device__ __forceinline__ void at_commit(floatx4 (&s_prev)[2][2], bf16x8 (&p)[2], uint32_t (&det)[2],
+__device__ __forceinline__ void at_commit(const floatx4 (&s_prev)[2][2], bf16x8 (&p)[2], uint32_t (&det)[2],
                                           floatx4 (&o)[9][2], float scale_log2, float (&m_run)[2],
                                           float (&l_mark)[2]) {
   if (__builtin_amdgcn_ballot_w64(((det[0] | det[1]) & AT_P_TOO_LARGE) != 0u) != 0ull) {
-    at_settle_s(s_prev);
-    float mx[2];
+    float mx[2];  // (S(j-1) is a whole stage old: no wait states needed before reading it)
     at_lanemax(s_prev, mx);
     const float m_new[2] = {at_max2(m_run[0], at_groupmax(mx[0] * scale_log2)),
                             at_max2(m_run[1], at_groupmax(mx[1] * scale_log2))};
