@@ -424,15 +424,19 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
         const int m = (idx - 3) >> 1;
         pk[m] = at_pack2(e[idx - 3], e[idx - 2]);
         // OR of the packed probabilities: any exponent >= 128 (P >= 2, inf, NaN) shows in bit 14 or 30
-        if (((idx - 3) & 7) == 0)
-          det[(idx - 3) >> 3] = pk[m];
-        else
-          det[(idx - 3) >> 3] |= pk[m];
+        // (three words at a time: one three-input instruction)
+        if ((m & 3) == 2) det[m >> 2] = pk[m - 2] | pk[m - 1] | pk[m];
+        if ((m & 3) == 3) det[m >> 2] |= pk[m];
       }
       // ... and the results to the slot they were produced in (instruction selection lets pure arithmetic float)
       asm volatile("" : "+v"(x[idx]));
       if (idx >= 1) asm volatile("" : "+v"(e[idx - 1]));
-      if (idx >= 3 && ((idx - 3) & 1) == 0) asm volatile("" : "+v"(pk[(idx - 3) >> 1]), "+v"(det[(idx - 3) >> 3]));
+      if (idx >= 3 && ((idx - 3) & 1) == 0) {
+        if ((((idx - 3) >> 1) & 3) >= 2)
+          asm volatile("" : "+v"(pk[(idx - 3) >> 1]), "+v"(det[(idx - 3) >> 3]));
+        else
+          asm volatile("" : "+v"(pk[(idx - 3) >> 1]));
+      }
     }
     AT_PIN();
     mfma(std::integral_constant<int, 1>{});
