@@ -1,5 +1,5 @@
 """GPU: seeded random sweeps over shapes, masks, thresholds and input scales -- attention against the fp32 oracle
-(including inputs whose running max keeps moving, which exercises the flush-and-rescale path of the kernel) and the
+(including inputs whose running max keeps moving, which exercises the rescale-and-redo path of the kernel) and the
 whole selection against the oracle's integer logic on the GPU's own scores (bit-exact)."""
 
 import importlib.util
