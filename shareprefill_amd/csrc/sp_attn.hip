@@ -406,7 +406,9 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
         at_mfma_acc(o[i][qt], opnd[k], p_prev[qt]);
       }
     };
-    mfma(std::integral_constant<int, 0>{});
+    // the two query tiles take turns at going first: across a slot boundary the B operand (Q or P of one query tile)
+    // stays the same for two MFMAs in a row, as the A operand does inside a slot (+0.5 % under the power cap)
+    mfma(std::integral_constant<int, (k & 1)>{});
     if constexpr (k + AHEAD < NP) fetch(std::integral_constant<int, k + AHEAD>{});
 #pragma unroll
     for (int u = 0; u < EPS; ++u) {
@@ -439,7 +441,7 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
       }
     }
     AT_PIN();
-    mfma(std::integral_constant<int, 1>{});
+    mfma(std::integral_constant<int, 1 - (k & 1)>{});
     if constexpr (DO_PV && k == NP - 1) {  // row sums of P(j-1) as rounded for the P.V product: ones . P
       at_mfma_acc(o[8][0], ones, p_prev[0]);
       at_mfma_acc(o[8][1], ones, p_prev[1]);
