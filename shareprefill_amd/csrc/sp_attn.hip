@@ -931,32 +931,22 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       }
     }
 
-    // ---- epilogue: normalise, transpose through LDS (padded rows, one region per row), coalesced bf16 store ----
-    __syncthreads();
-    sp_bf16* stage_out = reinterpret_cast<sp_bf16*>(lds) + grp * (AT_BS * AT_PITCH);
-#pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-      const float inv_l = 1.0f / l_tot[qt];
-      sp_bf16* orow = stage_out + (q_off + qt * 16) * AT_PITCH;
-#pragma unroll
-      for (int dt = 0; dt < 8; ++dt) {
-        const int d0 = dt * 16 + 4 * g;
-        const uint32_t b0 = sp_f32_to_bf16(o[dt][qt][0] * inv_l);
-        const uint32_t b1 = sp_f32_to_bf16(o[dt][qt][1] * inv_l);
-        const uint32_t b2 = sp_f32_to_bf16(o[dt][qt][2] * inv_l);
-        const uint32_t b3 = sp_f32_to_bf16(o[dt][qt][3] * inv_l);
-        *reinterpret_cast<uint2*>(orow + d0) = make_uint2(b0 | (b1 << 16), b2 | (b3 << 16));
-      }
-    }
-    __syncthreads();
+    // ---- epilogue: normalise and store straight from the accumulators.  A lane holds 4 consecutive channels of its
+    // query per channel tile: 8-byte stores, 32 contiguous bytes per query row and instruction; the four channel tiles
+    // that share a 128-byte line follow each other, and the write-back L2 merges them.  No LDS, no barrier: the
+    // workgroup goes on to its next item while the stores drain. ----
     if (row_ok) {
 #pragma unroll
-      for (int i8 = 0; i8 < 8; ++i8) {
-        const int row = i8 * 16 + (tq_o >> 4);
-        const int64_t qrow = (int64_t)r * AT_BS + row;
+      for (int qt = 0; qt < 2; ++qt) {
+        const int64_t qrow = (int64_t)r * AT_BS + q_off + qt * 16;
         if (qrow < n) {
-          *reinterpret_cast<uint4*>(out + (qrow * hq + h) * AT_D + (tq_o & 15) * 8) =
-              *reinterpret_cast<const uint4*>(stage_out + row * AT_PITCH + (tq_o & 15) * 8);
+          const float inv_l = 1.0f / l_tot[qt];
+          sp_bf16* dst = out + (qrow * hq + h) * AT_D + 4 * g;
+#pragma unroll
+          for (int dt = 0; dt < 8; ++dt)
+            *reinterpret_cast<uint2*>(dst + dt * 16) =
+                make_uint2(at_pack2(o[dt][qt][0] * inv_l, o[dt][qt][1] * inv_l),
+                           at_pack2(o[dt][qt][2] * inv_l, o[dt][qt][3] * inv_l));
         }
       }
     }
