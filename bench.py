@@ -115,8 +115,8 @@ def cpu_baseline(w, q, k, v, mask_bool, decision, kept_blocks, pt):
 
 # HBM-side bytes of one steady-state sp_attn_fwd_kernel launch of the default workload (C3, pattern_threshold
 # 0.95), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the V-repack kernel's known 256 MiB
-# (profiles/attention_layer_C3_hbm_traffic.txt): 102.7 GiB fetched + 1 GiB written.
-MEASURED_ATTN_TRAFFIC_BYTES = {("C3", 0.95): int((102.7 + 1.0) * 2 ** 30)}
+# (profiles/attention_layer_C3_hbm_traffic.txt): 101.7 GiB fetched + 1 GiB written.
+MEASURED_ATTN_TRAFFIC_BYTES = {("C3", 0.95): int((101.7 + 1.0) * 2 ** 30)}
 
 
 def library_gemm_tflops(dev, n=8192, reps=200):
