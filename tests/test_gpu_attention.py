@@ -115,6 +115,7 @@ def test_items_pair_rows_or_heads_whichever_overlaps_more(gpu_device, n):
     ref, avg_ref = O.masked_attention(q, k, v, m, 128, scale, want_avg=(dec == O.DEC_DENSE).numpy())
     mg = ops.bool_to_mask(torch.from_numpy(m)).to(gpu_device)
     qg, kg, vg = q.to(gpu_device), k.to(gpu_device), v.to(gpu_device)
+    outs = []
     for max_pivots, want_67 in ((0, True), (1, False)):
         avg = torch.zeros(hq, nb, nb, dtype=torch.float32, device=gpu_device)
         out = ops.block_sparse_attention(qg, kg, vg, mg, 128, scale, decision=dec.to(gpu_device), avg_attn=avg,
@@ -122,6 +123,10 @@ def test_items_pair_rows_or_heads_whichever_overlaps_more(gpu_device, n):
         assert ops.attention_pairing(n, hq, hkv, 128, 128, gpu_device) == [True, False, False, want_67, False]
         _check(out.transpose(0, 1), ref)
         assert (avg.cpu() - avg_ref).abs().max().item() <= 1e-3
+        outs.append(out)
+    # heads 6 and 7 were paired by heads in the first call and by rows in the second: the pairing decides who shares
+    # K / V tiles with whom, never a bit of the result
+    assert torch.equal(outs[0], outs[1])
 
 
 def test_measurement_aids(gpu_device):
