@@ -32,6 +32,12 @@ Parity pins (what each function is checked against, besides the HIP path):
   vs_ratio ........... literal gather-with-duplicates over vs_id_list
   csr_row_pointers ... reference docstring vector [0,5,8,9,13,14] -> [0,1,2,4,6]
   masked_attention ... torch SDPA (full mask), per-block causal attention (diagonal mask)
+  masked_attention_ref_roundings ... the fp32 masked_attention within the derived rounding noise; bit-equal to its
+                       bf16 rounding on inputs whose probabilities are exact powers of two
+  scaled_last_q ...... torch's own bf16-tensor / Python-float division, exhaustively over every bf16 value
+  pooled_qk_probs .... fp64 double loop; uniform 1/nb for equal keys; head -> kv head h // g (h % Hkv differs)
+  pool_q_head ........ torch's own expression (pad, mean, *bs/(bs-pad)) on CPU bf16, all tail lengths
+  block_probs ........ fp64 double loop; row r uniform 1/(r+1) for zero queries; rows sum to 1; upper triangle 0
   decode_attention ... torch SDPA with enable_gqa; one-key and uniform-logit closed forms
   rope_rotate ........ Hugging Face apply_rotary_pos_emb on bf16 CPU tensors (bit-exact); angle 0 / quarter turn
   layer() ............ scripted sharing scenarios (pivot / same-layer sibling / share / fallback)
@@ -366,14 +372,56 @@ def rope_rotate(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.
     return (a + b).to(torch.bfloat16)
 
 
-def masked_attention(q, k, v, mask, bs, scale, want_avg=None):
+def masked_attention_ref_roundings(q, k, v, mask, bs, scale):
+    """The reference kernel's own arithmetic, shareprefill_attn.py:383-471, block by block in ascending key-block
+    order: base-2 online softmax with the scale folded (softmax_scale * log2 e, :548-551), the probabilities of a
+    block formed against the running maximum and ROUNDED TO bf16 before P.V (:418-420) while the row sum adds them
+    unrounded (:409), fp32 accumulator rescaled by exp2(m_old - m_new), final scale exp2(m - lse), output rounded to
+    bf16 (:471).  q [Hq,N,D], k/v [Hkv,N,D] bf16 or float, mask bool [Hq,nb,nb] -> out bf16 [Hq,N,D]."""
+    hq, n, d = q.shape
+    g = hq // k.shape[0]
+    nb = -(-n // bs)
+    out = torch.zeros(hq, n, d, dtype=torch.bfloat16)
+    mask = np.asarray(mask)
+    pos = torch.arange(n)
+    sc = float(scale) * 1.44269504
+    for h in range(hq):
+        qh, kh = q[h].float(), k[h // g].float()
+        vh = v[h // g].to(torch.bfloat16).float()
+        for r in range(nb):
+            r0, r1 = r * bs, min((r + 1) * bs, n)
+            m = torch.full((r1 - r0,), float("-inf"))
+            lse = torch.full((r1 - r0,), float("-inf"))
+            acc = torch.zeros(r1 - r0, d)
+            for c in np.nonzero(mask[h, r, : r + 1])[0]:
+                c0, c1 = c * bs, min((c + 1) * bs, n)
+                s = (qh[r0:r1] @ kh[c0:c1].T) * sc
+                s = s.masked_fill(pos[None, c0:c1] > pos[r0:r1, None], float("-inf"))
+                m_new = torch.maximum(m, s.max(dim=1).values)
+                p = torch.exp2(s - m_new[:, None])
+                l_blk = p.sum(dim=1)
+                acc = acc * torch.exp2(m - m_new)[:, None] + p.to(torch.bfloat16).float() @ vh[c0:c1]
+                lse = m_new + torch.log2(torch.exp2(lse - m_new) + l_blk)
+                m = m_new
+            out[h, r0:r1] = (acc * torch.exp2(m - lse)[:, None]).to(torch.bfloat16)
+    return out
+
+
+def masked_attention(q, k, v, mask, bs, scale, want_avg=None, emulate_bf16=False):
     """fp32 causal block-sparse attention, shareprefill_attn.py:272-471.
 
     q [Hq,N,D], k/v [Hkv,N,D], mask bool [Hq,nb,nb] -> out fp32 [Hq,N,D].
     want_avg: optional bool[Hq]; for those heads also returns avg[h,r,c] = mean over the
     block's valid queries of the softmax mass falling into key block c (:425-457).
     Only kept blocks are computed.
+    emulate_bf16=True: the output comes from masked_attention_ref_roundings instead (the reference kernel's two
+    bf16 roundings: probabilities before P.V, and the output), returned as fp32 values of bf16 numbers.
     """
+    if emulate_bf16:
+        out_b = masked_attention_ref_roundings(q, k, v, mask, bs, scale).float()
+        if want_avg is None:
+            return out_b, torch.zeros(q.shape[0], -(-q.shape[1] // bs), -(-q.shape[1] // bs))
+        return out_b, masked_attention(q, k, v, mask, bs, scale, want_avg)[1]
     hq, n, d = q.shape
     g = hq // k.shape[0]
     nb = -(-n // bs)

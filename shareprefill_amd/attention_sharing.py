@@ -55,13 +55,19 @@ class LayerPlan:
         """bool [1, Hq], the reference's second return value (attention_sharing.py:366)."""
         return (self.decision == _lib.SP_DEC_DENSE).unsqueeze(0)
 
+    def _need_mask(self) -> torch.Tensor:
+        if self.mask is None:
+            raise RuntimeError("this layer's block mask was released when the next layer was planned; set "
+                               "AttentionSharing.keep_plans = True to keep every layer's mask")
+        return self.mask
+
     def block_idx(self) -> List[List[torch.Tensor]]:
         """The reference's first return value: [B][Hq] sorted unique flat ids (synchronises)."""
-        return [ops.mask_to_block_idx(self.mask, self.nb)]
+        return [ops.mask_to_block_idx(self._need_mask(), self.nb)]
 
     def density(self) -> torch.Tensor:
         """Kept blocks / lower-triangular blocks per head (synchronises when read)."""
-        kept = ops.mask_row_pointers(self.mask)[:, -1].to(torch.float64)
+        kept = ops.mask_row_pointers(self._need_mask())[:, -1].to(torch.float64)
         return kept / (self.nb * (self.nb + 1) / 2)
 
 
@@ -84,8 +90,12 @@ class AttentionSharing:
         self._head_cluster: Dict[Tuple[int, int, str], torch.Tensor] = {}
         self._layer_avg: Dict[int, torch.Tensor] = {}
         self.keep_pivot_maps = False  # keep every layer's avg_attn alive so get_pivotal_attn can return it
-        self.keep_debug = False
+        self.keep_debug = False   # keep every float intermediate of every layer (tests)
+        self.keep_plans = False   # keep every layer's block mask (64 MiB per layer at 512K tokens) until the reset
+        # one LayerPlan per layer planned since the last reset; unless keep_plans / keep_debug is set only the
+        # newest one still holds its mask, the older ones keep their few per-head integers
         self.plans: List[LayerPlan] = []
+        self._scratch: Dict[Tuple[str, str], torch.Tensor] = {}
         self.reset_state()
 
     # ---- table ------------------------------------------------------------------------------------
@@ -192,20 +202,30 @@ class AttentionSharing:
             plan.vert_tok, plan.slash_tok, plan.vert_blk, plan.slash_blk = vert_tok, slash_tok, vert_blk, slash_blk
             plan.kbar, plan.avg_qk, plan.js_qa, plan.js_v, plan.js_s = kbar, avg_qk, js_qa, js_v, js_s
             plan.qa_probs = qa_probs.clone()
+        if self.plans and not (self.keep_plans or self.keep_debug):
+            self.plans[-1].mask = None
         self.plans.append(plan)
         return plan
 
     def _qa_scratch(self, hq: int, nb: int, device) -> torch.Tensor:
-        buf = ops._workspace("qa_probs", hq * nb * nb * 4, device)
-        return buf[: hq * nb * nb * 4].view(torch.float32).view(hq, nb, nb)
+        """fp32 [Hq, nb, nb] scratch of the query-aware selection, owned by this object (one model, one stream of
+        layers in order), grow-only, reused by every layer."""
+        need = hq * nb * nb * 4
+        key = ("qa_probs", str(device))
+        buf = self._scratch.get(key)
+        if buf is None or buf.numel() < need:
+            buf = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+            self._scratch[key] = buf
+        return buf[:need].view(torch.float32).view(hq, nb, nb)
 
     def get_active_blocks(self, q, k, layer_idx, num_heads, block_size, min_budget, max_budget,
                           pattern_threshold=0.9, similarity_threshold=0.5, fallback_threshold=0.9,
-                          queryaware_threshold=0.1, gqa_interleave=False):
+                          queryaware_threshold=0.1, gqa_interleave=False, as_ids=False):
         """Reference signature (attention_sharing.py:105-119): q [B, N, Hq, D], k [B, N, Hkv or Hq, D].
 
-        Returns (block bit mask [B, Hq, nb, nbw], use_dense bool [B, Hq]); the reference returns ragged id
-        lists instead of the mask -- LayerPlan.block_idx() / ops.mask_to_block_idx give that form."""
+        Returns (block bit mask [B, Hq, nb, nbw], use_dense bool [B, Hq]).  With as_ids=True the first value is the
+        reference's form instead (attention_sharing.py:366): list[B][Hq] of sorted unique int64 flat block ids
+        row * nb + col; building the ragged lists synchronises the stream."""
         if gqa_interleave:
             raise NotImplementedError("gqa_interleave=True (query head h -> kv head h % Hkv) is not supported")
         if q.shape[0] != 1:
@@ -213,6 +233,8 @@ class AttentionSharing:
         plan = self.plan_layer(q[0].transpose(0, 1), k[0].transpose(0, 1), layer_idx, block_size, min_budget,
                                max_budget, pattern_threshold, similarity_threshold, fallback_threshold,
                                queryaware_threshold)
+        if as_ids:
+            return plan.block_idx(), plan.use_dense
         return plan.mask.unsqueeze(0), plan.use_dense
 
     def update_pivotal_attns(self, layer_idx, avg_attn, use_dense, pattern_threshold=0.9):
@@ -222,11 +244,12 @@ class AttentionSharing:
         if self._state is None:
             return
         hq = avg_attn.shape[1]
+        hc = self._head_cluster_tensor(layer_idx, hq, avg_attn.device)
         if use_dense.dtype == torch.bool:
-            decision = use_dense.reshape(-1).to(torch.int32) * _lib.SP_DEC_DENSE
+            # a caller's own flags may name heads outside every shared cluster: those keep no pattern
+            decision = (use_dense.reshape(-1) & (hc >= 0)).to(torch.int32) * _lib.SP_DEC_DENSE
         else:
             decision = use_dense.reshape(-1)
-        hc = self._head_cluster_tensor(layer_idx, hq, avg_attn.device)
         ops.pivot_update(self._state, hc, decision, avg_attn[0], pattern_threshold)
         if self.keep_pivot_maps:
             self._layer_avg[layer_idx] = avg_attn

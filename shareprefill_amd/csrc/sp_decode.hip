@@ -17,7 +17,7 @@
 #define DC_THREADS 256
 #define DC_TILE 128   // keys per tile
 #define DC_D 128
-#define DC_GMAX 8     // query heads per kv head
+#define DC_GMAX 32    // query heads per kv head (the 32-wide operand of the MFMAs); kernels are built for <= 8, 16, 32
 #define DC_PITCH 136  // bf16 elements per LDS row (272 bytes: conflict-free 128-bit reads)
 
 typedef uint32_t dc_u32x4 __attribute__((ext_vector_type(4)));
@@ -51,14 +51,17 @@ __device__ static __forceinline__ void dc_store(sp_bf16* tile, int t, const dc_u
 }
 
 // grid (splits, hkv); partial layout: o [hkv][splits][g][128] fp32, ml [hkv][splits][g] float2 (m in log2 units, l)
+// G8 = groups of 8 heads the instance handles (g <= 8 * G8): accumulator rows r < 4 * G8 can belong to real heads
+template <int G8>
 __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ v, int64_t n, int g,
     int64_t sq_h, int64_t sk_n, int64_t sk_h, int64_t sv_n, int64_t sv_h, float scale_log2, int64_t keys_per_split,
     float* __restrict__ o_part, float2* __restrict__ ml_part) {
   __shared__ __attribute__((aligned(16))) sp_bf16 Ks[DC_TILE * DC_PITCH];
   __shared__ __attribute__((aligned(16))) sp_bf16 Vs[DC_TILE * DC_PITCH];
-  __shared__ __attribute__((aligned(16))) sp_bf16 Ps[DC_GMAX * DC_PITCH];  // probabilities [head][key]
-  __shared__ float wmax[4][DC_GMAX], wsum[4][DC_GMAX], alpha_s[DC_GMAX];
+  constexpr int GM = 8 * G8;
+  __shared__ __attribute__((aligned(16))) sp_bf16 Ps[GM * DC_PITCH];  // probabilities [head][key]
+  __shared__ float wmax[4][GM], wsum[4][GM], alpha_s[GM];
   const int split = blockIdx.x, kvh = blockIdx.y, splits = gridDim.x;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int lh = lane & 31, hi = lane >> 5;  // operand column / row inside a 32-wide tile, lane half
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
   int64_t key_end = key_begin + keys_per_split;
   if (key_end > n) key_end = n;
 
-  dc_floatx16 o = {0};                   // rows = heads 8(r/4) + 4hi + r%4 (only r < 4 can be real), col = channel 32*wave + lh
+  dc_floatx16 o = {0};                   // rows = heads 8(r/4) + 4hi + r%4 (only r < 4 G8 can be real), col = channel 32*wave + lh
   float m_run = -INFINITY, l_run = 0.f;  // of head lh (every wave keeps the same copy)
   dc_u32x4 kr[8], vr[8];
   if (key_begin < key_end) {
@@ -142,8 +145,8 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
     }
     // ---- O += P . V for this wave's 32 channels; only accumulator rows of real heads need the rescale ----
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int h = 4 * hi + r;
+    for (int r = 0; r < 4 * G8; ++r) {
+      const int h = 8 * (r >> 2) + 4 * hi + (r & 3);
       if (h < g) o[r] *= alpha_s[h];
     }
     {
@@ -173,8 +176,8 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
 
   float* op = o_part + (((int64_t)kvh * splits + split) * g) * DC_D;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int h = 4 * hi + r;
+  for (int r = 0; r < 4 * G8; ++r) {
+    const int h = 8 * (r >> 2) + 4 * hi + (r & 3);
     if (h < g) op[h * DC_D + 32 * wave + lh] = o[r];
   }
   if (wave == 0 && hi == 0 && head_ok) ml_part[((int64_t)kvh * splits + split) * g + lh] = make_float2(m_run, l_run);
@@ -225,33 +228,64 @@ extern "C" size_t sp_decode_workspace_bytes(int64_t n, int32_t hq, int32_t hkv) 
   return (size_t)dc_splits(n, hkv) * hq * (DC_D * sizeof(float) + sizeof(float2));
 }
 
-extern "C" int sp_decode_attn_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,
-                                   int32_t d, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
-                                   int64_t v_stride_n, int64_t v_stride_h, float softmax_scale, void* out,
-                                   void* workspace, size_t workspace_bytes, sp_stream_t stream) {
-  SP_REQUIRE(q && k && v && out && workspace, SP_ERR_INVALID_ARGUMENT, "sp_decode_attn_bf16: null pointer");
-  SP_REQUIRE(n > 0 && hq > 0 && hkv > 0 && hq % hkv == 0, SP_ERR_INVALID_ARGUMENT,
-             "sp_decode_attn_bf16: bad shape n=%lld hq=%d hkv=%d", (long long)n, hq, hkv);
-  SP_REQUIRE(softmax_scale > 0.f, SP_ERR_INVALID_ARGUMENT, "sp_decode_attn_bf16: softmax_scale must be > 0");
-  SP_REQUIRE(d == DC_D, SP_ERR_UNSUPPORTED, "sp_decode_attn_bf16: head_dim %d unsupported (only 128)", d);
-  SP_REQUIRE(hq / hkv <= DC_GMAX, SP_ERR_UNSUPPORTED, "sp_decode_attn_bf16: more than %d query heads per kv head",
-             DC_GMAX);
+// argument checks shared by the two entry points
+static int dc_check(const char* who, const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,
+                    int32_t d, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n,
+                    int64_t v_stride_h, float softmax_scale, const void* out) {
+  SP_REQUIRE(q && k && v && out, SP_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  SP_REQUIRE(n > 0 && hq > 0 && hkv > 0 && hq % hkv == 0, SP_ERR_INVALID_ARGUMENT, "%s: bad shape n=%lld hq=%d hkv=%d",
+             who, (long long)n, hq, hkv);
+  SP_REQUIRE(softmax_scale > 0.f, SP_ERR_INVALID_ARGUMENT, "%s: softmax_scale must be > 0", who);
+  SP_REQUIRE(d == DC_D, SP_ERR_UNSUPPORTED, "%s: head_dim %d unsupported (only 128)", who, d);
+  SP_REQUIRE(hq / hkv <= DC_GMAX, SP_ERR_UNSUPPORTED, "%s: more than %d query heads per kv head", who, DC_GMAX);
+  // q, k and v are read with 16-byte loads
+  SP_REQUIRE(q_stride_h % 8 == 0 && ((uintptr_t)q % 16) == 0, SP_ERR_UNSUPPORTED,
+             "%s: q must be 16-byte aligned with a head stride multiple of 8", who);
   SP_REQUIRE(k_stride_n % 8 == 0 && k_stride_h % 8 == 0 && v_stride_n % 8 == 0 && v_stride_h % 8 == 0 &&
                  ((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0,
-             SP_ERR_UNSUPPORTED, "sp_decode_attn_bf16: k/v must be 16-byte aligned with strides multiple of 8");
-  SP_REQUIRE(workspace_bytes >= sp_decode_workspace_bytes(n, hq, hkv) && ((uintptr_t)workspace % 8) == 0,
-             SP_ERR_WORKSPACE, "sp_decode_attn_bf16: workspace too small or misaligned");
+             SP_ERR_UNSUPPORTED, "%s: k/v must be 16-byte aligned with strides multiple of 8", who);
+  return SP_OK;
+}
+
+// both kernels; `partials` holds sp_decode_workspace_bytes(n, hq, hkv) bytes, every one of which the first kernel
+// writes before the second reads it (nothing has to be cleared)
+static int dc_launch(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,
+                     int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
+                     float softmax_scale, void* out, void* partials, hipStream_t s) {
   const int g = hq / hkv;
   const int splits = dc_splits(n, hkv);
   const int64_t keys_per_split = sp_ceil_div(sp_ceil_div(n, splits), DC_TILE) * DC_TILE;
-  float* o_part = (float*)workspace;
+  float* o_part = (float*)partials;
   float2* ml_part = (float2*)(o_part + (size_t)splits * hq * DC_D);
-  hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_decode_partial_kernel, dim3(splits, hkv), dim3(DC_THREADS), 0, s, (const sp_bf16*)q,
-                     (const sp_bf16*)k, (const sp_bf16*)v, n, g, q_stride_h, k_stride_n, k_stride_h, v_stride_n,
-                     v_stride_h, softmax_scale * 1.4426950408889634f, keys_per_split, o_part, ml_part);
+  const float scale_log2 = softmax_scale * 1.4426950408889634f;
+#define DC_LAUNCH_PARTIAL(G8)                                                                                         \
+  hipLaunchKernelGGL(sp_decode_partial_kernel<G8>, dim3(splits, hkv), dim3(DC_THREADS), 0, s, (const sp_bf16*)q,      \
+                     (const sp_bf16*)k, (const sp_bf16*)v, n, g, q_stride_h, k_stride_n, k_stride_h, v_stride_n,      \
+                     v_stride_h, scale_log2, keys_per_split, o_part, ml_part)
+  if (g <= 8) {
+    DC_LAUNCH_PARTIAL(1);
+  } else if (g <= 16) {
+    DC_LAUNCH_PARTIAL(2);
+  } else {
+    DC_LAUNCH_PARTIAL(4);
+  }
+#undef DC_LAUNCH_PARTIAL
   SP_LAUNCH_CHECK();
   hipLaunchKernelGGL(sp_decode_combine_kernel, dim3(hq), dim3(DC_D), 0, s, o_part, ml_part, g, splits, (sp_bf16*)out);
   SP_LAUNCH_CHECK();
   return SP_OK;
+}
+
+extern "C" int sp_decode_attn_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,
+                                   int32_t d, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                                   int64_t v_stride_n, int64_t v_stride_h, float softmax_scale, void* out,
+                                   void* workspace, size_t workspace_bytes, sp_stream_t stream) {
+  int rc = dc_check("sp_decode_attn_bf16", q, k, v, n, hq, hkv, d, q_stride_h, k_stride_n, k_stride_h, v_stride_n,
+                    v_stride_h, softmax_scale, out);
+  if (rc) return rc;
+  SP_REQUIRE(workspace != nullptr, SP_ERR_INVALID_ARGUMENT, "sp_decode_attn_bf16: null workspace");
+  SP_REQUIRE(workspace_bytes >= sp_decode_workspace_bytes(n, hq, hkv) && ((uintptr_t)workspace % 8) == 0,
+             SP_ERR_WORKSPACE, "sp_decode_attn_bf16: workspace too small or misaligned");
+  return dc_launch(q, k, v, n, hq, hkv, q_stride_h, k_stride_n, k_stride_h, v_stride_n, v_stride_h, softmax_scale, out,
+                   workspace, (hipStream_t)stream);
 }

@@ -708,6 +708,9 @@ __device__ static void vs_sets(const float* __restrict__ vert, const float* __re
 // ------------------------------------------------------------------------------------------------
 #define DEC_THREADS 256
 #define DEC_MAX_HEADS 256
+// head_cluster[h] names a slot of the state only inside [0, n_clusters); -1 (no shared cluster) and anything a
+// caller got wrong must never be used as an index into the slabs
+__device__ __forceinline__ bool sp_slot_ok(const sp_cluster_state& st, int c) { return c >= 0 && c < st.n_clusters; }
 // similarity of every candidate head against its cluster's stored pivot (pivots of EARLIER layers only: this
 // launch precedes the layer's election)
 __global__ __launch_bounds__(2 * SP_WAVE) void sp_share_similarity_kernel(
@@ -718,7 +721,7 @@ __global__ __launch_bounds__(2 * SP_WAVE) void sp_share_similarity_kernel(
   const int h = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = head_cluster[h];
   float js = NAN;
-  if (c >= 0 && !use_qa[h] && st.info[c * 8 + 0] >= 0 && st.info[c * 8 + 1] != 0)
+  if (sp_slot_ok(st, c) && !use_qa[h] && st.info[c * 8 + 0] >= 0 && st.info[c * 8 + 1] != 0)
     js = wave == 0 ? wave_sqrt_js(st.vert + (int64_t)c * nb, vert_blk + (int64_t)h * nb, nb, lane)
                    : wave_sqrt_js(st.slash + (int64_t)c * nb, slash_blk + (int64_t)h * nb, nb, lane);
   if (lane == 0) (wave == 0 ? js_v : js_s)[h] = js;
@@ -736,7 +739,7 @@ __global__ __launch_bounds__(SP_WAVE) void sp_share_decide_kernel(
       dec = SP_DEC_QA;
     } else {
       const int c = head_cluster[h];
-      if (c >= 0) {
+      if (sp_slot_ok(st, c)) {
         if (st.info[c * 8 + 0] < 0) {
           st.info[c * 8 + 0] = h;
           st.info[c * 8 + 2] = nv[h];
@@ -765,7 +768,8 @@ __global__ __launch_bounds__(DEC_THREADS) void sp_share_keep_kernel(
   const int nb = st.nb;
   const int h = blockIdx.x;
   const int c = head_cluster[h];
-  if (c < 0 || decision[h] != SP_DEC_DENSE || st.info[c * 8 + 0] != h || st.info[c * 8 + 4] != layer_idx) return;
+  if (!sp_slot_ok(st, c) || decision[h] != SP_DEC_DENSE || st.info[c * 8 + 0] != h || st.info[c * 8 + 4] != layer_idx)
+    return;
   for (int i = threadIdx.x; i < nb; i += DEC_THREADS) {
     st.vert[(int64_t)c * nb + i] = vert_blk[(int64_t)h * nb + i];
     st.slash[(int64_t)c * nb + i] = slash_blk[(int64_t)h * nb + i];
@@ -830,7 +834,8 @@ __global__ __launch_bounds__(MASK_THREADS) void sp_build_mask_kernel(
     vs_sets(vert_blk + (int64_t)h * nb, slash_blk + (int64_t)h * nb, nb, nv_f[h], ns_f[h], s_keys, s_cols, s_dists,
             MASK_THREADS);
   const uint64_t* pat = nullptr;
-  if (dec == SP_DEC_SHARE) pat = st.pattern + (int64_t)head_cluster[h] * nb * nbw;
+  // a SHARE decision without a valid slot (only a caller's own decision vector can hold one) adds no pattern
+  if (dec == SP_DEC_SHARE && sp_slot_ok(st, head_cluster[h])) pat = st.pattern + (int64_t)head_cluster[h] * nb * nbw;
   uint64_t* mh = mask + (int64_t)h * nb * nbw;
   const int rows_per = (nb + MASK_SPLIT - 1) / MASK_SPLIT;
   const int r_begin = blockIdx.y * rows_per, r_end = min(nb, r_begin + rows_per);
@@ -973,6 +978,7 @@ __global__ __launch_bounds__(RS_THREADS) void sp_pivot_rows_kernel(sp_cluster_st
   const int r = blockIdx.x, h = blockIdx.y;
   if (decision[h] != SP_DEC_DENSE) return;
   const int c = head_cluster[h];
+  if (!sp_slot_ok(st, c)) return;  // a dense head outside every shared cluster keeps no pattern
   const float* row = avg_attn + ((int64_t)h * nb + r) * nb;
   const int keep = rs_row_keep(row, nb, t_lt, sh.row);
   uint32_t* prow = reinterpret_cast<uint32_t*>(st.pattern + ((int64_t)c * nb + r) * nbw);
@@ -1008,11 +1014,13 @@ __global__ __launch_bounds__(RS_THREADS) void sp_pivot_rows_kernel(sp_cluster_st
   }
 }
 
-__global__ void sp_pivot_zero_kernel(const int32_t* __restrict__ head_cluster, const int32_t* __restrict__ decision,
-                                     int hq, unsigned long long* __restrict__ accum) {
+__global__ void sp_pivot_zero_kernel(sp_cluster_state st, const int32_t* __restrict__ head_cluster,
+                                     const int32_t* __restrict__ decision, int hq,
+                                     unsigned long long* __restrict__ accum) {
   const int h = threadIdx.x;
   if (h < hq && decision[h] == SP_DEC_DENSE) {
     const int c = head_cluster[h];
+    if (!sp_slot_ok(st, c)) return;
     accum[c * 2 + 0] = 0;
     accum[c * 2 + 1] = 0;
   }
@@ -1024,6 +1032,7 @@ __global__ void sp_pivot_finish_kernel(sp_cluster_state st, const int32_t* __res
   const int h = threadIdx.x;
   if (h >= hq || decision[h] != SP_DEC_DENSE) return;
   const int c = head_cluster[h];
+  if (!sp_slot_ok(st, c)) return;
   // every out-of-range slash / vertical slot of the reference's id list is the padding id 0
   unsigned long long pad = 0;
   for (int i = 0; i < nb; ++i) {
@@ -1050,7 +1059,7 @@ extern "C" int sp_pivot_update(const sp_cluster_state* state, const int32_t* hea
   if (state->n_clusters == 0) return SP_OK;
   unsigned long long* accum = reinterpret_cast<unsigned long long*>(state->accum);
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_pivot_zero_kernel, dim3(1), dim3(1024), 0, s, head_cluster, decision, hq, accum);
+  hipLaunchKernelGGL(sp_pivot_zero_kernel, dim3(1), dim3(1024), 0, s, *state, head_cluster, decision, hq, accum);
   SP_LAUNCH_CHECK();
   hipLaunchKernelGGL(sp_pivot_rows_kernel, dim3(nb, hq), dim3(RS_THREADS), 0, s, *state, head_cluster, decision,
                      avg_attn, nb, (nb + 63) / 64, (long long)sp_thr_lt(pattern_threshold), accum);

@@ -21,12 +21,21 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
-def _stream() -> C.c_void_p:
-    """torch's current stream on the current device (every kernel of the path is launched on it).  Called a dozen
-    times per layer: the raw accessors cost a fraction of torch.cuda.current_stream()."""
+def _stream_handle(device=None) -> int:
+    """Raw handle of torch's current stream on the current device.  Every kernel of the path is launched on it, so
+    tensors of another device are refused rather than launched on a stream that does not belong to them.  Called a
+    dozen times per layer: the raw accessors cost a fraction of torch.cuda.current_stream()."""
     if _raw_stream is not None and _raw_device is not None:
-        return C.c_void_p(_raw_stream(_raw_device()))
-    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        cur = _raw_device()
+        if device is not None and device.index is not None and device.index != cur:
+            raise ValueError(f"tensors live on cuda:{device.index} but the current device is cuda:{cur}; "
+                             "run the call under torch.cuda.device(...)")
+        return int(_raw_stream(cur))
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _stream(device=None) -> C.c_void_p:
+    return C.c_void_p(_stream_handle(device))
 
 
 def _ptr(t: Optional[torch.Tensor]) -> C.c_void_p:
@@ -54,7 +63,7 @@ def pool_avg(x: torch.Tensor, block_size: int, tail_mode: int = _lib.SP_POOL_TAI
     if out is None:
         out = torch.empty(nb, h, d, dtype=torch.bfloat16, device=x.device)
     st = lib.sp_pool_avg_bf16(_ptr(x), _ptr(out), n, h, d, x.stride(1), x.stride(0), block_size, tail_mode,
-                              _ptr(head_enable), _stream())
+                              _ptr(head_enable), _stream(x.device))
     _lib.check(st, "sp_pool_avg_bf16")
     return out
 
@@ -63,13 +72,22 @@ _workspaces = {}
 
 
 def _workspace(tag: str, nbytes: int, device) -> torch.Tensor:
-    """Grow-only scratch buffers keyed by purpose and device (reused across layers)."""
-    key = (tag, str(device))
+    """Grow-only scratch buffers keyed by purpose, device AND stream (reused across layers).  Work on one stream is
+    ordered, so consecutive calls may share a buffer; two streams of one device (two models, two threads) get
+    buffers of their own and cannot race on the scheduler tickets or the repacked V they hold."""
+    key = (tag, str(device), _stream_handle(device))
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
+
+
+def release_workspaces(device=None) -> None:
+    """Drops the cached scratch buffers (all of them, or one device's).  Synchronise first: kernels still running
+    on a buffer's stream keep using it."""
+    for key in [k for k in _workspaces if device is None or k[1] == str(device)]:
+        del _workspaces[key]
 
 
 def lastq_scores(q: torch.Tensor, k: torch.Tensor, block_size: int, flags: int = _lib.SP_FLAG_LOGITS_BF16):
@@ -91,7 +109,7 @@ def lastq_scores(q: torch.Tensor, k: torch.Tensor, block_size: int, flags: int =
     ws = _workspace("lastq", need, dev)
     st = lib.sp_lastq_scores_bf16(_ptr(q), _ptr(k), n, hq, hkv, d, q.stride(1), q.stride(0), k.stride(1), k.stride(0),
                                   block_size, flags, _ptr(ws), ws.numel(), _ptr(vert_tok), _ptr(slash_tok),
-                                  _ptr(vert_blk), _ptr(slash_blk), _stream())
+                                  _ptr(vert_blk), _ptr(slash_blk), _stream(dev))
     _lib.check(st, "sp_lastq_scores_bf16")
     return vert_tok, slash_tok, vert_blk, slash_blk
 
@@ -102,7 +120,7 @@ def cover_count(x: torch.Tensor, thr: float) -> torch.Tensor:
     assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and x.is_cuda
     out = torch.empty(x.shape[0], dtype=torch.int32, device=x.device)
     ws = _workspace("cover_select", lib.sp_cover_select_workspace_bytes(x.shape[0]), x.device)
-    _lib.check(lib.sp_cover_count(_ptr(x), x.shape[0], x.shape[1], thr, _ptr(out), _ptr(ws), ws.numel(), _stream()),
+    _lib.check(lib.sp_cover_count(_ptr(x), x.shape[0], x.shape[1], thr, _ptr(out), _ptr(ws), ws.numel(), _stream(x.device)),
                "sp_cover_count")
     return out
 
@@ -116,7 +134,7 @@ def cover_budgets(vert_tok, slash_tok, block_size, pattern_threshold, min_blocks
     ns = torch.empty(hq, dtype=torch.int32, device=vert_tok.device)
     ws = _workspace("cover_select", lib.sp_cover_select_workspace_bytes(2 * hq), vert_tok.device)
     st = lib.sp_cover_budgets(_ptr(vert_tok), _ptr(slash_tok), hq, n, block_size, pattern_threshold, min_blocks,
-                              max_blocks, _ptr(nv), _ptr(ns), _ptr(ws), ws.numel(), _stream())
+                              max_blocks, _ptr(nv), _ptr(ns), _ptr(ws), ws.numel(), _stream(vert_tok.device))
     _lib.check(st, "sp_cover_budgets")
     return nv, ns
 
@@ -134,7 +152,7 @@ def queryaware_test(q, kbar, vert_blk, block_size, queryaware_threshold, flags=_
     use = torch.empty(hq, dtype=torch.int32, device=dev)
     st = lib.sp_queryaware_test_bf16(_ptr(q), _ptr(kbar), _ptr(vert_blk), n, hq, hkv, d, q.stride(1), q.stride(0),
                                      block_size, flags, queryaware_threshold, _ptr(avg_qk), _ptr(js), _ptr(use),
-                                     _stream())
+                                     _stream(dev))
     _lib.check(st, "sp_queryaware_test_bf16")
     return avg_qk, js, use
 
@@ -180,7 +198,7 @@ def share_decide(state: ClusterState, head_cluster, layer_idx, vert_blk, slash_b
     ns_f = torch.empty(hq, dtype=torch.int32, device=dev)
     st = lib.sp_share_decide(state.ref(), _ptr(head_cluster), layer_idx, hq, _ptr(vert_blk), _ptr(slash_blk),
                              _ptr(use_qa), _ptr(nv), _ptr(ns), min_blocks, similarity_threshold, fallback_threshold,
-                             _ptr(decision), _ptr(js_v), _ptr(js_s), _ptr(nv_f), _ptr(ns_f), _stream())
+                             _ptr(decision), _ptr(js_v), _ptr(js_s), _ptr(nv_f), _ptr(ns_f), _stream(dev))
     _lib.check(st, "sp_share_decide")
     return decision, js_v, js_s, nv_f, ns_f
 
@@ -191,7 +209,7 @@ def build_mask(state: ClusterState, head_cluster, decision, vert_blk, slash_blk,
     hq, nb = vert_blk.shape
     mask = torch.empty(hq, nb, (nb + 63) // 64, dtype=torch.int64, device=vert_blk.device)
     st = lib.sp_build_mask(state.ref(), _ptr(head_cluster), _ptr(decision), _ptr(vert_blk), _ptr(slash_blk),
-                           _ptr(nv_f), _ptr(ns_f), hq, nb, _ptr(mask), _stream())
+                           _ptr(nv_f), _ptr(ns_f), hq, nb, _ptr(mask), _stream(vert_blk.device))
     _lib.check(st, "sp_build_mask")
     return mask
 
@@ -206,7 +224,7 @@ def queryaware_select(qbar, kbar, decision, mask, pattern_threshold, flags=_lib.
         probs = torch.empty(hq, nb, nb, dtype=torch.float32, device=qbar.device)
     ws = _workspace("cover_select", lib.sp_cover_select_workspace_bytes(hq), qbar.device)
     st = lib.sp_queryaware_select_bf16(_ptr(qbar), _ptr(kbar), _ptr(decision), hq, hkv, d, nb, flags,
-                                       pattern_threshold, _ptr(probs), _ptr(mask), _ptr(ws), ws.numel(), _stream())
+                                       pattern_threshold, _ptr(probs), _ptr(mask), _ptr(ws), ws.numel(), _stream(qbar.device))
     _lib.check(st, "sp_queryaware_select_bf16")
     return probs
 
@@ -217,7 +235,7 @@ def cover_select_global(x: torch.Tensor, score: float, mask: torch.Tensor, enabl
     assert x.dtype == torch.float32 and x.is_contiguous() and mask.is_contiguous()
     v, nb, _ = x.shape
     ws = _workspace("cover_select", lib.sp_cover_select_workspace_bytes(v), x.device)
-    st = lib.sp_cover_select_global(_ptr(x), _ptr(enable), v, nb, score, _ptr(mask), _ptr(ws), ws.numel(), _stream())
+    st = lib.sp_cover_select_global(_ptr(x), _ptr(enable), v, nb, score, _ptr(mask), _ptr(ws), ws.numel(), _stream(x.device))
     _lib.check(st, "sp_cover_select_global")
     return mask
 
@@ -228,7 +246,7 @@ def cover_select_rows(x: torch.Tensor, thr: float) -> torch.Tensor:
     assert x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
     nb = x.shape[0]
     pat = torch.empty(nb, (nb + 63) // 64, dtype=torch.int64, device=x.device)
-    _lib.check(lib.sp_cover_select_rows(_ptr(x), nb, thr, _ptr(pat), _stream()), "sp_cover_select_rows")
+    _lib.check(lib.sp_cover_select_rows(_ptr(x), nb, thr, _ptr(pat), _stream(x.device)), "sp_cover_select_rows")
     return pat
 
 
@@ -254,7 +272,7 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
         need = (need + 255) // 256 * 256 + min(max_pivots, hq) * lib.sp_attn_pivot_scratch_bytes(n, block_size)
     ws = _workspace("attn_vt", need, dev)
     st = lib.sp_attn_repack_v_bf16(_ptr(v), n, hkv, d, v.stride(1), v.stride(0), block_size, _ptr(ws), ws.numel(),
-                                   _stream())
+                                   _stream(dev))
     _lib.check(st, "sp_attn_repack_v_bf16")
     timer = kernel_timer
     if timer is not None:
@@ -262,14 +280,15 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
     st = lib.sp_block_sparse_attn_fwd_bf16(_ptr(q), _ptr(k), _ptr(v), n, hq, hkv, d, q.stride(1), q.stride(0),
                                            k.stride(1), k.stride(0), v.stride(1), v.stride(0), block_size,
                                            softmax_scale, _ptr(mask), _ptr(decision), _ptr(out), _ptr(avg_attn),
-                                           _ptr(ws), need, _lib.SP_ATTN_V_REPACKED, _stream())
+                                           _ptr(ws), need, _lib.SP_ATTN_V_REPACKED, _stream(dev))
     if timer is not None:
         timer.stop("attn")
     _lib.check(st, "sp_block_sparse_attn_fwd_bf16")
     return out
 
 
-def decode_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float) -> torch.Tensor:
+def decode_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q bf16 [Hq, D] (one token), k / v bf16 [Hkv, N, D] views -> out bf16 [Hq, D].
 
     Reference: the flash_attn_func decode branch (shareprefill_attn.py:146-155)."""
@@ -280,10 +299,14 @@ def decode_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_
     hkv, n, _ = k.shape
     if q.dtype != torch.bfloat16 or q.stride(1) != 1:
         raise ValueError("q must be bfloat16 [Hq, D] with a contiguous head_dim axis")
-    out = torch.empty(hq, d, dtype=torch.bfloat16, device=q.device)
+    if out is None:
+        out = torch.empty(hq, d, dtype=torch.bfloat16, device=q.device)
+    elif out.dtype != torch.bfloat16 or tuple(out.shape) != (hq, d) or not out.is_contiguous() or out.device != q.device:
+        raise ValueError(f"out must be a contiguous bfloat16 [{hq}, {d}] tensor on {q.device}")
     ws = _workspace("decode", lib.sp_decode_workspace_bytes(n, hq, hkv), q.device)
     st = lib.sp_decode_attn_bf16(_ptr(q), _ptr(k), _ptr(v), n, hq, hkv, d, q.stride(0), k.stride(1), k.stride(0),
-                                 v.stride(1), v.stride(0), softmax_scale, _ptr(out), _ptr(ws), ws.numel(), _stream())
+                                 v.stride(1), v.stride(0), softmax_scale, _ptr(out), _ptr(ws), ws.numel(),
+                                 _stream(q.device))
     _lib.check(st, "sp_decode_attn_bf16")
     return out
 
@@ -307,7 +330,7 @@ def rope_inplace(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch
     if n > 1 and cos.stride(0) != sin.stride(0):
         raise ValueError("cos and sin must share their row stride")
     st = lib.sp_rope_inplace_bf16(_ptr(q), _ptr(k), _ptr(cos), _ptr(sin), n, hq, hkv, d, q.stride(1), q.stride(0),
-                                  k.stride(1), k.stride(0), cos.stride(0) if n > 1 else d, _stream())
+                                  k.stride(1), k.stride(0), cos.stride(0) if n > 1 else d, _stream(q.device))
     _lib.check(st, "sp_rope_inplace_bf16")
 
 
@@ -316,11 +339,11 @@ def attention_clock_mhz(n: int, hkv: int, d: int, block_size: int, device) -> fl
     (measurement aid; synchronises the current stream)."""
     import ctypes
     lib = _lib.load()
-    ws = _workspaces.get(("attn_vt", str(device)))
+    ws = _workspaces.get(("attn_vt", str(device), _stream_handle(device)))
     if ws is None:
-        raise RuntimeError("no attention launch on this device yet")
+        raise RuntimeError("no attention launch on this device and stream yet")
     buf = (ctypes.c_int64 * 2)()
-    st = lib.sp_attn_last_launch_clocks(_ptr(ws), n, hkv, d, block_size, ctypes.cast(buf, ctypes.c_void_p), _stream())
+    st = lib.sp_attn_last_launch_clocks(_ptr(ws), n, hkv, d, block_size, ctypes.cast(buf, ctypes.c_void_p), _stream(device))
     _lib.check(st, "sp_attn_last_launch_clocks")
     return float(buf[0]) / (float(buf[1]) / 100.0) if buf[1] > 0 else float("nan")
 
@@ -331,12 +354,12 @@ def attention_pairing(n: int, hq: int, hkv: int, d: int, block_size: int, device
     synchronises the current stream)."""
     import ctypes
     lib = _lib.load()
-    ws = _workspaces.get(("attn_vt", str(device)))
+    ws = _workspaces.get(("attn_vt", str(device), _stream_handle(device)))
     if ws is None:
-        raise RuntimeError("no attention launch on this device yet")
+        raise RuntimeError("no attention launch on this device and stream yet")
     buf = (ctypes.c_uint8 * ((hq + 1) // 2))()
     st = lib.sp_attn_last_launch_pairing(_ptr(ws), n, hq, hkv, d, block_size, ctypes.cast(buf, ctypes.c_void_p),
-                                         _stream())
+                                         _stream(device))
     _lib.check(st, "sp_attn_last_launch_pairing")
     return [bool(x) for x in buf]
 
@@ -387,7 +410,7 @@ def pivot_update(state: ClusterState, head_cluster, decision, avg_attn, pattern_
     lib = _lib.load()
     hq, nb, _ = avg_attn.shape
     st = lib.sp_pivot_update(state.ref(), _ptr(head_cluster), _ptr(decision), _ptr(avg_attn), hq, nb,
-                             pattern_threshold, _stream())
+                             pattern_threshold, _stream(avg_attn.device))
     _lib.check(st, "sp_pivot_update")
 
 
@@ -396,7 +419,7 @@ def mask_row_pointers(mask: torch.Tensor) -> torch.Tensor:
     lib = _lib.load()
     hq, nb, _ = mask.shape
     out = torch.empty(hq, nb + 1, dtype=torch.int32, device=mask.device)
-    _lib.check(lib.sp_mask_row_pointers(_ptr(mask), hq, nb, _ptr(out), _stream()), "sp_mask_row_pointers")
+    _lib.check(lib.sp_mask_row_pointers(_ptr(mask), hq, nb, _ptr(out), _stream(mask.device)), "sp_mask_row_pointers")
     return out
 
 

@@ -20,7 +20,6 @@ from . import _lib, ops
 from .attention_sharing import budget_blocks
 
 LOGGER = logging.getLogger(__name__)
-_warned_decode = False
 
 
 def _dense_causal_mask(hq: int, nb: int, device) -> torch.Tensor:
@@ -43,26 +42,14 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
         raise NotImplementedError("gqa_interleave=True (query head h -> kv head h % Hkv) is not supported")
 
     if q_len == 1:
-        # decode step (shareprefill_attn.py:146-155): one query against the whole cache, nothing is selected
-        hkv = key_states.shape[1]
-        native = (query_states.dtype == torch.bfloat16 and head_dim == 128 and num_heads % hkv == 0
-                  and num_heads // hkv <= 8 and key_states.stride(3) == 1 and value_states.stride(3) == 1
-                  and key_states.stride(2) % 8 == 0 and value_states.stride(2) % 8 == 0)
-        if native:
-            outs = [ops.decode_attention(query_states[b, :, 0], key_states[b], value_states[b], softmax_scale)
-                    for b in range(bsz)]
-            return torch.stack(outs).unsqueeze(2), None
-        global _warned_decode
-        if not _warned_decode:
-            _warned_decode = True
-            LOGGER.warning("SharePrefill decode step: %s head_dim %d with %d query heads per kv head is outside the HIP "
-                           "decode kernel (bf16, head_dim 128, at most 8 per kv head); using torch's "
-                           "scaled_dot_product_attention on the GPU for this model.", query_states.dtype, head_dim,
-                           num_heads // max(hkv, 1))
-        out = torch.nn.functional.scaled_dot_product_attention(
-            query_states, key_states, value_states, dropout_p=0.0, is_causal=False, scale=softmax_scale,
-            enable_gqa=hkv != num_heads)
-        return out, None
+        # decode step (shareprefill_attn.py:146-155): one query against the whole cache, nothing is selected.
+        # The HIP kernel is the only path (bf16, head_dim 128, at most 32 query heads per kv head, 16-byte aligned
+        # rows); anything else raises from the entry point's own checks, as every other unsupported shape does.
+        if query_states.dtype != torch.bfloat16:
+            raise AssertionError(f"SharePrefill attention expects bfloat16 q/k/v, got {query_states.dtype}")
+        outs = [ops.decode_attention(query_states[b, :, 0], key_states[b], value_states[b], softmax_scale)
+                for b in range(bsz)]
+        return torch.stack(outs).unsqueeze(2), None
 
     if bsz != 1:
         raise ValueError("SharePrefill prefill keeps per-cluster state for batch size 1 only")

@@ -28,7 +28,7 @@ def _inputs(hq, hkv, n, seed, token_major=True):
 
 
 @pytest.mark.parametrize("hq,hkv,n", [(32, 8, 4096), (28, 4, 1000), (8, 8, 129), (4, 1, 1), (16, 2, 70000),
-                                      (8, 1, 127)])
+                                      (8, 1, 127), (18, 2, 3000), (64, 4, 2500), (24, 1, 777), (64, 2, 4096)])
 @pytest.mark.parametrize("token_major", [True, False])
 def test_decode_matches_oracle(gpu_device, hq, hkv, n, token_major):
     from shareprefill_amd import ops
@@ -62,9 +62,14 @@ def test_decode_peaked_and_large_logits(gpu_device):
 def test_decode_rejects_unsupported(gpu_device):
     from shareprefill_amd import ops
 
-    q, k, v = _inputs(9, 1, 256, 1)
+    q, k, v = _inputs(33, 1, 256, 1)
     with pytest.raises(NotImplementedError):
-        ops.decode_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), 0.1)  # 9 heads per kv head
+        ops.decode_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), 0.1)  # 33 heads per kv head
+    q, k, v = _inputs(4, 2, 256, 1)
+    qg = torch.zeros(4, 132, dtype=torch.bfloat16, device=gpu_device)[:, 4:]  # rows start 8 bytes off a 16-byte line
+    qg.copy_(q)
+    with pytest.raises(NotImplementedError):
+        ops.decode_attention(qg, k.to(gpu_device), v.to(gpu_device), 0.1)
     q, k, v = _inputs(4, 2, 256, 1)
     with pytest.raises(ValueError):
         ops.decode_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), 0.0)

@@ -30,6 +30,7 @@ def c3(gpu_device, tmp_path_factory):
     table = synthetic.random_cluster_table(w.hq, w.n_clusters, 2, w.seed)
     path = synthetic.write_cluster_table(table, str(tmp_path_factory.mktemp("c3") / "table.json"))
     sharing = AttentionSharing(path)
+    sharing.keep_plans = True  # both layers' masks are inspected below
     cfg = types.SimpleNamespace(block_size=128, min_budget=w.min_budget, max_budget=None,
                                 pattern_threshold=w.pattern_threshold, similarity_threshold=w.similarity_threshold,
                                 fallback_threshold=w.fallback_threshold, queryaware_threshold=w.queryaware_threshold)
@@ -188,3 +189,68 @@ def test_maximum_supported_length_selection_bit_exact_and_rows_within_tolerance(
         qq = torch.zeros(1, 4097 * 128, 128, dtype=torch.bfloat16, device=gpu_device)
         mm = torch.zeros(1, 4097, 65, dtype=torch.int64, device=gpu_device)
         ops.block_sparse_attention(qq, qq, qq, mm, 128, scale)
+
+
+def _layer_helpers():
+    import importlib.util
+    import os
+
+    spec = importlib.util.spec_from_file_location(
+        "layer_helpers_full", os.path.join(os.path.dirname(__file__), "test_gpu_layer.py"))
+    helpers = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(helpers)
+    return helpers
+
+
+@pytest.mark.parametrize("name", ["C3", "C5"])
+def test_sharing_and_query_aware_heads_at_full_size_bit_exact(gpu_device, tmp_path, name):
+    """The share test, the pattern OR of the mask construction and the query-aware selection over nb^2 = 1 M (C3,
+    131072 tokens) and 4.2 M (C5, 262144 tokens, GQA 7:1) block probabilities, at the benchmark shapes.  With the
+    library's default thresholds no head of these synthetic inputs shares or goes query-aware, so the thresholds are
+    placed where they do: fallback_threshold is lifted (a local-attention pivot has vs_ratio >= (nb-1)/nb) and
+    queryaware_threshold is put between the heads' own sqrt-JS values so that a quarter of the heads take the
+    query-aware path.  Two layers (pivot election, then sharing): budgets, decisions, masks, pivot patterns and
+    coverage ratios must equal the oracle's integer logic on the GPU's own scores, every decision kind must occur,
+    and single query blocks of a shared and of a query-aware head are held to the attention tolerances."""
+    import numpy as np
+
+    from oracle import shareprefill_oracle as O
+
+    helpers = _layer_helpers()
+    w = synthetic.WORKLOADS[name]
+    kw = dict(hq=w.hq, hkv=w.hkv, n=w.seq_len, seed=w.seed, n_clusters=w.n_clusters, with_free=False,
+              pattern_threshold=w.pattern_threshold)
+    print(f"full-size sharing / query-aware parity: {name} probe layer", flush=True)
+    probe = helpers.run_layers(gpu_device, tmp_path, n_layers=1, with_forced=False, **kw)
+    js = np.sort(probe["layers"][0]["plan"].js_qa.cpu().numpy())
+    assert np.isfinite(js).all()
+    n_qa = w.hq // 4
+    assert js[n_qa] > js[n_qa - 1], "the two sqrt-JS values around the threshold coincide"
+    qat = float((js[n_qa - 1].astype(np.float64) + js[n_qa].astype(np.float64)) / 2)
+    del probe
+    torch.cuda.empty_cache()
+    print(f"full-size sharing / query-aware parity: {name} two layers, queryaware_threshold {qat:.6f}", flush=True)
+    run = helpers.run_layers(gpu_device, tmp_path, fallback_threshold=1e9, queryaware_threshold=qat, **kw)
+    helpers.check_forced(run)
+    d0, d1 = run["layers"][0]["dec"], run["layers"][1]["dec"]
+    assert (d0 == O.DEC_QA).sum() == n_qa and (d1 == O.DEC_QA).sum() == n_qa
+    assert (d0 == O.DEC_DENSE).sum() >= 1 and (d0 == O.DEC_SHARE).sum() == 0
+    assert (d1 == O.DEC_SHARE).sum() >= 1, "no head shared its cluster pivot's pattern in the second layer"
+    assert (d1 == O.DEC_VS).sum() + (d1 == O.DEC_SHARE).sum() + n_qa == w.hq
+    # a shared head's mask is the pivot's pattern OR its own minimum-budget vertical-slash set: strictly more than
+    # the latter alone
+    nb = run["nb"]
+    h_share = int(np.nonzero(d1 == O.DEC_SHARE)[0][0])
+    h_qa = int(np.nonzero(d1 == O.DEC_QA)[0][0])
+    assert run["layers"][1]["mask"][h_share].sum() > 3 * nb
+    q, k, v = (run[x][None].to(gpu_device) for x in ("q", "k", "v"))
+    scale = 1.0 / math.sqrt(128)
+    L = run["layers"][1]
+    mb = torch.from_numpy(L["mask"]).to(gpu_device)
+    out = L["out"][0].to(gpu_device)  # [N, Hq, D]
+    for h in (h_share, h_qa):
+        for r in (nb - 1, nb // 2 + 1, 3):
+            ref = _rows_reference(q, k, v, mb[h, r], h, r, w.hq // w.hkv, scale)
+            got = out[r * 128:(r + 1) * 128, h].float()
+            assert (got - ref).abs().max().item() <= MAX_ABS
+            assert ((got - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL

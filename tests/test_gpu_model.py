@@ -55,6 +55,7 @@ def test_patched_model_sparse_prefill_and_generate(gpu_device, tmp_path):
     model = SharePrefill(sharing_lookup_path=table(tmp_path, 2, 4), pattern_threshold=0.9, min_budget=256)(
         small_llama().to(gpu_device, torch.bfloat16))
     ids = torch.randint(0, 512, (1, 2048), generator=torch.Generator().manual_seed(2)).to(gpu_device)
+    model.attention_sharing.keep_plans = True  # every layer's mask is read below
     with torch.no_grad():
         logits = model(ids, use_cache=False, logits_to_keep=1).logits
     assert logits.shape == (1, 1, 512) and torch.isfinite(logits).all()

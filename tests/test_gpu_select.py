@@ -54,7 +54,7 @@ def test_budgets_bit_exact(gpu_device, hq, n):
     assert nv.cpu().tolist() == want(v) and ns.cpu().tolist() == want(s)
 
 
-@pytest.mark.parametrize("nb", [16, 64, 100, 256])
+@pytest.mark.parametrize("nb", [16, 64, 100, 256, 1024, 2048])
 @pytest.mark.parametrize("thr", [0.9, 0.95])
 def test_cover_select_global_bit_exact(gpu_device, nb, thr):
     from shareprefill_amd import ops
@@ -166,3 +166,61 @@ def test_row_pointers_docstring_vector(gpu_device):
     m = ops.bool_to_mask(b).to(gpu_device)
     assert ops.mask_row_pointers(m).cpu().tolist() == [v["row_pointers"]]
     assert ops.mask_to_block_idx(m, v["grid"])[0].cpu().tolist() == v["block_ids"]
+
+
+def test_heads_without_a_cluster_slot_never_touch_the_state(gpu_device):
+    """head_cluster[h] = -1 (no shared cluster) is legal for every head, also for one a caller marks dense or
+    shared in its own decision vector, and values >= n_clusters are a caller's mistake: neither may be used as an
+    index into the state slabs.  The state is surrounded by canaries here; a dense head with slot -1 (which would
+    write accum[-2], the pattern slab before slot 0 and ratio[-1]) and one with slot n_clusters must leave every slab
+    and every canary as it was, while the one dense head with a valid slot is processed."""
+    from shareprefill_amd import ops
+
+    hq, nb, c = 6, 40, 2
+    nbw = 1
+    g = torch.Generator().manual_seed(19)
+    state = ops.ClusterState(c, nb, gpu_device)
+
+    def guarded(shape, dtype, fill):
+        """a slab with one slot of canary in front and one behind; returns (whole buffer, view of the middle)"""
+        buf = torch.full((c + 2, *shape), fill, dtype=dtype, device=gpu_device)
+        return buf, buf[1:c + 1]
+
+    bufs = {}
+    for name, shape, dtype, fill in (("info", (8,), torch.int32, 77), ("ratio", (), torch.float64, 7.5),
+                                     ("vert", (nb,), torch.float32, 7.5), ("slash", (nb,), torch.float32, 7.5),
+                                     ("cols", (nb,), torch.uint8, 7), ("dists", (nb,), torch.uint8, 7),
+                                     ("pattern", (nb, nbw), torch.int64, 77), ("accum", (2,), torch.int64, 77)):
+        bufs[name], mid = guarded(shape, dtype, fill)
+        mid.copy_(getattr(state, name))
+        setattr(state, name, mid)
+    state.struct = ops.ClusterStateStruct(c, nb, nbw, 0, *(getattr(state, n).data_ptr() for n in
+                                          ("info", "ratio", "vert", "slash", "cols", "dists", "pattern", "accum")))
+    state.reset()
+    hc = torch.tensor([-1, 0, 2, -1, 1, 57], dtype=torch.int32, device=gpu_device)
+    vert = torch.softmax(torch.randn(hq, nb, generator=g) * 2, -1).to(gpu_device)
+    slash = torch.softmax(torch.randn(hq, nb, generator=g) * 2, -1).to(gpu_device)
+    nv = torch.full((hq,), 4, dtype=torch.int32, device=gpu_device)
+    use_qa = torch.zeros(hq, dtype=torch.int32, device=gpu_device)
+    dec, _, _, nvf, nsf = ops.share_decide(state, hc, 0, vert, slash, use_qa, nv, nv, 3, 0.5, 0.9)
+    # only the heads with slots 0 and 1 can become pivots; slot 2 and 57 do not exist, -1 is "no cluster"
+    assert dec.cpu().tolist() == [O.DEC_VS, O.DEC_DENSE, O.DEC_VS, O.DEC_VS, O.DEC_DENSE, O.DEC_VS]
+    before = {k: v.clone() for k, v in bufs.items()}
+    # a caller's own decision vector: dense and shared heads without a valid slot
+    mine = torch.tensor([O.DEC_DENSE, O.DEC_VS, O.DEC_DENSE, O.DEC_SHARE, O.DEC_VS, O.DEC_DENSE], dtype=torch.int32,
+                        device=gpu_device)
+    tri = torch.tril(torch.ones(nb, nb, device=gpu_device))
+    avg = (tri / tri.sum(-1, keepdim=True)).expand(hq, nb, nb).contiguous()
+    ops.pivot_update(state, hc, mine, avg, 0.9)
+    mask = ops.mask_to_bool(ops.build_mask(state, hc, mine, vert, slash, nvf, nsf), nb)
+    torch.cuda.synchronize()
+    for k, v in bufs.items():
+        assert torch.equal(v, before[k]), f"slab {k} changed although no head had a valid slot"
+    assert mask[0].cpu().equal(tri.bool().cpu())          # dense is dense, with or without a slot
+    assert mask[3, :, 0].all() and not torch.triu(mask[3], 1).any()  # SHARE without a slot: its own vertical-slash set
+    # the same call with the valid pivots does update their slots and nothing else
+    ops.pivot_update(state, hc, dec, avg, 0.9)
+    torch.cuda.synchronize()
+    assert state.info[:, 1].cpu().tolist() == [1, 1]
+    for k, v in bufs.items():
+        assert torch.equal(v[0], before[k][0]) and torch.equal(v[-1], before[k][-1]), f"canary of {k} overwritten"

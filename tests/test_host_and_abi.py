@@ -247,3 +247,115 @@ def test_synthetic_tables_and_generator_are_seeded():
     q1, k1, v1 = synthetic.planted_qkv(4, 2, 512, 128, 3)
     q2, _, _ = synthetic.planted_qkv(4, 2, 512, 128, 3)
     assert torch.equal(q1, q2) and q1.shape == (1, 4, 512, 128) and q1.stride(3) == 1 and q1.stride(1) == 128
+
+
+def test_reference_import_name_resolves_to_this_package():
+    """`from shareprefill import SharePrefill` (shareprefill/__init__.py:15-17 of the reference) and the reference's
+    module paths give the classes of this package."""
+    import shareprefill
+    import shareprefill_amd
+    from shareprefill import SharePrefill, SharePrefillConfig
+    from shareprefill.attn.attention_sharing import AttentionSharing
+    from shareprefill.attn.shareprefill_attn import shareprefill_attention_forward
+    from shareprefill.shareprefill_patch import shareprefill_patch
+
+    assert SharePrefill is shareprefill_amd.SharePrefill and SharePrefillConfig is shareprefill_amd.SharePrefillConfig
+    assert AttentionSharing is shareprefill_amd.AttentionSharing
+    assert shareprefill_attention_forward is shareprefill_amd.shareprefill_attention_forward
+    assert callable(shareprefill_patch) and shareprefill.attn.AttentionSharing is AttentionSharing
+
+
+def test_unpatch_restores_the_model(tmp_path):
+    from shareprefill_amd import SharePrefill, unpatch_model
+
+    model = tiny_llama()
+    before_impl = model.config._attn_implementation
+    before_forward = model.forward.__func__
+    SharePrefill(sharing_lookup_path=tiny_table(tmp_path), fuse_rope=True)(model)
+    assert model.config._attn_implementation == "shareprefill" and model.forward.__func__ is not before_forward
+    from transformers.models.llama import modeling_llama
+    try:
+        assert unpatch_model(model) is model
+        assert model.config._attn_implementation == before_impl
+        assert model.forward.__func__ is before_forward
+        assert not hasattr(model.model.layers[0].self_attn, "attention_sharing")
+        ids = torch.randint(0, 128, (1, 16))
+        assert model(ids).logits.shape == (1, 16, 128)  # runs on the CPU again: nothing of the patch is left
+        unpatch_model(model)  # a second call is a no-op
+    finally:
+        stock = getattr(modeling_llama.apply_rotary_pos_emb, "_shareprefill_original", None)
+        if stock is not None:
+            modeling_llama.apply_rotary_pos_emb = stock
+
+
+def test_fused_rope_is_taken_only_inside_a_patched_forward(tmp_path, monkeypatch):
+    """The module-level wrapper that fuse_rope=True installs hands every call to the stock function unless a forward
+    of a model patched with fuse_rope=True is on the stack: unpatched models of the architecture are not affected,
+    and call forms the wrapper does not know (keywords, extra arguments) go to the stock function as they are."""
+    from shareprefill_amd import SharePrefill, ops, shareprefill_patch as sp
+    from transformers.models.llama import modeling_llama
+
+    stock = modeling_llama.apply_rotary_pos_emb
+    calls = []
+    monkeypatch.setattr(ops, "rope_inplace", lambda *a: calls.append(a))
+    try:
+        model = SharePrefill(sharing_lookup_path=tiny_table(tmp_path), fuse_rope=True)(tiny_llama())
+        wrapped = modeling_llama.apply_rotary_pos_emb
+        g = torch.Generator().manual_seed(0)
+        q, k = torch.randn(1, 4, 9, 32, generator=g), torch.randn(1, 2, 9, 32, generator=g)
+        cos, sin = torch.randn(1, 9, 32, generator=g), torch.randn(1, 9, 32, generator=g)
+        a = wrapped(q, k, cos=cos, sin=sin)          # keyword form: straight to the stock function
+        b = stock(q, k, cos, sin)
+        assert torch.equal(a[0], b[0])
+        a = wrapped(q, k, cos, sin, unsqueeze_dim=1)
+        assert torch.equal(a[0], b[0]) and not calls
+        # outside a patched forward the depth counter is zero
+        assert getattr(sp._fused_rope_depth, "n", 0) == 0
+        seen = []
+        monkeypatch.setattr(model.model, "forward", lambda *a, **kw: seen.append(sp._fused_rope_depth.n) or 1 / 0)
+        with pytest.raises(ZeroDivisionError):
+            model(torch.zeros(1, 4, dtype=torch.long))
+        assert seen == [1] and sp._fused_rope_depth.n == 0  # set during the forward, restored when it raises
+        plain = SharePrefill(sharing_lookup_path=tiny_table(tmp_path))(tiny_llama())
+        seen.clear()
+        monkeypatch.setattr(plain.model, "forward", lambda *a, **kw: seen.append(getattr(sp._fused_rope_depth, "n", 0)) or 1 / 0)
+        with pytest.raises(ZeroDivisionError):
+            plain(torch.zeros(1, 4, dtype=torch.long))
+        assert seen == [0]  # a model patched without fuse_rope never switches the fused pass on
+    finally:
+        modeling_llama.apply_rotary_pos_emb = stock
+
+
+def test_update_pivotal_attns_masks_dense_flags_of_heads_without_a_slot(tmp_path, monkeypatch):
+    """A caller's bool use_dense may name heads outside every shared cluster (attention_sharing.py:94-103 would store
+    a pattern for any cluster id): those flags are dropped on the host before the device update."""
+    from shareprefill_amd import AttentionSharing, ops
+
+    sharing = AttentionSharing(tiny_table(tmp_path))  # head 0 in shared cluster "0", head 1 in unshared "1"
+    sharing._state = types.SimpleNamespace()
+    monkeypatch.setattr(sharing, "_head_cluster_tensor", lambda layer, hq, dev: torch.tensor([0, -1], dtype=torch.int32))
+    got = {}
+    monkeypatch.setattr(ops, "pivot_update", lambda st, hc, dec, avg, thr: got.update(dec=dec.tolist()))
+    avg = torch.zeros(1, 2, 4, 4)
+    sharing.update_pivotal_attns(0, avg, torch.tensor([[True, True]]), 0.9)
+    assert got["dec"] == [1, 0]
+    sharing.update_pivotal_attns(0, avg, torch.tensor([1, 1], dtype=torch.int32), 0.9)  # decision vector: as given
+    assert got["dec"] == [1, 1]
+
+
+def test_plans_release_older_masks_unless_asked_to_keep_them(tmp_path):
+    from shareprefill_amd import AttentionSharing
+    from shareprefill_amd.attention_sharing import LayerPlan
+
+    sharing = AttentionSharing(tiny_table(tmp_path))
+    mk = lambda i: LayerPlan(i, 2, torch.zeros(2, 2, 1, dtype=torch.int64), torch.zeros(2, dtype=torch.int32),
+                             None, None, None, None)
+    # plan_layer's bookkeeping, without the device work
+    for i in range(3):
+        if sharing.plans and not (sharing.keep_plans or sharing.keep_debug):
+            sharing.plans[-1].mask = None
+        sharing.plans.append(mk(i))
+    assert [p.mask is None for p in sharing.plans] == [True, True, False]
+    with pytest.raises(RuntimeError, match="keep_plans"):
+        sharing.plans[0].block_idx()
+    assert sharing.decision_histogram()["vertical_slash"] == 6  # the per-head decisions are kept

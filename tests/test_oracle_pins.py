@@ -440,3 +440,198 @@ def test_reset_state_clears_pivots():
     sh.layer(q, k, v, 0, **KW)
     sh.reset_state()
     assert sh.state["a"].pivot_head is None and sh.state["a"].pattern is None
+
+
+# ----- float stages of the query-aware path ------------------------------------------------------------
+def _all_bf16_values():
+    """Every one of the 65536 bf16 bit patterns, as a [65536] bf16 tensor."""
+    return torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+
+
+def _same_bits_or_both_nan(a, b):
+    a, b = a.contiguous(), b.contiguous()
+    same = a.view(torch.int16) == b.view(torch.int16)
+    return bool((same | (torch.isnan(a.float()) & torch.isnan(b.float()))).all())
+
+
+@pytest.mark.parametrize("d", [16, 32, 64, 128, 256])
+def test_scaled_last_q_is_torchs_tensor_by_float_division_exhaustively(d):
+    """attention_sharing.py:127 evaluates `q[:, -bs:] / math.sqrt(D)` on a bf16 tensor.  Checked against that very
+    expression (torch divides in fp32 and rounds to bf16) on EVERY bf16 value, so the multiply-by-reciprocal the
+    oracle and the kernels use instead of a true division is shown to give the same bits, also for D = 32 and 128
+    where sqrt(D) is no power of two."""
+    allv = _all_bf16_values()
+    bs = 128
+    q = allv.reshape(-1, bs, d)  # [Hq, N = bs, D]: the last block is the whole tensor
+    ref = q[:, -bs:] / math.sqrt(d)
+    assert ref.dtype == torch.bfloat16
+    assert _same_bits_or_both_nan(O.scaled_last_q(q, bs), ref)
+    # and only the last bs tokens are taken
+    q2 = torch.cat([torch.ones(q.shape[0], 5, d, dtype=torch.bfloat16), q], dim=1)
+    assert _same_bits_or_both_nan(O.scaled_last_q(q2, bs), ref)
+
+
+def test_pool_q_head_is_the_reference_expression_on_bf16():
+    """attention_sharing.py:350-356 literally (zero pad, view, mean, rescale the tail in place) on CPU bf16 tensors,
+    for every tail length; the tail's `* bs / (bs - pad)` is two bf16 roundings, which the oracle must reproduce."""
+    g = torch.Generator().manual_seed(21)
+    bs, d = 128, 16
+    for n in [128, 129, 200, 255, 256, 257, 300, 383]:
+        q = (torch.randn(n, d, generator=g) * 3).to(torch.bfloat16)
+        nb = math.ceil(n / bs)
+        pad_q = nb * bs - n
+        avg_q = torch.nn.functional.pad(q, (0, 0, 0, pad_q), value=0).view(nb, bs, d).mean(1)
+        avg_q[-1, :] = avg_q[-1, :] * bs / (bs - pad_q)
+        got = O.pool_q_head(q, bs)
+        assert got.dtype == torch.bfloat16
+        # the block means may differ by fp32 summation order (one bf16 ulp, rarely); the tail arithmetic on top of
+        # an identical mean must be identical, which the exhaustive check below covers
+        diff = (got.float() - avg_q.float()).abs()
+        assert (diff <= 2.0 ** -7 * avg_q.float().abs() + 1e-30).all()
+        assert (got.view(torch.int16) != avg_q.view(torch.int16)).float().mean().item() <= 0.02
+    # tail rescale alone, exhaustively: every bf16 mean value x every pad
+    allv = _all_bf16_values()
+    for pad in range(1, bs):
+        want = allv * bs / (bs - pad)
+        # the oracle's arithmetic for that step: fp32 product rounded to bf16, fp32 quotient rounded to bf16
+        mine = ((allv.float() * bs).to(torch.bfloat16).float() / (bs - pad)).to(torch.bfloat16)
+        assert _same_bits_or_both_nan(mine, want), pad
+    # and pool_q_head applies exactly that step to the tail block's mean
+    q = (torch.randn(130, d, generator=g)).to(torch.bfloat16)
+    tail_mean = torch.nn.functional.pad(q[128:], (0, 0, 0, 126)).float().mean(0).to(torch.bfloat16)
+    want = tail_mean * 128 / 2
+    assert _same_bits_or_both_nan(O.pool_q_head(q, 128)[1], want)
+
+
+def test_pooled_qk_probs_fp64_bruteforce_and_closed_forms():
+    """attention_sharing.py:197-200: softmax over the nb pooled keys of (mean of the last block's scaled queries) .
+    pooled key, query head h reading kv head h // g (repeat_interleave, :193-194)."""
+    g = torch.Generator().manual_seed(22)
+    hq, hkv, n, d, bs = 4, 2, 512, 16, 128
+    nb = n // bs
+    q = torch.randn(hq, n, d, generator=g)
+    k = torch.randn(hkv, n, d, generator=g)
+    kbar = O.pool_avg(k.transpose(0, 1).contiguous(), bs)  # [nb, Hkv, D]
+    got = O.pooled_qk_probs(q, kbar, bs, logits_in_input_dtype=False)
+    assert got.shape == (hq, nb) and got.dtype == torch.float32
+    ref = torch.zeros(hq, nb, dtype=torch.float64)
+    for h in range(hq):
+        qm = [sum(q[h, n - bs + i, c].item() / math.sqrt(d) for i in range(bs)) / bs for c in range(d)]
+        logits = [sum(qm[c] * kbar[j, h // 2, c].item() for c in range(d)) for j in range(nb)]
+        mx = max(logits)
+        e = [math.exp(x - mx) for x in logits]
+        for j in range(nb):
+            ref[h, j] = e[j] / sum(e)
+    assert torch.allclose(got.double(), ref, atol=2e-6)
+    assert torch.allclose(got.sum(-1), torch.ones(hq), atol=1e-6)
+    # a head mapping h % Hkv would give heads 1 and 2 each other's keys: the two mappings must be distinguishable here
+    wrong = torch.stack([ref[h] for h in (0, 2, 1, 3)])
+    assert (wrong - ref).abs().max().item() > 1e-3
+    # identical pooled keys -> every block gets 1/nb, whatever the queries
+    kconst = kbar[:1].expand(nb, hkv, d).contiguous()
+    assert torch.allclose(O.pooled_qk_probs(q, kconst, bs, logits_in_input_dtype=False),
+                          torch.full((hq, nb), 1.0 / nb), atol=1e-6)
+    # one pooled key aligned with the mean query and far longer than the others takes all the mass
+    kb2 = kbar.clone()
+    kb2[2, 0] = 1000.0 * q[0, -bs:].mean(0)
+    p = O.pooled_qk_probs(q, kb2, bs, logits_in_input_dtype=False)
+    assert p[0].argmax().item() == 2 and p[0, 2].item() > 0.999
+    # only the last block's queries matter
+    q2 = q.clone()
+    q2[:, : n - bs] = 0
+    assert torch.equal(O.pooled_qk_probs(q2, kbar, bs, logits_in_input_dtype=False), got)
+
+
+def test_pooled_qk_probs_bf16_logit_rounding_is_the_einsums():
+    """With bf16 inputs the reference's einsum returns bf16 logits (attention_sharing.py:197-199): compared with that
+    very einsum on CPU bf16 tensors (fp32 accumulation order may move a logit by one bf16 ulp, rarely)."""
+    g = torch.Generator().manual_seed(23)
+    hq, hkv, n, d, bs = 8, 2, 2048, 64, 128
+    q = torch.randn(hq, n, d, generator=g).to(torch.bfloat16)
+    k = torch.randn(hkv, n, d, generator=g).to(torch.bfloat16)
+    kbar = O.pool_avg(k.transpose(0, 1).contiguous(), bs)
+    last_q = (q[:, -bs:] / math.sqrt(d)).transpose(0, 1)[None]          # [1, bs, Hq, D] as in the reference
+    avg_k = kbar[None].repeat_interleave(hq // hkv, 2)                   # [1, nb, Hq, D]
+    lit = torch.einsum("bihd, bjhd -> bhij", last_q.mean(1, keepdim=True), avg_k).squeeze(2)
+    lit = torch.softmax(lit, dim=-1, dtype=torch.float32)[0]
+    got = O.pooled_qk_probs(q, kbar, bs, logits_in_input_dtype=True)
+    assert torch.allclose(got, lit, rtol=2.0 ** -6, atol=1e-7)  # one bf16 ulp of a logit of size <= 2 moves p by <= 2^-7
+    assert ((got - lit).abs() > 1e-6 * lit).float().mean().item() <= 0.05
+
+
+def test_block_probs_fp64_bruteforce_and_closed_forms():
+    """attention_sharing.py:357-360: rows of softmax((avg_q / sqrt(D)) . avg_k^T) under the block-causal mask."""
+    g = torch.Generator().manual_seed(24)
+    nb, d = 7, 16
+    qbar = torch.randn(nb, d, generator=g)
+    kbar = torch.randn(nb, d, generator=g)
+    got = O.block_probs(qbar, kbar, logits_in_input_dtype=False)
+    assert got.shape == (nb, nb) and got.dtype == torch.float32
+    for r in range(nb):
+        logits = [sum(qbar[r, c].item() / math.sqrt(d) * kbar[j, c].item() for c in range(d)) for j in range(r + 1)]
+        mx = max(logits)
+        e = [math.exp(x - mx) for x in logits]
+        for j in range(nb):
+            want = e[j] / sum(e) if j <= r else 0.0
+            assert math.isclose(got[r, j].item(), want, rel_tol=1e-5, abs_tol=1e-8), (r, j)
+    assert torch.allclose(got.sum(-1), torch.ones(nb), atol=1e-6)
+    assert (torch.triu(got, 1) == 0).all()
+    assert got[0, 0].item() == 1.0
+    # zero queries: row r is uniform over its r + 1 visible blocks
+    z = O.block_probs(torch.zeros(nb, d), kbar, logits_in_input_dtype=False)
+    for r in range(nb):
+        assert torch.allclose(z[r, : r + 1], torch.full((r + 1,), 1.0 / (r + 1)), atol=1e-7)
+    # transposed operands (k . q^T) must be caught: the matrix is not symmetric
+    swapped = O.block_probs(kbar, qbar, logits_in_input_dtype=False)
+    assert (swapped - got).abs().max().item() > 1e-3
+    # the scale matters: dropping 1/sqrt(D) changes the result
+    unscaled = O.block_probs(qbar * math.sqrt(d), kbar, logits_in_input_dtype=False)
+    assert (unscaled - got).abs().max().item() > 1e-3
+
+
+def test_block_probs_bf16_is_the_reference_expression():
+    """bf16 inputs: the literal expression of attention_sharing.py:357-360 on CPU bf16 tensors."""
+    g = torch.Generator().manual_seed(25)
+    nb, d = 24, 128
+    avg_q = torch.randn(nb, d, generator=g).to(torch.bfloat16)
+    avg_k = torch.randn(nb, d, generator=g).to(torch.bfloat16)
+    tri = torch.tril(torch.ones(nb, nb, dtype=torch.bool))
+    attn = torch.einsum("id, jd -> ij", avg_q / math.sqrt(d), avg_k).masked_fill_(~tri, float("-inf"))
+    lit = torch.softmax(attn, dim=-1, dtype=torch.float32)
+    got = O.block_probs(avg_q, avg_k, logits_in_input_dtype=True)
+    assert torch.allclose(got, lit, rtol=2.0 ** -5, atol=1e-7)
+    assert ((got - lit).abs() > 1e-6 * lit).float().mean().item() <= 0.05
+
+
+# ----- the reference kernel's own roundings ---------------------------------------------------------------
+def test_masked_attention_ref_roundings_against_fp32_and_exact_case():
+    """masked_attention_ref_roundings (shareprefill_attn.py:383-471 with its bf16 roundings) must sit within the
+    rounding noise of the fp32 oracle: the output rounding alone gives mean|d|/mean|x| ~ 1.4e-3, the bf16
+    probabilities add ~1.6e-3 in quadrature (2.06e-3 together); anything systematic (a dropped block, a wrong
+    rescale) shows in the bias, which rounding noise does not have.  On inputs whose probabilities are exact powers
+    of two the probability rounding vanishes and the result must equal the bf16 rounding of the fp32 oracle."""
+    g = torch.Generator().manual_seed(26)
+    hq, hkv, n, d, bs = 4, 2, 700, 64, 128
+    q, k, v = (torch.randn(h, n, d, generator=g).to(torch.bfloat16) for h in (hq, hkv, hkv))
+    nb = math.ceil(n / bs)
+    mask = np.tril(torch.rand(hq, nb, nb, generator=g).numpy() < 0.6)
+    mask[:, np.arange(nb), np.arange(nb)] = True
+    mask[:, :, 0] = True
+    scale = 1.0 / math.sqrt(d)
+    ref, _ = O.masked_attention(q, k, v, mask, bs, scale)
+    emu, _ = O.masked_attention(q, k, v, mask, bs, scale, emulate_bf16=True)
+    mean_rel = ((emu - ref).abs().mean() / ref.abs().mean()).item()
+    only_out = ((ref.to(torch.bfloat16).float() - ref).abs().mean() / ref.abs().mean()).item()
+    assert 1.2e-3 <= only_out <= 1.6e-3
+    assert only_out <= mean_rel <= 2.4e-3
+    assert abs((emu - ref).mean().item()) / ref.abs().mean().item() <= 1e-4
+    assert (emu - ref).abs().max().item() <= 2e-2
+    # exact case: integer logits in base-2 units (softmax_scale = ln 2, q and k with entries in {-1, 0, 1})
+    qi = torch.randint(-1, 2, (hq, n, d), generator=g).float() * (torch.rand(hq, n, d, generator=g) < 0.15)
+    ki = torch.randint(-1, 2, (hkv, n, d), generator=g).float() * (torch.rand(hkv, n, d, generator=g) < 0.3)
+    ref, _ = O.masked_attention(qi, ki, v, mask, bs, math.log(2.0))
+    emu = O.masked_attention_ref_roundings(qi, ki, v, mask, bs, math.log(2.0))
+    want = ref.to(torch.bfloat16)
+    neq = (emu.view(torch.int16) != want.view(torch.int16))
+    assert neq.float().mean().item() <= 2e-3          # a value within fp32 noise of a rounding boundary may flip
+    assert ((emu.float() - ref).abs().mean() / ref.abs().mean()).item() <= only_out * 1.05
