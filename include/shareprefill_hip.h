@@ -216,6 +216,21 @@ int sp_decode_attn_bf16(const void* q, const void* k, const void* v, int64_t n, 
                         int64_t v_stride_h, float softmax_scale, void* out, void* workspace,
                         size_t workspace_bytes, sp_stream_t stream);
 
+/* The same decode step for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no counterpart in the reference.  Identical arguments and results, but the chunk
+ * partials live in a device array built into the library (SP_DECODE_STATIC_SCRATCH_BYTES = 8 MiB per GPU, held
+ * until the process ends) instead of a caller's workspace; nothing is allocated or freed, here or in any routine it
+ * calls.  Shapes whose partials exceed the array (sp_decode_workspace_bytes(n, hq, hkv) > 8 MiB, e.g. more than about
+ * 16000 (chunk, head) pairs) are refused with SP_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls
+ * that overlap in time on one GPU (two streams, two threads) race; calls ordered on one stream are safe, and
+ * nothing needs clearing between them.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress); make that call outside graph capture. */
+#define SP_DECODE_STATIC_SCRATCH_BYTES (8u << 20)
+int sp_decode_attn_static_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,
+                               int32_t d, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                               int64_t v_stride_n, int64_t v_stride_h, float softmax_scale, void* out,
+                               sp_stream_t stream);
+
 /* ---- rotary position embedding in front of the attention function ---------------------------------
  * The reference's patched model produces (cos, sin) per position (model_patch.py:121) and leaves the rotation to
  * the Hugging Face attention layer, which evaluates  x*cos + rotate_half(x)*sin  (rotate_half(x) =

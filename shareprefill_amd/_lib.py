@@ -17,6 +17,7 @@ SP_DEC_VS, SP_DEC_DENSE, SP_DEC_SHARE, SP_DEC_QA = 0, 1, 2, 3
 SP_FLAG_LOGITS_BF16 = 1
 SP_POOL_TAIL_TRUE_LENGTH, SP_POOL_TAIL_RESCALE = 0, 1
 SP_ATTN_V_REPACKED = 1
+SP_DECODE_STATIC_SCRATCH_BYTES = 8 << 20
 
 
 class ClusterStateStruct(C.Structure):
@@ -62,6 +63,7 @@ SIGNATURES = {
     "sp_decode_workspace_bytes": (_SZ, [_I64, _I32, _I32]),
     "sp_decode_attn_bf16": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I64, _F, _P, _P, _SZ,
                                    _P]),
+    "sp_decode_attn_static_bf16": (_I32, [_P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I64, _F, _P, _P]),
     "sp_rope_inplace_bf16": (_I32, [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I64, _P]),
     "sp_pivot_update": (_I32, [_ST, _P, _P, _P, _I32, _I32, _F, _P]),
     "sp_cover_select_rows": (_I32, [_P, _I32, _F, _P, _P]),

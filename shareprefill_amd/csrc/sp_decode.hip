@@ -14,6 +14,8 @@
 //                                  consecutive keys of one channel.
 #include "sp_common.h"
 
+#include <mutex>
+
 #define DC_THREADS 256
 #define DC_TILE 128   // keys per tile
 #define DC_D 128
@@ -288,4 +290,49 @@ extern "C" int sp_decode_attn_bf16(const void* q, const void* k, const void* v, 
              SP_ERR_WORKSPACE, "sp_decode_attn_bf16: workspace too small or misaligned");
   return dc_launch(q, k, v, n, hq, hkv, q_stride_h, k_stride_n, k_stride_h, v_stride_n, v_stride_h, softmax_scale, out,
                    workspace, (hipStream_t)stream);
+}
+
+// ---- the same step for callers that cannot allocate ---------------------------------------------------------------
+// The chunk partials live in a file-scope device array instead of a caller's workspace.  Every GPU the library runs on
+// holds its own copy of the array (at its own address) until the process ends; the array's name is only a host-side
+// handle, so the device address is looked up once per device with hipGetSymbolAddress and that pointer is what the
+// kernels get.
+#define DC_STATIC_BYTES SP_DECODE_STATIC_SCRATCH_BYTES
+#define DC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[DC_STATIC_BYTES];
+static void* dc_scratch_ptr[DC_MAX_DEVICES];  // device address of `scratch` per device, nullptr = not looked up yet
+static std::mutex dc_scratch_mutex;
+
+static int dc_static_scratch(void** ptr) {
+  int dev = -1;
+  SP_HIP(hipGetDevice(&dev));
+  SP_REQUIRE(dev >= 0 && dev < DC_MAX_DEVICES, SP_ERR_UNSUPPORTED, "sp_decode_attn_static_bf16: device index %d", dev);
+  std::lock_guard<std::mutex> lock(dc_scratch_mutex);
+  if (dc_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    SP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    SP_REQUIRE(p != nullptr, SP_ERR_HIP, "sp_decode_attn_static_bf16: no device address for the scratch array");
+    dc_scratch_ptr[dev] = p;
+  }
+  *ptr = dc_scratch_ptr[dev];
+  return SP_OK;
+}
+
+extern "C" int sp_decode_attn_static_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq,
+                                          int32_t hkv, int32_t d, int64_t q_stride_h, int64_t k_stride_n,
+                                          int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
+                                          float softmax_scale, void* out, sp_stream_t stream) {
+  int rc = dc_check("sp_decode_attn_static_bf16", q, k, v, n, hq, hkv, d, q_stride_h, k_stride_n, k_stride_h,
+                    v_stride_n, v_stride_h, softmax_scale, out);
+  if (rc) return rc;
+  const size_t need = sp_decode_workspace_bytes(n, hq, hkv);
+  SP_REQUIRE(need <= DC_STATIC_BYTES, SP_ERR_WORKSPACE,
+             "sp_decode_attn_static_bf16: n=%lld hq=%d hkv=%d needs %zu bytes of partials, the built-in scratch holds "
+             "%u; use sp_decode_attn_bf16 with a workspace",
+             (long long)n, hq, hkv, need, (unsigned)DC_STATIC_BYTES);
+  void* partials = nullptr;
+  rc = dc_static_scratch(&partials);
+  if (rc) return rc;
+  return dc_launch(q, k, v, n, hq, hkv, q_stride_h, k_stride_n, k_stride_h, v_stride_n, v_stride_h, softmax_scale, out,
+                   partials, (hipStream_t)stream);
 }

@@ -288,10 +288,12 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
 
 
 def decode_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float,
-                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     out: Optional[torch.Tensor] = None, static_scratch: bool = False) -> torch.Tensor:
     """q bf16 [Hq, D] (one token), k / v bf16 [Hkv, N, D] views -> out bf16 [Hq, D].
 
-    Reference: the flash_attn_func decode branch (shareprefill_attn.py:146-155)."""
+    Reference: the flash_attn_func decode branch (shareprefill_attn.py:146-155).  static_scratch=True takes the
+    entry point that allocates nothing (sp_decode_attn_static_bf16: the chunk partials live in an 8 MiB array built
+    into the library instead of a torch workspace); pass `out` as well and the call touches no allocator at all."""
     lib = _lib.load()
     _check_hnd(k, "k")
     _check_hnd(v, "v")
@@ -303,6 +305,12 @@ def decode_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_
         out = torch.empty(hq, d, dtype=torch.bfloat16, device=q.device)
     elif out.dtype != torch.bfloat16 or tuple(out.shape) != (hq, d) or not out.is_contiguous() or out.device != q.device:
         raise ValueError(f"out must be a contiguous bfloat16 [{hq}, {d}] tensor on {q.device}")
+    if static_scratch:
+        st = lib.sp_decode_attn_static_bf16(_ptr(q), _ptr(k), _ptr(v), n, hq, hkv, d, q.stride(0), k.stride(1),
+                                            k.stride(0), v.stride(1), v.stride(0), softmax_scale, _ptr(out),
+                                            _stream(q.device))
+        _lib.check(st, "sp_decode_attn_static_bf16")
+        return out
     ws = _workspace("decode", lib.sp_decode_workspace_bytes(n, hq, hkv), q.device)
     st = lib.sp_decode_attn_bf16(_ptr(q), _ptr(k), _ptr(v), n, hq, hkv, d, q.stride(0), k.stride(1), k.stride(0),
                                  v.stride(1), v.stride(0), softmax_scale, _ptr(out), _ptr(ws), ws.numel(),
