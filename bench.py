@@ -7,6 +7,12 @@ share decision, mask build, Q pooling + query-aware selection, V repack, block-s
 update) over one synthetic Q/K/V batch that is already resident in HBM.  The layer timed is layer 1, after
 one untimed call of layer 0 has elected the cluster pivots (sharing can only start in the layer after the
 pivot's, shareprefill/attn/shareprefill_attn.py:141-143).  Prints ONE JSON line.
+
+The default run carries the whole metric in that one line: the 128K layer (value, roofline of the attention kernel),
+the pattern_threshold sweep 0.9 / 0.95 / 0.99 with the dense causal baseline, a second timed variant of the same layer
+whose thresholds make heads share and go query-aware (`sharing_layer`), the end-to-end TTFT of the whole
+Llama-3.1-8B architecture at 131072 tokens (`ttft`), and the CPU baseline.  --no-sweep / --no-ttft / --no-extras /
+--no-cpu-baseline drop parts of it.
 """
 
 from __future__ import annotations
@@ -39,7 +45,11 @@ def parse():
     ap.add_argument("--pattern-threshold", type=float, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the stage breakdown / dense baseline / sweep")
-    ap.add_argument("--sweep", action="store_true", help="also time pattern_threshold 0.9 and 0.99")
+    ap.add_argument("--sweep", action="store_true", help="(default now) time pattern_threshold 0.9, 0.95 and 0.99")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the pattern_threshold sweep")
+    ap.add_argument("--no-ttft", action="store_true",
+                    help="skip the end-to-end TTFT block (whole Llama-3.1-8B architecture, 131072 tokens, 1 warm-up + 1 "
+                         "timed forward) that the default C3 run appends")
     ap.add_argument("--fuse-rope", action="store_true",
                     help="C4 only: rotary embedding by the one-pass in-place HIP kernel instead of the model's "
                          "elementwise kernels (bit-identical)")
@@ -107,16 +117,36 @@ def cpu_baseline(w, q, k, v, mask_bool, decision, kept_blocks, pt):
         blocks += len(cols)
     per_block = t_att / max(blocks, 1)
     total_ms = (t_sel + per_block * kept_blocks) * 1e3
-    return {"value": round(total_ms, 1), "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"selection float stages on heads {heads} (x{hq // len(heads)}), fp32 block-sparse attention on "
+    return {"value": round(total_ms, 1), "unit": "ms", "cores": torch.get_num_threads(), "kind": "port, extrapolated",
+            "extrapolated": True,
+            "sample": f"EXTRAPOLATED from a bounded sample: selection float stages on heads {heads} (x{hq // len(heads)}), fp32 block-sparse attention on "
                       f"{len(rows)} (head, query-block) rows = {blocks} kept blocks at {per_block * 1e3:.3f} ms/block, "
                       f"scaled to {kept_blocks} kept blocks; extrapolated"}
 
 
-# HBM-side bytes of one steady-state sp_attn_fwd_kernel launch of the default workload (C3, pattern_threshold
-# 0.95), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the V-repack kernel's known 256 MiB
-# (profiles/attention_layer_C3_hbm_traffic.txt): 101.7 GiB fetched + 1 GiB written.
-MEASURED_ATTN_TRAFFIC_BYTES = {("C3", 0.95): int((101.7 + 1.0) * 2 ** 30)}
+# Bytes one steady-state sp_attn_fwd_kernel launch moves past the L2 caches, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE scaled by the V-repack kernel's known 256 MiB (profiles/attention_layer_C3_hbm_traffic.txt).  A counter
+# run cannot happen inside this script, so the figure is tied to the kernel source it was measured on: it is
+# reported only while shareprefill_amd/csrc/sp_attn.hip still has that hash, and is null (with a note) after any
+# change to the kernel until the profile is taken again.
+MEASURED_ATTN_TRAFFIC = {
+    ("C3", 0.95): {"bytes": int((101.7 + 1.0) * 2 ** 30), "sp_attn_hip_sha256_16": "e161e6e5d4b37039",
+                   "profile": "profiles/attention_layer_C3_hbm_traffic.txt"},
+}
+
+
+def measured_traffic(workload, pt):
+    """-> (bytes or None, note)"""
+    import hashlib
+
+    rec = MEASURED_ATTN_TRAFFIC.get((workload, pt))
+    if rec is None:
+        return None, "no counter profile for this workload"
+    with open(os.path.join(ROOT, "shareprefill_amd", "csrc", "sp_attn.hip"), "rb") as f:
+        sha = hashlib.sha256(f.read()).hexdigest()[:16]
+    if sha != rec["sp_attn_hip_sha256_16"]:
+        return None, f"kernel source changed since {rec['profile']} was taken (sha {rec['sp_attn_hip_sha256_16']} -> {sha})"
+    return rec["bytes"], f"FETCH_SIZE + WRITE_SIZE past L2 (memory-side cache + HBM), {rec['profile']}, kernel source sha {sha}"
 
 
 def library_gemm_tflops(dev, n=8192, reps=200):
@@ -137,7 +167,7 @@ def library_gemm_tflops(dev, n=8192, reps=200):
     return 2.0 * n ** 3 * reps / (time.perf_counter() - t0) / 1e12
 
 
-def run_c4(args):
+def c4_line(args):
     """TTFT of the full Llama-3.1-8B architecture (random-init bf16, 32 layers, hidden 4096, Hq32 Hkv8, RoPE theta
     5e5, vocab 128256) on uniform-random token ids, SharePrefill patched into every layer with the shipped
     Llama-3.1-8B-Instruct table; one prefill forward with last-token logits only."""
@@ -163,6 +193,7 @@ def run_c4(args):
     gen = torch.Generator(device=dev)
     gen.manual_seed(1238)
     ids = torch.randint(0, cfg.vocab_size, (1, args.seq_len), generator=gen, device=dev)
+    model.attention_sharing.keep_plans = True  # every layer's mask (4 MiB at 128K) stays for the density below
 
     def fwd():
         with torch.no_grad():
@@ -214,7 +245,111 @@ def run_c4(args):
                 row["speedup"] = round(row["dense_sdpa_s"] / row["shareprefill_s"], 3)
             sweep.append(row)
         line["length_sweep"] = sweep
-    print(json.dumps(line))
+    del model
+    import gc
+
+    gc.collect()
+    torch.cuda.empty_cache()
+    return line
+
+
+def run_c4(args):
+    print(json.dumps(c4_line(args)))
+
+
+def sharing_layer_variant(args, w, pt, q, k, v, table):
+    """The same layer on the same inputs with thresholds under which heads DO share and go query-aware (with the
+    library defaults none of these synthetic heads does: a pivot with local attention has vs_ratio >= (nb-1)/nb >
+    fallback_threshold 0.9, and no head's sqrt-JS is below queryaware_threshold 0.1): fallback_threshold lifted,
+    queryaware_threshold placed between the heads' own sqrt-JS values so that a quarter of them are query-aware.
+    Layer 0 once (pivot election), then warm-up and timed calls of layer 1; plus the time of the stages that only
+    these head kinds use."""
+    import torch
+
+    from shareprefill_amd import AttentionSharing, _lib, ops, shareprefill_attention_forward
+
+    nb = w.seq_len // w.block_size
+    tri = w.hq * nb * (nb + 1) // 2
+    scale = w.head_dim ** -0.5
+    with tempfile.TemporaryDirectory() as tmp:
+        from shareprefill_amd import synthetic
+
+        sh = AttentionSharing(synthetic.write_cluster_table(table, os.path.join(tmp, "table.json")))
+
+    def cfg(fallback, qat):
+        return types.SimpleNamespace(block_size=w.block_size, min_budget=w.min_budget, max_budget=None,
+                                     pattern_threshold=pt, similarity_threshold=w.similarity_threshold,
+                                     fallback_threshold=fallback, queryaware_threshold=qat)
+
+    def run(layer, c):
+        mod = types.SimpleNamespace(config=c, attention_sharing=sh, layer_idx=layer, scaling=scale)
+        return shareprefill_attention_forward(mod, q, k, v, None, scaling=scale)
+
+    sh.keep_debug = True
+    run(0, cfg(w.fallback_threshold, w.queryaware_threshold))
+    js = torch.sort(sh.plans[-1].js_qa.double().cpu()).values
+    n_qa = max(w.hq // 4, 1)
+    qat = float((js[n_qa - 1] + js[n_qa]) / 2)
+    c2 = cfg(1e9, qat)
+    sh.keep_debug = False
+    sh.reset_state()
+    _, avg0 = run(0, c2)
+    plan0 = sh.plans[-1]
+    for _ in range(2):
+        run(1, c2)
+    torch.cuda.synchronize()
+    steps = max(1, min(args.steps, 10))
+    tm = ops.KernelTimer()
+    ops.kernel_timer = tm
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run(1, c2)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    ops.kernel_timer = None
+    attn_ms = sum(tm.durations_ms("attn")) / steps
+    names = {0: "vertical_slash", 1: "dense_pivot", 2: "shared", 3: "query_aware"}
+
+    def hist(plan):
+        return {names[int(c)]: int(n) for c, n in zip(*torch.unique(plan.decision.cpu(), return_counts=True))}
+
+    plan1 = sh.plans[-1]
+    kept = int(ops.mask_row_pointers(plan1.mask)[:, -1].sum())
+    out = {"thresholds": {"pattern": pt, "similarity": w.similarity_threshold, "fallback": 1e9,
+                          "queryaware": round(qat, 6)},
+           "steps": steps, "layer_ms": round(ms, 3), "attn_ms": round(attn_ms, 3), "kept_blocks": kept,
+           "density": round(kept / tri, 4), "decisions": hist(plan1), "layer0_decisions": hist(plan0),
+           "attn_tflops": round(kept * FLOP_PER_BLOCK / attn_ms / 1e9, 1),
+           "attn_frac_of_peak": round(kept * FLOP_PER_BLOCK / attn_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+           "layer_frac_of_peak": round(kept * FLOP_PER_BLOCK / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    # stages that only shared / query-aware / pivot heads use, timed alone on this layer's own intermediates
+    sh.keep_debug = True
+    run(1, c2)
+    p = sh.plans[-1]
+    sh.keep_debug = False
+    state = sh._state
+    hc = sh._head_cluster_tensor(1, w.hq, q.device)
+    use_qa = (p.decision == _lib.SP_DEC_QA).to(torch.int32)
+    minb = math.ceil(w.min_budget / w.block_size)
+    qh = q[0]
+    stage = {}
+    stage["share_decide"] = event_ms(lambda: ops.share_decide(state, hc, 1, p.vert_blk, p.slash_blk, use_qa, p.nv, p.ns,
+                                                              minb, w.similarity_threshold, 1e9))
+    stage["build_mask"] = event_ms(lambda: ops.build_mask(state, hc, p.decision, p.vert_blk, p.slash_blk, p.nv_final,
+                                                          p.ns_final))
+    scratch_mask = p.mask.clone()
+
+    def qa_select():
+        qbar = ops.pool_avg(qh, w.block_size, tail_mode=_lib.SP_POOL_TAIL_RESCALE, head_enable=use_qa)
+        ops.queryaware_select(qbar, p.kbar, p.decision, scratch_mask, pt, probs=sh._qa_scratch(w.hq, nb, q.device))
+
+    stage["queryaware_select_incl_q_pooling"] = event_ms(qa_select)
+    hc0 = sh._head_cluster_tensor(0, w.hq, q.device)
+    # the layer-0 pivots' update (row patterns + coverage ratio); repeating it rewrites the same values
+    stage["pivot_update_layer0_pivots"] = event_ms(lambda: ops.pivot_update(state, hc0, plan0.decision, avg0[0], pt))
+    out["stage_ms"] = {a: round(b, 3) for a, b in stage.items()}
+    out["n_pivots_layer0"] = int((plan0.decision == _lib.SP_DEC_DENSE).sum())
+    return out
 
 
 def main():
@@ -274,6 +409,7 @@ def main():
     # ---- layer 0 once (pivot election), then W warm-up and K timed steps of layer 1 -----------------
     layer0_ms = prime(pt)
     plan0 = sharing.plans[-1]
+    kept0 = int(ops.mask_row_pointers(plan0.mask)[:, -1].sum())  # now: the mask is released when layer 1 is planned
     for _ in range(args.warmup):
         run_layer(1, pt)
     torch.cuda.synchronize()
@@ -302,7 +438,6 @@ def main():
     hist0 = {}
     for code, cnt in zip(*torch.unique(plan0.decision.cpu(), return_counts=True)):
         hist0[names[int(code)]] = int(cnt)
-    kept0 = int(ops.mask_row_pointers(plan0.mask)[:, -1].sum())
 
     line = {
         "metric": "sparse_attn_prefill_ms_per_layer_128k" if args.workload == "C3" else
@@ -325,7 +460,8 @@ def main():
         "roofline": {"bound": "mfma", "kernel": "sp_attn_fwd_kernel", "achieved": round(attn_tflops, 1),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(attn_tflops / PEAK_BF16_TFLOPS, 4),
                      "avg_launch_ms": round(attn_avg_ms, 3), "launches": len(attn_ms),
-                     "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get((args.workload, pt)),
+                     "traffic": measured_traffic(args.workload, pt)[0],
+                     "traffic_note": measured_traffic(args.workload, pt)[1],
                      "sclk_mhz": round(ops.attention_clock_mhz(w.seq_len, w.hkv, w.head_dim, w.block_size, dev))},
     }
     pairing = ops.attention_pairing(w.seq_len, w.hq, w.hkv, w.head_dim, w.block_size, dev)
@@ -402,7 +538,7 @@ def main():
                                          "constant_operands": round(ops.mfma_probe_tflops(0), 1),
                                          "library_gemm_8192_random_data": round(library_gemm_tflops(dev), 1),
                                          "nominal_peak": PEAK_BF16_TFLOPS}
-        if args.sweep:
+        if not args.no_sweep:
             sweep = []
             for thr in (0.9, 0.95, 0.99):
                 prime(thr)
@@ -420,14 +556,30 @@ def main():
                 ams = sum(tm.durations_ms("attn")) / 3
                 sweep.append({"pattern_threshold": thr, "density": round(kb / tri, 4), "layer_ms": round(ms, 3),
                               "attn_ms": round(ams, 3), "attn_tflops": round(kb * FLOP_PER_BLOCK / ams / 1e9, 1),
+                              "attn_frac_of_peak": round(kb * FLOP_PER_BLOCK / ams / 1e9 / PEAK_BF16_TFLOPS, 4),
                               "layer_frac_of_peak": round(kb * FLOP_PER_BLOCK / ms / 1e9 / PEAK_BF16_TFLOPS, 4)})
             line["threshold_sweep"] = sweep
+        line["sharing_layer"] = sharing_layer_variant(args, w, pt, q, k, v, table)
 
     if not args.no_cpu_baseline:
         mask_bool = ops.mask_to_bool(plan.mask, nb).cpu().numpy()
         line["cpu_baseline"] = cpu_baseline(w, q, k, v, mask_bool, plan.decision.cpu().numpy(), kept, pt)
     else:
         line["cpu_baseline"] = None
+    if args.workload == "C3" and not args.no_ttft and not args.no_extras:
+        # the metric's third part: end-to-end TTFT of the whole architecture at the same 131072 tokens
+        del q, k, v
+        ops.release_workspaces()
+        torch.cuda.empty_cache()
+        targs = argparse.Namespace(**vars(args))
+        targs.seq_len, targs.warmup, targs.steps = 131072, 1, 1
+        targs.length_sweep = "1024,4096,16384"
+        c4 = c4_line(targs)
+        line["ttft"] = {"value": c4["value"], "unit": "s", "steps": c4["steps"], "warmup": c4["warmup"],
+                        "tokens_per_s": c4["tokens_per_s"], "mean_block_density": c4["mean_block_density"],
+                        "decisions": c4["decisions"], "finite_logits": c4["finite_logits"],
+                        "workload": c4["config"]["workload"], "fuse_rope": c4["config"]["fuse_rope"],
+                        "length_sweep": c4.get("length_sweep")}
     print(json.dumps(line))
 
 
