@@ -130,6 +130,8 @@ class AttentionSharing:
             self._state.reset()
         self._layer_avg = {}
         self.plans = []
+        self.dense_layers = 0
+        self._dense_heads = 0
 
     def _ensure_state(self, nb: int, device) -> ops.ClusterState:
         st = self._state
@@ -254,12 +256,20 @@ class AttentionSharing:
         if self.keep_pivot_maps:
             self._layer_avg[layer_idx] = avg_attn
 
+    def note_dense_layer(self, layer_idx: int, hq: int, nb: int) -> None:
+        """A layer whose prompt is no longer than the minimum budget ran on the dense causal mask without any
+        selection (see shareprefill_attention_core); counted for decision_histogram."""
+        self.dense_layers += 1
+        self._dense_heads += hq
+
     # ---- counters -----------------------------------------------------------------------------------------
     def decision_histogram(self) -> Dict[str, int]:
         """Counts of vertical-slash / dense / shared / query-aware heads over the layers planned since the
         last reset (synchronises)."""
         names = {0: "vertical_slash", 1: "dense_pivot", 2: "shared", 3: "query_aware"}
         out = {v: 0 for v in names.values()}
+        if self.dense_layers:
+            out["all_blocks_kept_no_selection"] = self._dense_heads
         for p in self.plans:
             for code, cnt in zip(*torch.unique(p.decision.cpu(), return_counts=True)):
                 out[names[int(code)]] += int(cnt)

@@ -22,8 +22,9 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define LQ_TILE 128          // keys per tile
 #define LQ_D 128             // head dim
 #define LQ_THREADS 256       // 4 waves, wave w owns query rows 32w..32w+31
-#define LQ_MIN_TILES 8       // key tiles per workgroup (probs: output tiles, plus one leading tile): 8 for short
-#define LQ_MAX_TILES 32      // sequences, up to 32 when that still leaves a thousand workgroups
+#define LQ_MIN_TILES 1       // key tiles per workgroup (probs: output tiles, plus one leading tile): as many (a power
+#define LQ_MAX_TILES 32      // of two, at most 32) as still leave about a thousand workgroups -- 1 at 4K tokens and
+                             // Llama head counts, where a launch is a single round of workgroups, 32 at 128K
 #define LQ_PITCH 136         // LDS row pitch (floats) of the probability tile
 // Row maxima are kept in base-2 units (max logit * log2 e), so a probability is one fused multiply-add and one
 // hardware exp2.  "No logit seen yet" is a large finite negative number, not -inf: then max, difference and exp2
@@ -362,13 +363,15 @@ static inline int lq_tiles_per_wg(int64_t n, int32_t hq) {
   while (tiles < LQ_MAX_TILES && work / (2 * tiles) >= 1024) tiles *= 2;
   return tiles;
 }
-// upper bound of the chunk count (the workspace is sized for it whatever the launch picks)
-static inline int lq_chunks(int64_t n) { return (int)sp_ceil_div(sp_ceil_div(n, LQ_TILE), LQ_MIN_TILES); }
+// chunk count of the launch (the workspace is sized for it)
+static inline int lq_chunks(int64_t n, int32_t hq) {
+  return (int)sp_ceil_div(sp_ceil_div(n, LQ_TILE), lq_tiles_per_wg(n, hq));
+}
 
 extern "C" size_t sp_lastq_scores_workspace_bytes(int64_t n, int32_t hq, int32_t bs) {
   (void)bs;
   if (n <= 0 || hq <= 0) return 0;
-  size_t partial = (size_t)hq * lq_chunks(n) * LQ_ROWS * sizeof(float2);
+  size_t partial = (size_t)hq * lq_chunks(n, hq) * LQ_ROWS * sizeof(float2);
   size_t rowstat = (size_t)hq * LQ_ROWS * sizeof(float2);
   return partial + rowstat;
 }
@@ -395,7 +398,7 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
   const int n_chunks = (int)sp_ceil_div(sp_ceil_div(n, LQ_TILE), tiles_per_wg);
   const int64_t nb = sp_ceil_div(n, bs);
   float2* partial = (float2*)workspace;
-  float2* rowstat = partial + (size_t)hq * lq_chunks(n) * LQ_ROWS;
+  float2* rowstat = partial + (size_t)hq * lq_chunks(n, hq) * LQ_ROWS;
   const float inv_sqrt_d = 1.0f / sqrtf((float)d);
   const int group = hq / hkv;
   hipStream_t s = (hipStream_t)stream;

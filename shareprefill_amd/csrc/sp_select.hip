@@ -131,26 +131,15 @@ __global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_hist_kernel(const float*
   }
 }
 
+// One level of the descent on a histogram that sits in sh.sum / sh.cnt: finds the bin in which the running mass
+// (from the top bin down) first exceeds the budget left, and moves the state below it.  Called by all SEL_THREADS
+// threads of a workgroup with the same `s`; every thread returns with the same updated `s`.  sh may be refilled
+// afterwards (the function ends with a barrier).
 template <int LEVEL>
-__global__ __launch_bounds__(SEL_THREADS) void sp_gsel_pick_kernel(GselState* __restrict__ st,
-                                                                   uint32_t* __restrict__ gcnt,
-                                                                   unsigned long long* __restrict__ gsum) {
-  __shared__ SelShared sh;
-  const int v = blockIdx.x, t = threadIdx.x;
-  GselState s = st[v];
-  if (!s.enabled || s.all) return;
+__device__ static void sel_pick_level(SelShared& sh, GselState& s) {
+  const int t = threadIdx.x;
   constexpr int width = LEVEL == 2 ? 10 : 11;
   const int nbins = 1 << width;
-  uint32_t* gc = gcnt + (int64_t)v * SEL_BINS;
-  unsigned long long* gs = gsum + (int64_t)v * SEL_BINS;
-  sh.sum[t] = gs[t];
-  sh.sum[t + SEL_THREADS] = gs[t + SEL_THREADS];
-  sh.cnt[t] = gc[t];
-  sh.cnt[t + SEL_THREADS] = gc[t + SEL_THREADS];
-  gs[t] = 0;  // ready for the next level
-  gs[t + SEL_THREADS] = 0;
-  gc[t] = 0;
-  gc[t + SEL_THREADS] = 0;
   if (t == 0) {
     sh.bin = -1;
     sh.cnt_above = 0;
@@ -176,10 +165,8 @@ __global__ __launch_bounds__(SEL_THREADS) void sp_gsel_pick_kernel(GselState* __
   __syncthreads();
   const int bin = sh.bin;
   if (bin < 0) {  // the running mass never exceeds the budget (top level only): keep everything
-    if (t == 0) {
-      s.all = 1;
-      st[v] = s;
-    }
+    s.all = 1;
+    __syncthreads();
     return;
   }
   uint32_t c = 0;
@@ -190,18 +177,183 @@ __global__ __launch_bounds__(SEL_THREADS) void sp_gsel_pick_kernel(GselState* __
   }
   if (c) atomicAdd(&sh.cnt_above, c);
   __syncthreads();
-  if (t == 0) {
-    s.prefix = (s.prefix << width) | (uint32_t)bin;
-    s.above += sh.cnt_above;
-    s.rem -= sh.sum_above;
-    if (LEVEL == 2) {
-      s.n_equal = sh.bin_cnt;
-      const unsigned long long each = sh.bin_sum / (sh.bin_cnt ? sh.bin_cnt : 1u);
-      unsigned long long take = each ? s.rem / each : (unsigned long long)s.n_equal;
-      if (take > s.n_equal) take = s.n_equal;
-      s.n_take = (uint32_t)take;
+  s.prefix = (s.prefix << width) | (uint32_t)bin;
+  s.above += sh.cnt_above;
+  s.rem -= sh.sum_above;
+  if (LEVEL == 2) {
+    s.n_equal = sh.bin_cnt;
+    const unsigned long long each = sh.bin_sum / (sh.bin_cnt ? sh.bin_cnt : 1u);
+    unsigned long long take = each ? s.rem / each : (unsigned long long)s.n_equal;
+    if (take > s.n_equal) take = s.n_equal;
+    s.n_take = (uint32_t)take;
+  }
+  __syncthreads();
+}
+
+template <int LEVEL>
+__global__ __launch_bounds__(SEL_THREADS) void sp_gsel_pick_kernel(GselState* __restrict__ st,
+                                                                   uint32_t* __restrict__ gcnt,
+                                                                   unsigned long long* __restrict__ gsum) {
+  __shared__ SelShared sh;
+  const int v = blockIdx.x, t = threadIdx.x;
+  GselState s = st[v];
+  if (!s.enabled || s.all) return;
+  uint32_t* gc = gcnt + (int64_t)v * SEL_BINS;
+  unsigned long long* gs = gsum + (int64_t)v * SEL_BINS;
+  sh.sum[t] = gs[t];
+  sh.sum[t + SEL_THREADS] = gs[t + SEL_THREADS];
+  sh.cnt[t] = gc[t];
+  sh.cnt[t + SEL_THREADS] = gc[t + SEL_THREADS];
+  gs[t] = 0;  // ready for the next level
+  gs[t + SEL_THREADS] = 0;
+  gc[t] = 0;
+  gc[t + SEL_THREADS] = 0;
+  sel_pick_level<LEVEL>(sh, s);
+  if (t == 0) st[v] = s;
+}
+
+// ---- the same descent by ONE workgroup per vector, histograms in LDS only -------------------------------------------
+// For short vectors (a few thousand to 16 K entries) the multi-workgroup descent is nothing but launch latency: ten
+// launches whose kernels run a few microseconds each.  Here one workgroup of SEL_THREADS threads makes the three
+// passes over its vector itself; the arithmetic (keys, fixed-point masses, pick rule, tie rule) is the very same
+// code, so both paths select the same entries.
+__device__ static inline GselState sel_fresh_state(long long t_le, bool enabled) {
+  GselState s;
+  s.rem = t_le < 0 ? 0ull : (unsigned long long)t_le;
+  s.prefix = 0;
+  s.above = 0;
+  s.n_equal = 0;
+  s.n_take = 0;
+  s.all = 0;
+  s.enabled = (enabled && t_le >= 0) ? 1 : 0;
+  for (int i = 0; i < 8; ++i) s.pad[i] = 0;
+  return s;
+}
+
+template <int LEVEL>
+__device__ static inline void sel_hist_add(SelShared& sh, const GselState& s, float val) {
+  constexpr int shift = LEVEL == 0 ? 21 : (LEVEL == 1 ? 10 : 0);
+  constexpr int width = LEVEL == 2 ? 10 : 11;
+  constexpr int pshift = LEVEL == 0 ? 32 : (LEVEL == 1 ? 21 : 10);
+  const uint32_t key = sp_sort_key(val);
+  if (pshift < 32 && (key >> (pshift & 31)) != s.prefix) return;
+  const uint32_t b = (key >> shift) & ((1u << width) - 1u);
+  atomicAdd(&sh.cnt[b], 1u);
+  const unsigned long long fx = sp_to_fixed(val);
+  if (fx) atomicAdd(&sh.sum[b], fx);
+}
+
+__device__ static inline void sel_hist_clear(SelShared& sh) {
+  sh.sum[threadIdx.x] = 0;
+  sh.sum[threadIdx.x + SEL_THREADS] = 0;
+  sh.cnt[threadIdx.x] = 0;
+  sh.cnt[threadIdx.x + SEL_THREADS] = 0;
+  __syncthreads();
+}
+
+// flat vectors (score_cover_topk, the budgets): vectors 0..n0-1 are rows of x0, the others rows of x1
+#define GSEL_SMALL_LEN 16384
+template <int LEVEL>
+__device__ static inline void sel_flat_level(SelShared& sh, GselState& s, const float* __restrict__ xv, int len) {
+  sel_hist_clear(sh);
+  for (int i = threadIdx.x; i < len; i += SEL_THREADS) sel_hist_add<LEVEL>(sh, s, xv[i]);
+  __syncthreads();
+  sel_pick_level<LEVEL>(sh, s);
+}
+
+__global__ __launch_bounds__(SEL_THREADS) void sp_gsel_count_small_kernel(
+    const float* __restrict__ x0, const float* __restrict__ x1, int n0, int len, long long t_le,
+    int32_t* __restrict__ out0, int32_t* __restrict__ out1, int bs, int minb, int maxb) {
+  __shared__ SelShared sh;
+  const int v = blockIdx.x;
+  const float* xv = v < n0 ? x0 + (int64_t)v * len : x1 + (int64_t)(v - n0) * len;
+  GselState s = sel_fresh_state(t_le, true);
+  if (s.enabled) {
+    sel_flat_level<0>(sh, s, xv, len);
+    if (!s.all) sel_flat_level<1>(sh, s, xv, len);
+    if (!s.all) sel_flat_level<2>(sh, s, xv, len);
+  }
+  if (threadIdx.x == 0) {  // as sp_gsel_count_kernel
+    long long m = 0;
+    if (t_le >= 0) m = s.all ? (long long)len : (long long)s.above + s.n_take;
+    long long r = m + 1;
+    if (bs > 0) {
+      r = r / bs + 1;
+      if (r < minb) r = minb;
+      if (r > maxb) r = maxb;
     }
-    st[v] = s;
+    if (v < n0)
+      out0[v] = (int32_t)r;
+    else
+      out1[v - n0] = (int32_t)r;
+  }
+}
+
+// lower triangle of an [nb][nb] map (score_cover_idx), nb <= GSEL_SMALL_NB: wave w of the 16 owns rows w, w+16, ...
+#define GSEL_SMALL_NB 128
+template <int LEVEL>
+__device__ static inline void sel_tri_level(SelShared& sh, GselState& s, const float* __restrict__ xv, int nb) {
+  sel_hist_clear(sh);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int r = wave; r < nb; r += SEL_THREADS / SP_WAVE)
+    for (int c = lane; c <= r; c += SP_WAVE) sel_hist_add<LEVEL>(sh, s, xv[(int64_t)r * nb + c]);
+  __syncthreads();
+  sel_pick_level<LEVEL>(sh, s);
+}
+
+__global__ __launch_bounds__(SEL_THREADS) void sp_gsel_small_kernel(const float* __restrict__ x,
+                                                                    const int32_t* __restrict__ enable,
+                                                                    int enable_match, int nb, int nbw, long long t_le,
+                                                                    uint64_t* __restrict__ mask) {
+  __shared__ SelShared sh;
+  __shared__ uint32_t row_ties[GSEL_SMALL_NB];
+  const int v = blockIdx.x;
+  if (!gsel_enabled(enable, enable_match, v)) return;
+  const float* xv = x + (int64_t)v * nb * nb;
+  uint64_t* mv = mask + (int64_t)v * nb * nbw;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  GselState s = sel_fresh_state(t_le, true);
+  if (s.enabled) {
+    sel_tri_level<0>(sh, s, xv, nb);
+    if (!s.all) sel_tri_level<1>(sh, s, xv, nb);
+    if (!s.all) sel_tri_level<2>(sh, s, xv, nb);
+  }
+  // the boundary group of equal values is taken partially: its n_take lowest indices (row-major) win
+  const bool ranked = s.enabled && !s.all && s.n_take != 0 && s.n_take < s.n_equal;
+  const bool take_all_equal = s.all || s.n_take >= s.n_equal;
+  if (ranked) {
+    for (int r = wave; r < nb; r += SEL_THREADS / SP_WAVE) {
+      uint32_t cnt = 0;
+      for (int c0 = 0; c0 <= r; c0 += SP_WAVE) {
+        const int c = c0 + lane;
+        cnt += __popcll(__ballot(c <= r && sp_sort_key(xv[(int64_t)r * nb + c]) == s.prefix));
+      }
+      if (lane == 0) row_ties[r] = cnt;
+    }
+    __syncthreads();
+  }
+  for (int r = wave; r < nb; r += SEL_THREADS / SP_WAVE) {
+    uint32_t before = 0;  // members of the boundary group in rows above this one (uniform per wave)
+    if (ranked)
+      for (int i = 0; i < r; ++i) before += row_ties[i];
+    for (int c0 = 0; c0 <= r; c0 += SP_WAVE) {
+      const int c = c0 + lane;
+      bool sel = false, eq = false;
+      if (s.enabled && c <= r) {
+        const uint32_t key = sp_sort_key(xv[(int64_t)r * nb + c]);
+        eq = key == s.prefix;
+        sel = s.all || key > s.prefix || (eq && take_all_equal);
+      }
+      if (ranked) {
+        const unsigned long long eqb = __ballot(eq);
+        if (eq && before + (uint32_t)__popcll(eqb & ((1ull << lane) - 1ull)) < s.n_take) sel = true;
+        before += (uint32_t)__popcll(eqb);
+      }
+      unsigned long long bal = __ballot(sel);
+      if (r == 0 && c0 == 0) bal |= 1ull;  // block (0,0): the padding id of the reference
+      // this wave alone writes the words of its rows (the kernels that wrote the mask before have finished)
+      if (lane == 0 && bal) mv[(int64_t)r * nbw + (c0 >> 6)] |= bal;
+    }
   }
 }
 
@@ -382,6 +534,12 @@ static int gsel_run(const float* x, const int32_t* enable, int enable_match, int
   SP_REQUIRE(workspace && workspace_bytes >= sp_cover_select_workspace_bytes(n_vec) && ((uintptr_t)workspace % 8) == 0,
              SP_ERR_WORKSPACE, "%s: workspace missing, misaligned or too small", who);
   const int nbw = (nb + 63) / 64;
+  if (nb <= GSEL_SMALL_NB) {  // one workgroup per map does the whole descent and writes the bits
+    hipLaunchKernelGGL(sp_gsel_small_kernel, dim3(n_vec), dim3(SEL_THREADS), 0, s, x, enable, enable_match, nb, nbw,
+                       (long long)sp_thr_le(score), mask);
+    SP_LAUNCH_CHECK();
+    return SP_OK;
+  }
   GselState* st = reinterpret_cast<GselState*>(workspace);
   unsigned long long* gsum = reinterpret_cast<unsigned long long*>(st + n_vec);
   uint32_t* gcnt = reinterpret_cast<uint32_t*>(gsum + (size_t)n_vec * SEL_BINS);
@@ -414,6 +572,12 @@ static int gsel_count_run(const float* x0, const float* x1, int n0, int n_vec, i
   unsigned long long* gsum = reinterpret_cast<unsigned long long*>(st + n_vec);
   uint32_t* gcnt = reinterpret_cast<uint32_t*>(gsum + (size_t)n_vec * SEL_BINS);
   const long long t_le = (long long)sp_thr_le(thr);
+  if (len <= GSEL_SMALL_LEN) {  // one workgroup per vector, one launch
+    hipLaunchKernelGGL(sp_gsel_count_small_kernel, dim3(n_vec), dim3(SEL_THREADS), 0, s, x0, x1, n0, (int)len, t_le, out0,
+                       out1, bs, minb, maxb);
+    SP_LAUNCH_CHECK();
+    return SP_OK;
+  }
   hipLaunchKernelGGL(sp_gsel_init_kernel, dim3(n_vec), dim3(256), 0, s, st, gcnt, gsum, (const int32_t*)nullptr, -1,
                      n_vec, t_le, (uint64_t*)nullptr, 0, 0);
   SP_LAUNCH_CHECK();
@@ -572,30 +736,60 @@ __global__ __launch_bounds__(QA_THREADS) void sp_queryaware_test_kernel(
   const int h = blockIdx.x;
   const int kvh = h / (hq / hkv);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  // mean over the last bs queries of bf16(q / sqrt(d)), rounded to bf16 (last_q.mean(1), :197-199)
-  for (int c = threadIdx.x; c < d; c += QA_THREADS) {
-    const sp_bf16* src = q + (int64_t)h * sq_h + (n - bs) * sq_n + c;
-    float s = 0.f;
-    for (int i = 0; i < bs; ++i) s += sp_round_bf16(sp_bf16_to_f32(src[(int64_t)i * sq_n]) * inv_sqrt_d);
-    qmean[c] = sp_round_bf16(s / (float)bs);
-  }
-  __syncthreads();
-  float lmax = -INFINITY;
-  for (int b = threadIdx.x; b < nb; b += QA_THREADS) {
-    const sp_bf16* kr = kbar + ((int64_t)b * hkv + kvh) * d;
-    float s = 0.f;
-    for (int c = 0; c < d; c += 8) {
-      const uint4 raw = *reinterpret_cast<const uint4*>(kr + c);
-      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  // mean over the last bs queries of bf16(q / sqrt(d)), rounded to bf16 (last_q.mean(1), :197-199): thread
+  // (row group rg, chunk of 8 channels) sums its rows rg, rg + 16, ..., the 16 partials meet in LDS in a fixed order
+  {
+    float* part = logit;  // [16][d] partial sums, reused for the logits afterwards (nb >= 1: sized max(nb, 16 d) by the host)
+    const int nchunk = d >> 3;
+    for (int item = threadIdx.x; item < 16 * nchunk; item += QA_THREADS) {
+      const int ch = item % nchunk, rg = item / nchunk;
+      float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (int i = rg; i < bs; i += 16) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(q + (int64_t)h * sq_h + (n - bs + i) * sq_n + ch * 8);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        s += qmean[c + 2 * j] * __uint_as_float(w[j] << 16);
-        s += qmean[c + 2 * j + 1] * __uint_as_float(w[j] & 0xffff0000u);
+        for (int j = 0; j < 4; ++j) {
+          acc[2 * j] += sp_round_bf16(__uint_as_float(w[j] << 16) * inv_sqrt_d);
+          acc[2 * j + 1] += sp_round_bf16(__uint_as_float(w[j] & 0xffff0000u) * inv_sqrt_d);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) part[rg * d + ch * 8 + j] = acc[j];
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < d; c += QA_THREADS) {
+      float sum = 0.f;
+#pragma unroll
+      for (int rg = 0; rg < 16; ++rg) sum += part[rg * d + c];
+      qmean[c] = sp_round_bf16(sum / (float)bs);
+    }
+    __syncthreads();
+  }
+  // logits against the pooled keys: four threads per key (32 channels each), partials folded in a fixed order
+  float lmax = -INFINITY;
+  const int quarter = threadIdx.x & 3;
+  for (int b0 = 0; b0 < nb; b0 += QA_THREADS / 4) {
+    const int b = b0 + (threadIdx.x >> 2);
+    float sacc = 0.f;
+    if (b < nb) {
+      const sp_bf16* kr = kbar + ((int64_t)b * hkv + kvh) * d;
+      for (int c = quarter * 8; c < d; c += 32) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(kr + c);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          sacc += qmean[c + 2 * j] * __uint_as_float(w[j] << 16);
+          sacc += qmean[c + 2 * j + 1] * __uint_as_float(w[j] & 0xffff0000u);
+        }
       }
     }
-    if (flags & SP_FLAG_LOGITS_BF16) s = sp_round_bf16(s);
-    logit[b] = s;
-    lmax = fmaxf(lmax, s);
+    const float s1 = sacc + __shfl_xor(sacc, 1, SP_WAVE);
+    float sfull = s1 + __shfl_xor(s1, 2, SP_WAVE);
+    if (b < nb && quarter == 0) {  // (the partial sums that shared `logit` were consumed before the barrier above)
+      if (flags & SP_FLAG_LOGITS_BF16) sfull = sp_round_bf16(sfull);
+      logit[b] = sfull;
+      lmax = fmaxf(lmax, sfull);
+    }
   }
   lmax = sp_wave_max(lmax);
   if (lane == 0) red[wave] = lmax;
@@ -648,7 +842,10 @@ extern "C" int sp_queryaware_test_bf16(const void* q, const void* kbar, const fl
   SP_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0 && d % 8 == 0 && n >= bs && bs > 0, SP_ERR_INVALID_ARGUMENT,
              "sp_queryaware_test_bf16: bad shape");
   const int nb = (int)sp_ceil_div(n, bs);
-  const size_t lds = (size_t)(d + nb) * sizeof(float);
+  SP_REQUIRE(d <= 256, SP_ERR_UNSUPPORTED, "sp_queryaware_test_bf16: head_dim %d too large", d);
+  SP_REQUIRE(q_stride_n % 8 == 0 && q_stride_h % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)kbar % 16) == 0,
+             SP_ERR_UNSUPPORTED, "sp_queryaware_test_bf16: q / kbar must be 16-byte aligned with strides multiple of 8");
+  const size_t lds = (size_t)(d + (nb > 16 * d ? nb : 16 * d)) * sizeof(float);
   SP_REQUIRE(lds <= 60000, SP_ERR_UNSUPPORTED, "sp_queryaware_test_bf16: nb=%d too large", nb);
   hipLaunchKernelGGL(sp_queryaware_test_kernel, dim3(hq), dim3(QA_THREADS), lds, (hipStream_t)stream,
                      (const sp_bf16*)q, (const sp_bf16*)kbar, vert_blk, n, hq, hkv, d, q_stride_n, q_stride_h, bs, nb,
@@ -702,7 +899,7 @@ __device__ static void vs_sets(const float* __restrict__ vert, const float* __re
 // ------------------------------------------------------------------------------------------------
 // pivot election / share test (attention_sharing.py:204-301): three launches.
 //   similarity : one workgroup per head, its sqrt-JS against the cluster's stored pivot (one wave per vector);
-//   decide     : one thread walks the heads in ascending order (the election is sequential by definition);
+//   decide     : one thread per head; the election's ascending order is resolved by looking at the lower heads;
 //   keep       : one workgroup per head; the newly elected pivots store their pooled vectors and their own
 //                vertical-slash sets.
 // ------------------------------------------------------------------------------------------------
@@ -727,35 +924,50 @@ __global__ __launch_bounds__(2 * SP_WAVE) void sp_share_similarity_kernel(
   if (lane == 0) (wave == 0 ? js_v : js_s)[h] = js;
 }
 
-__global__ __launch_bounds__(SP_WAVE) void sp_share_decide_kernel(
+__global__ __launch_bounds__(DEC_MAX_HEADS) void sp_share_decide_kernel(
     sp_cluster_state st, const int32_t* __restrict__ head_cluster, int layer_idx, int hq,
     const int32_t* __restrict__ use_qa, const int32_t* __restrict__ nv, const int32_t* __restrict__ ns, int minb,
     float sim_thr, double fb_thr, int32_t* __restrict__ decision, const float* __restrict__ js_v,
     const float* __restrict__ js_s, int32_t* __restrict__ nv_f, int32_t* __restrict__ ns_f) {
-  if (threadIdx.x != 0) return;
-  for (int h = 0; h < hq; ++h) {
-    int dec = SP_DEC_VS;
-    if (use_qa[h]) {
-      dec = SP_DEC_QA;
-    } else {
-      const int c = head_cluster[h];
-      if (sp_slot_ok(st, c)) {
-        if (st.info[c * 8 + 0] < 0) {
-          st.info[c * 8 + 0] = h;
-          st.info[c * 8 + 2] = nv[h];
-          st.info[c * 8 + 3] = ns[h];
-          st.info[c * 8 + 4] = layer_idx;
-          dec = SP_DEC_DENSE;
-        } else if (st.info[c * 8 + 1] != 0) {
-          if (js_v[h] < sim_thr && js_s[h] < sim_thr && st.ratio[c] < fb_thr) dec = SP_DEC_SHARE;
-        }
-      }
-    }
-    decision[h] = dec;
-    const bool reset = (dec == SP_DEC_QA || dec == SP_DEC_SHARE);
-    nv_f[h] = reset ? minb : nv[h];
-    ns_f[h] = reset ? minb : ns[h];
+  // The reference walks the heads in ascending order (attention_sharing.py:209-295): the first head of a shared
+  // cluster that is not query-aware and finds no pivot becomes the pivot; its later siblings of the same layer find
+  // a pivot without a pattern and fall back; heads of clusters with a pattern take the share test.  One thread per
+  // head reaches the same decisions: "first" = no lower head of the same cluster is a candidate too.
+  __shared__ int s_slot[DEC_MAX_HEADS];
+  __shared__ int s_cand[DEC_MAX_HEADS];
+  const int h = threadIdx.x;
+  int c = -1, qa = 0;
+  bool member = false, candidate = false;
+  if (h < hq) {
+    c = head_cluster[h];
+    qa = use_qa[h];
+    member = !qa && sp_slot_ok(st, c);
+    candidate = member && st.info[c * 8 + 0] < 0;  // the state as the previous layers left it
   }
+  s_slot[h] = c;
+  s_cand[h] = candidate ? 1 : 0;
+  __syncthreads();  // every read of the pivot slots precedes the writes below
+  if (h >= hq) return;
+  int dec = SP_DEC_VS;
+  if (qa) {
+    dec = SP_DEC_QA;
+  } else if (candidate) {
+    bool first = true;
+    for (int h2 = 0; h2 < h; ++h2) first = first && !(s_cand[h2] && s_slot[h2] == c);
+    if (first) {
+      st.info[c * 8 + 0] = h;
+      st.info[c * 8 + 2] = nv[h];
+      st.info[c * 8 + 3] = ns[h];
+      st.info[c * 8 + 4] = layer_idx;
+      dec = SP_DEC_DENSE;
+    }
+  } else if (member && st.info[c * 8 + 1] != 0) {
+    if (js_v[h] < sim_thr && js_s[h] < sim_thr && st.ratio[c] < fb_thr) dec = SP_DEC_SHARE;
+  }
+  decision[h] = dec;
+  const bool reset = (dec == SP_DEC_QA || dec == SP_DEC_SHARE);
+  nv_f[h] = reset ? minb : nv[h];
+  ns_f[h] = reset ? minb : ns[h];
 }
 
 // newly elected pivots (the cluster's pivot is this head, elected in this layer) keep their pooled vectors and
@@ -807,7 +1019,7 @@ extern "C" int sp_share_decide(const sp_cluster_state* state, const int32_t* hea
   hipLaunchKernelGGL(sp_share_similarity_kernel, dim3(hq), dim3(2 * SP_WAVE), 0, s, *state, head_cluster, vert_blk,
                      slash_blk, use_qa, js_v, js_s);
   SP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sp_share_decide_kernel, dim3(1), dim3(SP_WAVE), 0, s, *state, head_cluster, layer_idx, hq, use_qa,
+  hipLaunchKernelGGL(sp_share_decide_kernel, dim3(1), dim3(DEC_MAX_HEADS), 0, s, *state, head_cluster, layer_idx, hq, use_qa,
                      nv, ns, min_blocks, similarity_threshold, fallback_threshold, decision, js_v, js_s, nv_final,
                      ns_final);
   SP_LAUNCH_CHECK();

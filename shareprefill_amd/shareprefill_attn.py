@@ -22,9 +22,19 @@ from .attention_sharing import budget_blocks
 LOGGER = logging.getLogger(__name__)
 
 
+_dense_masks = {}
+
+
 def _dense_causal_mask(hq: int, nb: int, device) -> torch.Tensor:
-    tri = torch.tril(torch.ones(nb, nb, dtype=torch.bool, device=device))
-    return ops.bool_to_mask(tri).unsqueeze(0).expand(hq, -1, -1).contiguous()
+    """Bit mask with every lower-triangular block set, cached per shape (short prompts ask for it in every layer)."""
+    key = (hq, nb, str(device))
+    m = _dense_masks.get(key)
+    if m is None:
+        tri = torch.tril(torch.ones(nb, nb, dtype=torch.bool, device=device))
+        m = ops.bool_to_mask(tri).unsqueeze(0).expand(hq, -1, -1).contiguous()
+        if nb <= 64:
+            _dense_masks[key] = m
+    return m
 
 
 def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: torch.Tensor,
@@ -69,6 +79,19 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
         return out.unsqueeze(0).transpose(1, 2), avg_attn
 
     minb, maxb = budget_blocks(config.min_budget, config.max_budget, block_size)
+    if nb <= minb and getattr(config, "dense_short_prompts", True):
+        # The prompt has no more blocks than the minimum budget.  Every head's budgets are then clamped to nb
+        # (attention_sharing.py:173-176: raised to min_budget, cut to min(max_budget, nb)), its vertical-slash set is
+        # every column and every distance, and whatever the head's decision (pivot, shared, query-aware, fallback) its
+        # mask is the whole lower triangle -- in this layer and, with the same prompt, in every later one.  Nothing the
+        # selection computes can change an output, so it is skipped and the attention runs on the dense mask: the
+        # same result at a fraction of the launches.  What is not produced on this path: decisions, pivot state and
+        # the pivots' block-average maps (attn_weights is all zeros).  config.dense_short_prompts = False takes the
+        # full path instead.
+        mask = _dense_causal_mask(num_heads, nb, q.device)
+        out = ops.block_sparse_attention(q, k, v, mask, block_size, softmax_scale)
+        sharing.note_dense_layer(module.layer_idx, num_heads, nb)
+        return out.unsqueeze(0).transpose(1, 2), avg_attn
     plan = sharing.plan_layer(q, k, module.layer_idx, block_size, minb, maxb, config.pattern_threshold,
                               config.similarity_threshold, config.fallback_threshold, config.queryaware_threshold)
     # room for the block sums of this layer's possible pivots (at most 16 GiB of it; pivots beyond that take the

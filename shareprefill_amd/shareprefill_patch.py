@@ -126,6 +126,8 @@ def shareprefill_patch(model, config: SharePrefillConfig):
             self.attention_sharing.reset_state()
         for name in _CONFIG_FIELDS:
             setattr(self.config, name, getattr(config, name))
+        # not in the reference: prompts no longer than min_budget run on the dense mask without any selection
+        self.config.dense_short_prompts = bool(config.extra.get("dense_short_prompts", True))
         for m in self.modules():
             if isinstance(m, attention_cls):
                 m.attention_sharing = self.attention_sharing

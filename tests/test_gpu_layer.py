@@ -42,8 +42,10 @@ class FakeAttention:
 def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_free=True, with_forced=True, **thr):
     from shareprefill_amd import AttentionSharing, shareprefill_attention_forward, ops
 
+    # dense_short_prompts off: these tests compare the selection itself, also where the prompt is so short that every
+    # mask comes out dense and the attention function would skip it
     kw = dict(block_size=128, min_budget=1024, max_budget=None, pattern_threshold=0.95, similarity_threshold=0.5,
-              fallback_threshold=0.9, queryaware_threshold=0.1)
+              fallback_threshold=0.9, queryaware_threshold=0.1, dense_short_prompts=False)
     kw.update(thr)
     table = synthetic.random_cluster_table(hq, n_clusters, n_layers, seed)
     path = synthetic.write_cluster_table(table, str(tmp_path / "table.json"))
@@ -221,6 +223,37 @@ def test_layer_sharing_and_query_aware_paths(gpu_device, tmp_path):
     assert (d1 == O.DEC_SHARE).sum() >= 1          # next layer: same inputs -> JS = 0 -> shared
     hist = run["sharing"].decision_histogram()
     assert hist["dense_pivot"] == 2 and hist["shared"] == int((d1 == O.DEC_SHARE).sum())
+
+
+def test_prompt_within_the_minimum_budget_skips_selection_with_identical_output(gpu_device, tmp_path):
+    """1024 tokens = 8 blocks = the minimum budget: every head's mask is the whole lower triangle whatever it decides
+    (the oracle says so too), so the attention function runs the dense mask directly.  Same bits as the full path,
+    no plan, zero attn_weights."""
+    full = run_layers(gpu_device, tmp_path, hq=8, hkv=2, n=1024, seed=44, n_clusters=2, fallback_threshold=1e9)
+    check_forced(full)
+    tri = np.tril(np.ones((8, 8), dtype=bool))
+    for L in full["layers"]:
+        assert all(np.array_equal(L["mask"][h], tri) for h in range(8))
+        assert all(np.array_equal(L["forced"].mask[h], tri) for h in range(8))
+    sub = tmp_path / "fast"
+    sub.mkdir()
+    fast = run_layers(gpu_device, sub, hq=8, hkv=2, n=1024, seed=44, n_clusters=2, fallback_threshold=1e9,
+                      n_layers=0)
+    from shareprefill_amd import shareprefill_attention_forward
+
+    sharing = fast["sharing"]
+    cfg = types.SimpleNamespace(**{**fast["kw"], "dense_short_prompts": True})
+    q, k, v = (fast[x][None].to(gpu_device) for x in ("q", "k", "v"))
+    for layer in range(2):
+        mod = FakeAttention(cfg, sharing, layer, 128, 8, 2)
+        out, avg = shareprefill_attention_forward(mod, q, k, v, None, scaling=mod.scaling)
+        assert torch.equal(out.cpu(), full["layers"][layer]["out"])
+        assert float(avg.abs().sum()) == 0.0 and avg.shape == (1, 8, 8, 8)
+    assert sharing.plans == [] and sharing.decision_histogram()["all_blocks_kept_no_selection"] == 16
+    # one block more than the budget: the selection runs
+    cfg9 = types.SimpleNamespace(**{**fast["kw"], "dense_short_prompts": True, "min_budget": 896})
+    shareprefill_attention_forward(FakeAttention(cfg9, sharing, 0, 128, 8, 2), q, k, v, None, scaling=128 ** -0.5)
+    assert len(sharing.plans) == 1
 
 
 def test_layer_ragged_length(gpu_device, tmp_path):

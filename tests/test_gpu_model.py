@@ -42,6 +42,15 @@ def test_patched_model_matches_eager_when_every_block_is_kept(gpu_device, tmp_pa
     assert out.shape == ref.shape
     assert (out - ref).abs().max().item() < 0.15 and ((out - ref).abs().mean() / ref.abs().mean()).item() < 2e-2
     hist = model.attention_sharing.decision_histogram()
+    # 1024 tokens lie within min_budget: both layers ran on the dense mask without any selection
+    assert hist["all_blocks_kept_no_selection"] == 8 and model.attention_sharing.plans == []
+    # ... and with that shortcut switched off the selection decides, and keeps every block just the same
+    model_full = SharePrefill(sharing_lookup_path=table(tmp_path, 2, 4), min_budget=8192, dense_short_prompts=False)(
+        small_llama().to(gpu_device, torch.bfloat16))
+    with torch.no_grad():
+        out_full = model_full(ids, use_cache=False).logits.float()
+    assert torch.equal(out_full, out)
+    hist = model_full.attention_sharing.decision_histogram()
     assert sum(hist.values()) == 8 and hist["dense_pivot"] <= 2  # 2 layers x 4 heads, at most one pivot per cluster
     # a second forward resets the sharing state and gives the same result
     with torch.no_grad():
