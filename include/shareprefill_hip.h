@@ -57,14 +57,16 @@ typedef struct sp_cluster_state {
   int32_t nb;  /* blocks per side the slabs are sized for */
   int32_t nbw; /* ceil(nb/64) */
   int32_t reserved;
-  int32_t* info;     /* [C][8]: 0 pivot head (-1 none), 1 has_pattern, 2 pivot nv, 3 pivot ns, 4 pivot layer */
+  int32_t* info;     /* [C][8]: 0 pivot head (-1 none), 1 has_pattern, 2 pivot nv, 3 pivot ns, 4 pivot layer,
+                        5 rows counted by a running sp_pivot_update (zero between calls) */
   double* ratio;     /* [C]     vs_ratio of the pivot (valid once has_pattern) */
   float* vert;       /* [C][nb] pivot's pooled last-row vertical vector */
   float* slash;      /* [C][nb] pivot's pooled last-row slash vector */
   uint8_t* cols;     /* [C][nb] 1 = block column in the pivot's own vertical set */
   uint8_t* dists;    /* [C][nb] 1 = block distance in the pivot's own slash set */
   uint64_t* pattern; /* [C][nb][nbw] pivot block pattern */
-  uint64_t* accum;   /* [C][2]  scratch of sp_pivot_update (covered / total mass, fixed point) */
+  uint64_t* accum;   /* [C][2]  scratch of sp_pivot_update (covered / total mass, fixed point); zero on entry, and
+                        every completed call leaves it zero again: allocate it zero-filled */
 } sp_cluster_state;
 
 /* ---- library info ------------------------------------------------------------------------- */
@@ -175,6 +177,8 @@ int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec,
  * sp_attn_repack_v_bf16 fills it; sp_block_sparse_attn_fwd_bf16 calls it first unless flags has
  * SP_ATTN_V_REPACKED (the caller already repacked this v into this workspace). */
 #define SP_ATTN_V_REPACKED 1u
+#define SP_ATTN_PAIR_ROWS 2u /* skip the per-call analysis of how to pair query blocks into work items and pair rows
+                                2p, 2p+1 of every head: what a dense mask wants; the result never depends on it */
 size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs);
 /* Optional extra workspace per pivot head (decision == SP_DEC_DENSE with avg_attn requested): with
  * sp_attn_workspace_bytes rounded up to 256 bytes + p * sp_attn_pivot_scratch_bytes(n, bs) bytes of workspace, the

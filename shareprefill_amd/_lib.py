@@ -17,6 +17,7 @@ SP_DEC_VS, SP_DEC_DENSE, SP_DEC_SHARE, SP_DEC_QA = 0, 1, 2, 3
 SP_FLAG_LOGITS_BF16 = 1
 SP_POOL_TAIL_TRUE_LENGTH, SP_POOL_TAIL_RESCALE = 0, 1
 SP_ATTN_V_REPACKED = 1
+SP_ATTN_PAIR_ROWS = 2
 SP_DECODE_STATIC_SCRATCH_BYTES = 8 << 20
 
 

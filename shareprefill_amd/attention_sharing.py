@@ -96,6 +96,7 @@ class AttentionSharing:
         # newest one still holds its mask, the older ones keep their few per-head integers
         self.plans: List[LayerPlan] = []
         self._scratch: Dict[Tuple[str, str], torch.Tensor] = {}
+        self._max_pivots: Dict[Tuple[int, int], int] = {}
         self.reset_state()
 
     # ---- table ------------------------------------------------------------------------------------
@@ -198,8 +199,7 @@ class AttentionSharing:
         qa_probs = ops.queryaware_select(qbar, kbar, decision, mask, pattern_threshold, self.flags,
                                          probs=self._qa_scratch(hq, nb, dev))
         plan = LayerPlan(layer_idx, nb, mask, decision, nv, ns, nv_f, ns_f)
-        plan.max_pivots = len({self._slot[c] for h in range(hq)
-                               for c in (self._pair_to_cluster.get((layer_idx, h)),) if c in self._slot})
+        plan.max_pivots = self.max_pivots(layer_idx, hq)
         if self.keep_debug:
             plan.vert_tok, plan.slash_tok, plan.vert_blk, plan.slash_blk = vert_tok, slash_tok, vert_blk, slash_blk
             plan.kbar, plan.avg_qk, plan.js_qa, plan.js_v, plan.js_s = kbar, avg_qk, js_qa, js_v, js_s
@@ -208,6 +208,16 @@ class AttentionSharing:
             self.plans[-1].mask = None
         self.plans.append(plan)
         return plan
+
+    def max_pivots(self, layer_idx: int, hq: int) -> int:
+        """Shared clusters with a head in this layer: no more heads than that can become pivots in it."""
+        key = (layer_idx, hq)
+        n = self._max_pivots.get(key)
+        if n is None:
+            n = len({self._slot[c] for h in range(hq)
+                     for c in (self._pair_to_cluster.get((layer_idx, h)),) if c in self._slot})
+            self._max_pivots[key] = n
+        return n
 
     def _qa_scratch(self, hq: int, nb: int, device) -> torch.Tensor:
         """fp32 [Hq, nb, nb] scratch of the query-aware selection, owned by this object (one model, one stream of

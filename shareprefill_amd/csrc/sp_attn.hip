@@ -91,11 +91,13 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 // The 1 KiB scheduler area (int indices): 0..127 eight queue tickets (one per 64 bytes), 128..191 the pivot slot of
 // every head (one byte each, AT_NO_SLOT = its block sums are not kept), 192..195 {shader cycles, 100 MHz ticks} of
 // workgroup 0, 196 the number of pivot slots in use, 200..231 the pairing of every two adjacent heads (one byte each,
-// see sp_attn_pairing_kernel).
+// see sp_attn_pairing_kernel), 232..239 the queue tickets of the pivot heads' launch (so that both launches of a call
+// find their tickets cleared by sp_attn_prep_kernel and nothing has to be cleared in between).
 #define AT_SLOT_TABLE 128
 #define AT_CLOCK_SLOT 192
 #define AT_NPIV_SLOT 196
 #define AT_PAIR_TABLE 200
+#define AT_PIVOT_TICKETS 232  // 232..239: the eight queue tickets of the pivot heads' own launch
 #define AT_NO_SLOT 255
 #define AT_MAX_HEADS 256
 #define AT_FWD_THREADS 512
@@ -608,7 +610,7 @@ __device__ __forceinline__ void at_step(const AtAddr& ad, const bf16x8 (&qb)[2][
 
 // PIVOT = false: every head except the pivots that have a slot in the scheduler area's table (when skip_slotted).
 // PIVOT = true: only those pivots; besides the output it leaves, per (query, key block), the softmax mass of the
-// block relative to the running max at that time as u = log2(sum) + max, from which sp_attn_avg_finish_kernel makes
+// block relative to the running max at that time as u = log2(sum) + max, from which at_avg_from_block_sums (sp_attn_avg_kernel) makes
 // the block-average map without recomputing any logit.  pivot_u: fp32 [slot][r*(r+1)/2 + c][128 queries].
 template <bool PIVOT>
 __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
@@ -663,7 +665,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       int found = -1, tk = 0;
       for (int a = first_try; a < 8; ++a) {
         const int xq = (xcd + a) & 7;
-        tk = atomicAdd(&sched[xq * 16], 1);
+        tk = atomicAdd(&sched[PIVOT ? AT_PIVOT_TICKETS + xq : xq * 16], 1);
         if (tk < at_queue_items(gm, xq)) {
           found = xq;
           first_try = a;
@@ -953,15 +955,13 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
   }
 }
 
-__global__ void sp_zero_i32_kernel(int* p, int count) {
-  for (int i = threadIdx.x; i < count; i += blockDim.x) p[i] = 0;
-}
-
 // Before the forward launches: clears the queue tickets and gives the first max_pivots heads whose decision is
 // DENSE a slot for their block sums (ascending head order); every other head gets AT_NO_SLOT.
 __global__ void sp_attn_prep_kernel(int* __restrict__ sched, const int32_t* __restrict__ decision, int hq,
                                     int max_pivots) {
   for (int i = threadIdx.x; i < AT_SLOT_TABLE; i += blockDim.x) sched[i] = 0;
+  // pivot launch tickets; pairing table = rows 2p, 2p+1 of a head (sp_attn_pairing_kernel may choose otherwise)
+  for (int i = AT_PAIR_TABLE + threadIdx.x; i < AT_PIVOT_TICKETS + 8; i += blockDim.x) sched[i] = 0;
   if (threadIdx.x == 0) {
     uint8_t* slots = reinterpret_cast<uint8_t*>(sched + AT_SLOT_TABLE);
     int cnt = 0;
@@ -1012,13 +1012,12 @@ __global__ __launch_bounds__(256) void sp_attn_pairing_kernel(int* __restrict__ 
 
 // ---- pivot heads with a slot: block-averaged attention map from the block sums the forward kernel kept ----
 // avg[h][r][c] = mean over the valid queries of block r of  exp2(u[q][c] - m[q]) / l[q]  (m, l: the query's final
-// softmax statistics).  One workgroup per (query block, head); a wave takes every fourth kept block.
-__global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_finish_kernel(
-    const uint64_t* __restrict__ mask, const int* __restrict__ sched, const float2* __restrict__ rowstat,
-    const float* __restrict__ pivot_u, float* __restrict__ avg_attn, int64_t n, int nb, int nbw) {
+// softmax statistics).  One workgroup per (query block, head) of sp_attn_avg_kernel; a wave takes every fourth kept
+// block.
+__device__ static void at_avg_from_block_sums(const uint64_t* __restrict__ mask, int slot,
+                                              const float2* __restrict__ rowstat, const float* __restrict__ pivot_u,
+                                              float* __restrict__ avg_attn, int64_t n, int nb, int nbw) {
   const int r = nb - 1 - blockIdx.x, h = blockIdx.y;
-  const int slot = reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE)[h];
-  if (slot == AT_NO_SLOT) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t rem = n - (int64_t)r * AT_BS;
   const int valid_q = rem < AT_BS ? (int)rem : AT_BS;
@@ -1051,18 +1050,24 @@ __global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_finish_kernel(
 // ---- pivot heads: block-averaged attention map (shareprefill_attn.py:425-457) ---------------------------
 // avg[h][r][c] = mean over the valid queries of block r of the softmax mass that falls into key block c,
 // recomputed from the row statistics the forward kernel left behind (the pivots for which the workspace has no
-// room to keep block sums; the others go through sp_attn_avg_finish_kernel).  One workgroup per (query block,
-// head); heads that are not such pivots leave at once.
+// room to keep block sums; the others are made from their block sums by at_avg_from_block_sums, in the same launch).
+// One workgroup per (query block, head); heads that are no pivots leave at once.
 __global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const uint64_t* __restrict__ mask,
     const int32_t* __restrict__ decision, const float2* __restrict__ rowstat, float* __restrict__ avg_attn, int64_t n,
     int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n, int64_t sk_h, int nb, int nbw, float scale_log2,
-    const int* __restrict__ sched) {
+    const int* __restrict__ sched, const float* __restrict__ pivot_u) {
   __shared__ __attribute__((aligned(16))) sp_bf16 Ks[AT_BS * AT_PITCH];
   __shared__ float wred[2][4];
   const int r = nb - 1 - blockIdx.x, h = blockIdx.y;
   if (decision[h] != SP_DEC_DENSE) return;
-  if (reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE)[h] != AT_NO_SLOT) return;  // done from its block sums
+  {
+    const int slot = reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE)[h];
+    if (slot != AT_NO_SLOT) {  // (uniform) the forward pass kept this head's block sums
+      at_avg_from_block_sums(mask, slot, rowstat, pivot_u, avg_attn, n, nb, nbw);
+      return;
+    }
+  }
   const int kvh = h / (hq / hkv);
   const int t = threadIdx.x;
   const int wave = t >> 6, lane = t & 63;
@@ -1255,9 +1260,11 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   float* pivot_u = reinterpret_cast<float*>(ws + base_aligned);
   hipLaunchKernelGGL(sp_attn_prep_kernel, dim3(1), dim3(128), 0, s, counter, decision, (int)hq, max_pivots);
   SP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sp_attn_pairing_kernel, dim3((unsigned)((hq + 1) / 2)), dim3(256), 0, s, counter, mask, (int)hq,
-                     (int)(hq / hkv), (int)nb, (int)((nb + 63) / 64), max_pivots > 0 ? 1 : 0);
-  SP_LAUNCH_CHECK();
+  if (!(flags & SP_ATTN_PAIR_ROWS)) {  // (otherwise the table stays as sp_attn_prep_kernel left it: rows paired)
+    hipLaunchKernelGGL(sp_attn_pairing_kernel, dim3((unsigned)((hq + 1) / 2)), dim3(256), 0, s, counter, mask, (int)hq,
+                       (int)(hq / hkv), (int)nb, (int)((nb + 63) / 64), max_pivots > 0 ? 1 : 0);
+    SP_LAUNCH_CHECK();
+  }
   const size_t lds_bytes = AT_LDS_BYTES;
   // per device, once: the kernels' LDS allowance and the CU count (idempotent, so a race between two host threads
   // at worst repeats it)
@@ -1284,22 +1291,17 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
                      counter, max_pivots > 0 ? 1 : 0, (float*)nullptr);
   SP_LAUNCH_CHECK();
   if (max_pivots > 0) {
-    hipLaunchKernelGGL(sp_zero_i32_kernel, dim3(1), dim3(128), 0, s, counter, AT_SLOT_TABLE);  // the tickets again
-    SP_LAUNCH_CHECK();
     hipLaunchKernelGGL(sp_attn_fwd_kernel<true>, dim3(grid), dim3(AT_FWD_THREADS), lds_bytes, s, (const sp_bf16*)q,
                        (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out, stats, n, hq,
                        hkv, q_stride_n, q_stride_h, k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64),
                        scale_log2, counter, 0, pivot_u);
     SP_LAUNCH_CHECK();
-    hipLaunchKernelGGL(sp_attn_avg_finish_kernel, dim3((unsigned)nb, hq), dim3(AT_THREADS), 0, s, mask,
-                       (const int*)counter, (const float2*)rowstat, (const float*)pivot_u, avg_attn, n, (int)nb,
-                       (int)((nb + 63) / 64));
-    SP_LAUNCH_CHECK();
   }
   if (want_avg) {
     hipLaunchKernelGGL(sp_attn_avg_kernel, dim3((unsigned)nb, hq), dim3(AT_THREADS), 0, s, (const sp_bf16*)q,
                        (const sp_bf16*)k, mask, decision, rowstat, avg_attn, n, hq, hkv, q_stride_n, q_stride_h,
-                       k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, (const int*)counter);
+                       k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, (const int*)counter,
+                       (const float*)pivot_u);
     SP_LAUNCH_CHECK();
   }
   return SP_OK;

@@ -22,9 +22,9 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define LQ_TILE 128          // keys per tile
 #define LQ_D 128             // head dim
 #define LQ_THREADS 256       // 4 waves, wave w owns query rows 32w..32w+31
-#define LQ_MIN_TILES 1       // key tiles per workgroup (probs: output tiles, plus one leading tile): as many (a power
-#define LQ_MAX_TILES 32      // of two, at most 32) as still leave about a thousand workgroups -- 1 at 4K tokens and
-                             // Llama head counts, where a launch is a single round of workgroups, 32 at 128K
+#define LQ_MIN_TILES 1       // key tiles per workgroup (probs: output tiles, plus one leading tile): a power of two, at
+#define LQ_MAX_TILES 32      // most 32 -- as many as still leave about a thousand workgroups at long sequences (32 at
+                             // 128K tokens and Llama head counts), as few as give one round of ~512 at short ones (2 at 4K)
 #define LQ_PITCH 136         // LDS row pitch (floats) of the probability tile
 // Row maxima are kept in base-2 units (max logit * log2 e), so a probability is one fused multiply-add and one
 // hardware exp2.  "No logit seen yet" is a large finite negative number, not -inf: then max, difference and exp2
@@ -187,18 +187,16 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_stats_kernel(
       m[r] = mn;
     }
   }
-  // merge the 32 lanes that share a row (fixed xor tree)
+  // merge the 32 lanes that share a row: the row's maximum first, then every lane's sum is brought to that maximum
+  // once and the sums are added over a fixed xor tree (one exp2 per row instead of two per tree level)
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    float mm = m[r], ll = l[r];
+    float mm = m[r];
 #pragma unroll
-    for (int o = 1; o < 32; o <<= 1) {
-      const float m2 = __shfl_xor(mm, o, SP_WAVE);
-      const float l2 = __shfl_xor(ll, o, SP_WAVE);
-      const float mn = fmaxf(mm, m2);
-      ll = ll * __builtin_amdgcn_exp2f(mm - mn) + l2 * __builtin_amdgcn_exp2f(m2 - mn);
-      mm = mn;
-    }
+    for (int o = 1; o < 32; o <<= 1) mm = fmaxf(mm, __shfl_xor(mm, o, SP_WAVE));
+    float ll = l[r] * __builtin_amdgcn_exp2f(m[r] - mm);  // (a lane that saw nothing: l = 0)
+#pragma unroll
+    for (int o = 1; o < 32; o <<= 1) ll += __shfl_xor(ll, o, SP_WAVE);
     if ((lane & 31) == 0) {
       partial[((int64_t)h * n_chunks + chunk) * LQ_ROWS + lq_row_of(wave, lane, r)] = make_float2(mm, ll);
     }
@@ -359,8 +357,10 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
 // ---- host -------------------------------------------------------------------------------------------------
 static inline int lq_tiles_per_wg(int64_t n, int32_t hq) {
   const int64_t work = sp_ceil_div(n, LQ_TILE) * hq;  // (head, key tile) pairs
-  int tiles = LQ_MIN_TILES;
+  int tiles = 8;
   while (tiles < LQ_MAX_TILES && work / (2 * tiles) >= 1024) tiles *= 2;
+  // short sequences: one round of workgroups (two per CU) rather than few long-running ones
+  while (tiles > LQ_MIN_TILES && work / tiles < 512) tiles /= 2;
   return tiles;
 }
 // chunk count of the launch (the workspace is sized for it)

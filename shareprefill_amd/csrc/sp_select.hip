@@ -1178,8 +1178,14 @@ extern "C" int sp_queryaware_select_bf16(const void* qbar, const void* kbar, con
 struct PivotRowShared {
   RowShared row;
   unsigned long long cov, tot;
+  unsigned long long pad[RS_THREADS / SP_WAVE];
+  int last;
 };
 
+// One workgroup per (row, head).  The workgroup that finishes a head's last row (a counter in the cluster's info
+// slot 5, which is zero between calls) turns the accumulated masses into the coverage ratio, publishes the pattern
+// and leaves counter and accumulators zero again.  Invariant: state.accum and info[.][5] are zero on entry; the
+// caller's slabs start zeroed and every completed call restores that.
 __global__ __launch_bounds__(RS_THREADS) void sp_pivot_rows_kernel(sp_cluster_state st,
                                                                    const int32_t* __restrict__ head_cluster,
                                                                    const int32_t* __restrict__ decision,
@@ -1223,41 +1229,38 @@ __global__ __launch_bounds__(RS_THREADS) void sp_pivot_rows_kernel(sp_cluster_st
   if (threadIdx.x == 0) {
     if (sh.cov) atomicAdd(&accum[c * 2 + 0], sh.cov);
     if (sh.tot) atomicAdd(&accum[c * 2 + 1], sh.tot);
+    __threadfence();  // this row's pattern words and masses are visible before the row is counted
+    sh.last = atomicAdd(&st.info[c * 8 + 5], 1) == nb - 1;
   }
-}
-
-__global__ void sp_pivot_zero_kernel(sp_cluster_state st, const int32_t* __restrict__ head_cluster,
-                                     const int32_t* __restrict__ decision, int hq,
-                                     unsigned long long* __restrict__ accum) {
-  const int h = threadIdx.x;
-  if (h < hq && decision[h] == SP_DEC_DENSE) {
-    const int c = head_cluster[h];
-    if (!sp_slot_ok(st, c)) return;
-    accum[c * 2 + 0] = 0;
-    accum[c * 2 + 1] = 0;
-  }
-}
-
-__global__ void sp_pivot_finish_kernel(sp_cluster_state st, const int32_t* __restrict__ head_cluster,
-                                       const int32_t* __restrict__ decision, const float* __restrict__ avg_attn,
-                                       int hq, int nb, const unsigned long long* __restrict__ accum) {
-  const int h = threadIdx.x;
-  if (h >= hq || decision[h] != SP_DEC_DENSE) return;
-  const int c = head_cluster[h];
-  if (!sp_slot_ok(st, c)) return;
+  __syncthreads();
+  if (!sh.last) return;
+  // ---- the head's last row: every other row of it has been counted, so its atomics and stores are visible ----
+  __threadfence();
   // every out-of-range slash / vertical slot of the reference's id list is the padding id 0
   unsigned long long pad = 0;
-  for (int i = 0; i < nb; ++i) {
-    if (st.cols[(int64_t)c * nb + i]) pad += (unsigned long long)i;
-    if (st.dists[(int64_t)c * nb + i]) pad += (unsigned long long)i;
+  for (int i = threadIdx.x; i < nb; i += RS_THREADS) {
+    if (cols[i]) pad += (unsigned long long)i;
+    if (dists[i]) pad += (unsigned long long)i;
   }
-  const unsigned long long a00 = sp_to_fixed(avg_attn[(int64_t)h * nb * nb]);
-  // one IEEE operation at a time (no fused multiply-add), so the value is reproducible on a CPU
-  const double cov = __dadd_rn((double)accum[c * 2 + 0], __dmul_rn((double)pad, (double)a00));
-  const double tot = (double)accum[c * 2 + 1];
-  st.ratio[c] = tot > 0.0 ? __ddiv_rn(cov, tot) : (double)NAN;
-  __threadfence();
-  st.info[c * 8 + 1] = 1;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) pad += __shfl_xor(pad, o, SP_WAVE);
+  if ((threadIdx.x & 63) == 0) sh.pad[threadIdx.x >> 6] = pad;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    pad = 0;
+    for (int w = 0; w < RS_THREADS / SP_WAVE; ++w) pad += sh.pad[w];
+    const unsigned long long acc_cov = atomicAdd(&accum[c * 2 + 0], 0ull), acc_tot = atomicAdd(&accum[c * 2 + 1], 0ull);
+    const unsigned long long a00 = sp_to_fixed(avg_attn[(int64_t)h * nb * nb]);
+    // one IEEE operation at a time (no fused multiply-add), so the value is reproducible on a CPU
+    const double covd = __dadd_rn((double)acc_cov, __dmul_rn((double)pad, (double)a00));
+    const double totd = (double)acc_tot;
+    st.ratio[c] = totd > 0.0 ? __ddiv_rn(covd, totd) : (double)NAN;
+    accum[c * 2 + 0] = 0;
+    accum[c * 2 + 1] = 0;
+    st.info[c * 8 + 5] = 0;
+    __threadfence();
+    st.info[c * 8 + 1] = 1;
+  }
 }
 
 extern "C" int sp_pivot_update(const sp_cluster_state* state, const int32_t* head_cluster, const int32_t* decision,
@@ -1271,13 +1274,8 @@ extern "C" int sp_pivot_update(const sp_cluster_state* state, const int32_t* hea
   if (state->n_clusters == 0) return SP_OK;
   unsigned long long* accum = reinterpret_cast<unsigned long long*>(state->accum);
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_pivot_zero_kernel, dim3(1), dim3(1024), 0, s, *state, head_cluster, decision, hq, accum);
-  SP_LAUNCH_CHECK();
   hipLaunchKernelGGL(sp_pivot_rows_kernel, dim3(nb, hq), dim3(RS_THREADS), 0, s, *state, head_cluster, decision,
                      avg_attn, nb, (nb + 63) / 64, (long long)sp_thr_lt(pattern_threshold), accum);
-  SP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sp_pivot_finish_kernel, dim3(1), dim3(1024), 0, s, *state, head_cluster, decision, avg_attn, hq,
-                     nb, accum);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

@@ -250,13 +250,37 @@ def cover_select_rows(x: torch.Tensor, thr: float) -> torch.Tensor:
     return pat
 
 
-def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=None, avg_attn=None, max_pivots=0):
+def attention_workspace(n: int, hq: int, hkv: int, d: int, block_size: int, device, max_pivots: int = 0):
+    """-> (buffer, bytes in use) of the attention call's scratch on torch's CURRENT stream: the key-major repack of V,
+    the scheduler area, the pivots' row statistics and, for max_pivots > 0, room for that many heads' block sums."""
+    lib = _lib.load()
+    need = lib.sp_attn_workspace_bytes(n, hq, hkv, d, block_size)
+    if max_pivots > 0:
+        need = (need + 255) // 256 * 256 + min(max_pivots, hq) * lib.sp_attn_pivot_scratch_bytes(n, block_size)
+    return _workspace("attn_vt", need, device), need
+
+
+def repack_v(v: torch.Tensor, block_size: int, ws: torch.Tensor) -> None:
+    """Key-major repack of v [Hkv, N, D] into the attention workspace (the step depends on v alone)."""
+    lib = _lib.load()
+    _check_hnd(v, "v")
+    hkv, n, d = v.shape
+    st = lib.sp_attn_repack_v_bf16(_ptr(v), n, hkv, d, v.stride(1), v.stride(0), block_size, _ptr(ws), ws.numel(),
+                                   _stream(v.device))
+    _lib.check(st, "sp_attn_repack_v_bf16")
+
+
+def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=None, avg_attn=None, max_pivots=0,
+                           workspace=None, pair_rows=False):
     """q [Hq,N,D], k/v [Hkv,N,D] views, mask int64 [Hq,nb,nbw] -> out bf16 [N,Hq,D] contiguous.
 
     Reference: triton_block_wise_prefill_attention (shareprefill_attn.py:474-620).  avg_attn (fp32 [Hq,nb,nb],
     zero-filled) receives the block-averaged attention map of the heads whose decision is DENSE; max_pivots = how
     many such heads there can be (an upper bound the host knows): the workspace then has room to keep their block
-    sums during the forward pass, which saves the second pass over Q.K^T."""
+    sums during the forward pass, which saves the second pass over Q.K^T.
+    workspace: (buffer, bytes) from attention_workspace into which repack_v has ALREADY put this v (and the current
+    stream has been made to wait for that); by default the call takes the buffer and repacks itself.
+    pair_rows: skip the per-call analysis of which query blocks share a work item (a dense mask has no use for it)."""
     lib = _lib.load()
     _check_hnd(q, "q")
     _check_hnd(k, "k")
@@ -267,20 +291,21 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
     assert mask.is_contiguous() and mask.dtype == torch.int64
     dev = q.device
     out = torch.empty(n, hq, d, dtype=torch.bfloat16, device=dev)
-    need = lib.sp_attn_workspace_bytes(n, hq, hkv, d, block_size)
-    if avg_attn is not None and decision is not None and max_pivots > 0:
-        need = (need + 255) // 256 * 256 + min(max_pivots, hq) * lib.sp_attn_pivot_scratch_bytes(n, block_size)
-    ws = _workspace("attn_vt", need, dev)
-    st = lib.sp_attn_repack_v_bf16(_ptr(v), n, hkv, d, v.stride(1), v.stride(0), block_size, _ptr(ws), ws.numel(),
-                                   _stream(dev))
-    _lib.check(st, "sp_attn_repack_v_bf16")
+    if workspace is None:
+        pivots = max_pivots if (avg_attn is not None and decision is not None) else 0
+        ws, need = attention_workspace(n, hq, hkv, d, block_size, dev, pivots)
+        repack_v(v, block_size, ws)
+    else:
+        ws, need = workspace
     timer = kernel_timer
     if timer is not None:
         timer.start("attn")
     st = lib.sp_block_sparse_attn_fwd_bf16(_ptr(q), _ptr(k), _ptr(v), n, hq, hkv, d, q.stride(1), q.stride(0),
                                            k.stride(1), k.stride(0), v.stride(1), v.stride(0), block_size,
                                            softmax_scale, _ptr(mask), _ptr(decision), _ptr(out), _ptr(avg_attn),
-                                           _ptr(ws), need, _lib.SP_ATTN_V_REPACKED, _stream(dev))
+                                           _ptr(ws), need,
+                                           _lib.SP_ATTN_V_REPACKED | (_lib.SP_ATTN_PAIR_ROWS if pair_rows else 0),
+                                           _stream(dev))
     if timer is not None:
         timer.stop("attn")
     _lib.check(st, "sp_block_sparse_attn_fwd_bf16")

@@ -71,16 +71,10 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
     block_size = config.block_size
     nb = -(-q_len // block_size)
     sharing = module.attention_sharing
-    avg_attn = torch.zeros(1, num_heads, nb, nb, dtype=torch.float32, device=q.device)
-    if q_len < block_size:
-        # shorter than one block: a single diagonal block, nothing to select (the reference cannot run here)
-        mask = _dense_causal_mask(num_heads, nb, q.device)
-        out = ops.block_sparse_attention(q, k, v, mask, block_size, softmax_scale)
-        return out.unsqueeze(0).transpose(1, 2), avg_attn
-
     minb, maxb = budget_blocks(config.min_budget, config.max_budget, block_size)
-    if nb <= minb and getattr(config, "dense_short_prompts", True):
-        # The prompt has no more blocks than the minimum budget.  Every head's budgets are then clamped to nb
+    if q_len < block_size or (nb <= minb and getattr(config, "dense_short_prompts", True)):
+        # (a) Shorter than one block: a single diagonal block, nothing to select (the reference cannot run here).
+        # (b) The prompt has no more blocks than the minimum budget.  Every head's budgets are then clamped to nb
         # (attention_sharing.py:173-176: raised to min_budget, cut to min(max_budget, nb)), its vertical-slash set is
         # every column and every distance, and whatever the head's decision (pivot, shared, query-aware, fallback) its
         # mask is the whole lower triangle -- in this layer and, with the same prompt, in every later one.  Nothing the
@@ -88,17 +82,25 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
         # same result at a fraction of the launches.  What is not produced on this path: decisions, pivot state and
         # the pivots' block-average maps (attn_weights is all zeros).  config.dense_short_prompts = False takes the
         # full path instead.
+        avg_attn = torch.zeros(1, num_heads, nb, nb, dtype=torch.float32, device=q.device)
         mask = _dense_causal_mask(num_heads, nb, q.device)
-        out = ops.block_sparse_attention(q, k, v, mask, block_size, softmax_scale)
-        sharing.note_dense_layer(module.layer_idx, num_heads, nb)
+        out = ops.block_sparse_attention(q, k, v, mask, block_size, softmax_scale, pair_rows=True)
+        if q_len >= block_size:
+            sharing.note_dense_layer(module.layer_idx, num_heads, nb)
         return out.unsqueeze(0).transpose(1, 2), avg_attn
+
+    # Room for the block sums of this layer's possible pivots (at most 16 GiB of it; pivots beyond that take the
+    # recomputing pass).  How many heads can become pivots is known from the table alone.
+    slab = _lib.load().sp_attn_pivot_scratch_bytes(q_len, block_size)
+    max_pivots = min(sharing.max_pivots(module.layer_idx, num_heads), (16 << 30) // slab)
+    ws = ops.attention_workspace(q_len, num_heads, key_states.shape[1], head_dim, block_size, q.device, max_pivots)
+    avg_attn = torch.empty(1, num_heads, nb, nb, dtype=torch.float32, device=q.device)
+    ops.repack_v(v, block_size, ws[0])
+    avg_attn.zero_()
     plan = sharing.plan_layer(q, k, module.layer_idx, block_size, minb, maxb, config.pattern_threshold,
                               config.similarity_threshold, config.fallback_threshold, config.queryaware_threshold)
-    # room for the block sums of this layer's possible pivots (at most 16 GiB of it; pivots beyond that take the
-    # recomputing pass)
-    slab = _lib.load().sp_attn_pivot_scratch_bytes(q_len, block_size)
     out = ops.block_sparse_attention(q, k, v, plan.mask, block_size, softmax_scale, decision=plan.decision,
-                                     avg_attn=avg_attn[0], max_pivots=min(plan.max_pivots, (16 << 30) // slab))
+                                     avg_attn=avg_attn[0], max_pivots=max_pivots, workspace=ws)
     sharing.update_pivotal_attns(module.layer_idx, avg_attn, plan.decision, config.pattern_threshold)
     return out.unsqueeze(0).transpose(1, 2), avg_attn
 
