@@ -30,18 +30,38 @@ struct SelShared {
   unsigned long long bin_sum;
 };
 
-// suffix-inclusive scan of sh.sum over SEL_BINS bins (bin b <- sum of bins >= b)
+// suffix-inclusive scan of sh.sum over SEL_BINS bins (bin b <- sum of bins >= b), all SEL_THREADS threads.
+// Thread t owns bins t and t + SEL_THREADS.  Inside a wave (64 consecutive bins of either half) the suffix sums come
+// from lane shuffles; the waves' totals meet in LDS.  Integer sums: any association gives the same result.
 __device__ static void sel_suffix_scan(SelShared& sh) {
-  const int t = threadIdx.x;
-  for (int off = 1; off < SEL_BINS; off <<= 1) {
-    unsigned long long a0 = 0, a1 = 0;
-    if (t + off < SEL_BINS) a0 = sh.sum[t + off];
-    if (t + SEL_THREADS + off < SEL_BINS) a1 = sh.sum[t + SEL_THREADS + off];
-    __syncthreads();
-    sh.sum[t] += a0;
-    sh.sum[t + SEL_THREADS] += a1;
-    __syncthreads();
+  __shared__ unsigned long long wave_tot[2][SEL_THREADS / SP_WAVE];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  unsigned long long v0 = sh.sum[t], v1 = sh.sum[t + SEL_THREADS];
+#pragma unroll
+  for (int off = 1; off < SP_WAVE; off <<= 1) {
+    const unsigned long long a0 = __shfl_down(v0, off, SP_WAVE), a1 = __shfl_down(v1, off, SP_WAVE);
+    if (lane + off < SP_WAVE) {
+      v0 += a0;
+      v1 += a1;
+    }
   }
+  if (lane == 0) {
+    wave_tot[0][wave] = v0;
+    wave_tot[1][wave] = v1;
+  }
+  __syncthreads();
+  unsigned long long above0 = 0, above1 = 0;  // bins of the same half in higher waves
+#pragma unroll
+  for (int w = 0; w < SEL_THREADS / SP_WAVE; ++w) {
+    if (w > wave) {
+      above0 += wave_tot[0][w];
+      above1 += wave_tot[1][w];
+    }
+    above0 += wave_tot[1][w];  // the whole upper half lies above every bin of the lower half
+  }
+  sh.sum[t] = v0 + above0;
+  sh.sum[t + SEL_THREADS] = v1 + above1;
+  __syncthreads();
 }
 
 // ---- score_cover_idx (attn/utils.py:53-57) on [nb][nb] maps, written into bit masks -----------------

@@ -104,3 +104,65 @@ def test_patched_qwen2_model_prefill_and_generate(gpu_device, tmp_path):
             modeling_qwen2.apply_rotary_pos_emb = stock
     assert (out - ref).abs().max().item() < 0.15 and ((out - ref).abs().mean() / ref.abs().mean()).item() < 2e-2
     assert gen.shape == (1, 203)
+
+
+def test_llama31_8b_architecture_at_131072_tokens(gpu_device):
+    """The end-to-end configuration of the benchmark at its real layer shape and length: Llama-3.1-8B architecture
+    (hidden 4096, Hq32 Hkv8 head_dim 128, intermediate 14336, RoPE theta 5e5, vocab 128256, random-init bf16) cut to
+    two decoder layers, 131072 uniform-random token ids, patched with the shipped Llama-3.1-8B-Instruct table.
+      * budgets that keep every block: the last-token logits must match the stock model's (torch SDPA) -- the patch,
+        the strided q/k/v hand-over, the fused rotary pass and the attention kernel at 1024 key blocks, end to end;
+      * the benchmark's thresholds: finite logits, every head of both layers decided, density within (0, 1]."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from shareprefill_amd import SharePrefill, unpatch_model
+
+    n = 131072
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=2, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, vocab_size=128256, max_position_embeddings=n,
+                      rope_parameters={"rope_type": "default", "rope_theta": 500000.0}, rms_norm_eps=1e-5,
+                      tie_word_embeddings=False)
+    torch.manual_seed(1238)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(gpu_device):
+            model = LlamaForCausalLM(cfg)
+    finally:
+        torch.set_default_dtype(old)
+    model.eval()
+    gen = torch.Generator(device=gpu_device).manual_seed(1238)
+    ids = torch.randint(0, cfg.vocab_size, (1, n), generator=gen, device=gpu_device)
+    print("C4-shaped model test: stock SDPA forward", flush=True)
+    model.config._attn_implementation = "sdpa"
+    with torch.no_grad():
+        ref = model(ids, use_cache=False, logits_to_keep=1).logits.float()
+    print("C4-shaped model test: patched forward, every block kept", flush=True)
+    SharePrefill(model_name="meta-llama/Llama-3.1-8B-Instruct", pattern_threshold=0.95, min_budget=n, fuse_rope=True,
+                 dense_short_prompts=False)(model)
+    from transformers.models.llama import modeling_llama
+    try:
+        with torch.no_grad():
+            out = model(ids, use_cache=False, logits_to_keep=1).logits.float()
+        assert out.shape == ref.shape == (1, 1, cfg.vocab_size)
+        assert torch.isfinite(out).all()
+        # two layers of bf16 arithmetic in a different summation order
+        assert (out - ref).abs().max().item() < 0.1 and ((out - ref).abs().mean() / ref.abs().mean()).item() < 2e-2
+        hist = model.attention_sharing.decision_histogram()
+        assert sum(hist.values()) == 64
+        print("C4-shaped model test: patched forward, benchmark thresholds", flush=True)
+        unpatch_model(model)
+        SharePrefill(model_name="meta-llama/Llama-3.1-8B-Instruct", pattern_threshold=0.95, similarity_threshold=0.5,
+                     fallback_threshold=0.95, block_size=128, min_budget=1024)(model)
+        model.attention_sharing.keep_plans = True
+        with torch.no_grad():
+            out2 = model(ids, use_cache=False, logits_to_keep=1).logits.float()
+        assert torch.isfinite(out2).all()
+        hist = model.attention_sharing.decision_histogram()
+        assert sum(hist.values()) == 64
+        dens = [p.density().cpu() for p in model.attention_sharing.plans]
+        assert len(dens) == 2 and all((d > 0).all() and (d <= 1).all() for d in dens)
+    finally:
+        stock = getattr(modeling_llama.apply_rotary_pos_emb, "_shareprefill_original", None)
+        if stock is not None:
+            modeling_llama.apply_rotary_pos_emb = stock
