@@ -139,67 +139,125 @@ __device__ static __forceinline__ void lq_finish_logits(floatx16 (&acc)[4], uint
 }
 
 // ---- kernel 1: chunk partials of the row max / row sum ------------------------------------------
-__global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_stats_kernel(
+// Built for occupancy: four workgroups per CU (16 waves) hide each other's load and barrier latencies.  That needs
+// <= 128 registers per lane and <= 40 KiB of LDS per workgroup, so
+//   * the K tile goes from global memory straight into LDS (128-bit direct loads, no staging registers), unpadded,
+//     with the 16-byte chunk index XOR-swizzled by the row so that the operand reads stay conflict-free;
+//   * the product is taken transposed, S^T = K . Q^T: in the 32x32 accumulators a lane then owns ONE query (column
+//     lane % 32) and 16 of the tile's keys per 32-key group, so the running max and sum are two registers, not 32,
+//     and the fold at the end is one exchange between the two lane halves.
+#define LQ_KSW_BYTES (LQ_TILE * LQ_D * 2)  // 32 KiB: [128 keys][16 chunks of 16 bytes], chunk c of row r at c ^ (r & 15)
+
+typedef __attribute__((address_space(3))) void* lq_lds_ptr;
+typedef const __attribute__((address_space(1))) void* lq_gbl_ptr;
+
+// Eight wave-instructions per wave fill the tile: instruction `it` of wave w writes the 1 KiB segment 4 * it + w
+// (4 key rows); lane i writes chunk position i of the segment and fetches the global chunk that belongs there.
+__device__ static __forceinline__ void lq_issue_k_direct(const sp_bf16* __restrict__ k, int64_t n, int64_t sk_n, int64_t kb,
+                                                         char* ks, int wave, int lane) {
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int seg = it * 4 + wave;
+    const int row = seg * 4 + (lane >> 4);
+    const int cl = (lane & 15) ^ (row & 15);
+    int64_t key = kb + row;
+    if (key > n - 1) key = n - 1;  // rows past the end are clamped onto the last key (masked later)
+    __builtin_amdgcn_global_load_lds((lq_gbl_ptr)(k + key * sk_n + cl * 8), (lq_lds_ptr)(ks + seg * 1024), 16, 0, 0);
+  }
+}
+
+__global__ __launch_bounds__(LQ_THREADS, 4) void sp_lastq_stats_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
     int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, int n_chunks, int tiles_per_wg,
     float2* __restrict__ partial /* [hq][n_chunks][128] */) {
+  __shared__ __attribute__((aligned(1024))) char Ksw[LQ_KSW_BYTES];
   const int h = blockIdx.y;
   const int chunk = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lq = lane & 31, hi = lane >> 5;
   const sp_bf16* qh = q + (int64_t)h * sq_h;
   const sp_bf16* kh = k + (int64_t)(h / group) * sk_h;
-  bf16x8 qa[8];
+  bf16x8 qa[8];  // the lane's query (row 32 wave + lq of the last block), channels 16 ks + 8 hi .. + 7
   lq_load_q(qh, n, sq_n, wave, lane, inv_sqrt_d, qa);
-
-  float m[16], l[16];
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    m[r] = LQ_NO_MAX;
-    l[r] = 0.f;
-  }
-  __shared__ sp_bf16 Ks[LQ_TILE * LQ_KPITCH];
+  float m = LQ_NO_MAX, l = 0.f;
   const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
   const int64_t tile0 = (int64_t)chunk * tiles_per_wg;
-  LqKRegs kr;
-  if (tile0 < n_tiles) lq_fetch_k(kh, n, sk_n, tile0 * LQ_TILE, threadIdx.x, kr);
+  // byte offset of the lane's operand chunk inside a 32-key group: row lq, logical chunk 2 ks + hi
+  const int row_off = lq * 256;
   for (int t = 0; t < tiles_per_wg; ++t) {
     const int64_t tile = tile0 + t;
     if (tile >= n_tiles) break;
     const int64_t kb = tile * LQ_TILE;
     __syncthreads();  // the previous tile's operand reads are done
-    lq_store_k(Ks, threadIdx.x, kr);
+    lq_issue_k_direct(kh, n, sk_n, kb, Ksw, wave, lane);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's direct loads have landed
     __syncthreads();
-    if (t + 1 < tiles_per_wg && tile + 1 < n_tiles) lq_fetch_k(kh, n, sk_n, kb + LQ_TILE, threadIdx.x, kr);
-    floatx16 acc[4];
-    lq_tile_logits(Ks, lane, qa, acc);
-    if (kb + LQ_TILE <= n - LQ_ROWS)
-      lq_finish_logits<false>(acc, flags, kb, n, wave, lane);
-    else
-      lq_finish_logits<true>(acc, flags, kb, n, wave, lane);
+    const bool masked = kb + LQ_TILE > n - LQ_ROWS;  // (tile-uniform) reaches into the last block or past the end
+    // key <= query position  <=>  c - row <= (n - 128) - kb;  key < n  <=>  c < n - kb   (c, row: offsets in the tile)
+    const int64_t d64 = (n - LQ_ROWS) - kb, e64 = n - kb;
+    const int dlim = d64 > 1024 ? 1024 : (int)d64, elim = e64 > 1024 ? 1024 : (int)e64;
+    // the tile in two halves of 64 keys: 32 accumulator registers alive at a time
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+      // S^T: acc[j][r] = logit(key kb + 64 half + 32 j + 8 (r / 4) + 4 hi + r % 4, this lane's query)
+      floatx16 acc[2];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float tmax = fmaxf(fmaxf(acc[0][r], acc[1][r]), fmaxf(acc[2][r], acc[3][r]));
-      const float mn = fmaxf(m[r], tmax * LQ_LOG2E);
-      float add = 0.f;
+      for (int j = 0; j < 2; ++j) {
+        const char* src = Ksw + (2 * half + j) * 32 * 256 + row_off;
+        floatx16 c = {0};
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) add += __builtin_amdgcn_exp2f(__builtin_fmaf(acc[nt][r], LQ_LOG2E, -mn));
-      l[r] = __builtin_fmaf(l[r], __builtin_amdgcn_exp2f(m[r] - mn), add);
-      m[r] = mn;
+        for (int ks = 0; ks < 8; ++ks) {
+          const uint4 raw = *reinterpret_cast<const uint4*>(src + (((2 * ks + hi) ^ (lq & 15)) << 4));
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), qa[ks], c, 0, 0, 0);
+        }
+        acc[j] = c;
+      }
+      if (flags & SP_FLAG_LOGITS_BF16) {  // the reference's qk tensor is bf16 (attention_sharing.py:129-139)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            lq_floatx2 f;
+            f[0] = acc[j][r];
+            f[1] = acc[j][r + 1];
+            const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, lq_bf16x2));
+            acc[j][r] = __uint_as_float(pk << 16);
+            acc[j][r + 1] = __uint_as_float(pk & 0xffff0000u);
+          }
+      }
+      if (masked) {
+        const int row = wave * 32 + lq;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int c = 64 * half + 32 * j + 8 * (r >> 2) + 4 * hi + (r & 3);
+            if (!(c - row <= dlim && c < elim)) acc[j][r] = -INFINITY;
+          }
+      }
+      float tmax = acc[0][0];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, acc[j][r]);
+      const float mn = fmaxf(m, tmax * LQ_LOG2E);
+      float add[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) add[r & 3] += __builtin_amdgcn_exp2f(__builtin_fmaf(acc[j][r], LQ_LOG2E, -mn));
+      l = __builtin_fmaf(l, __builtin_amdgcn_exp2f(m - mn), (add[0] + add[1]) + (add[2] + add[3]));
+      m = mn;
     }
   }
-  // merge the 32 lanes that share a row: the row's maximum first, then every lane's sum is brought to that maximum
-  // once and the sums are added over a fixed xor tree (one exp2 per row instead of two per tree level)
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    float mm = m[r];
-#pragma unroll
-    for (int o = 1; o < 32; o <<= 1) mm = fmaxf(mm, __shfl_xor(mm, o, SP_WAVE));
-    float ll = l[r] * __builtin_amdgcn_exp2f(m[r] - mm);  // (a lane that saw nothing: l = 0)
-#pragma unroll
-    for (int o = 1; o < 32; o <<= 1) ll += __shfl_xor(ll, o, SP_WAVE);
-    if ((lane & 31) == 0) {
-      partial[((int64_t)h * n_chunks + chunk) * LQ_ROWS + lq_row_of(wave, lane, r)] = make_float2(mm, ll);
-    }
+  // the two lane halves hold disjoint keys of the same query
+  {
+    const float m2 = __shfl_xor(m, 32, SP_WAVE), l2 = __shfl_xor(l, 32, SP_WAVE);
+    const float mn = fmaxf(m, m2);
+    // (hi = 0 adds its own part first, then the other half's: one order for both lanes)
+    const float a = (hi ? l2 : l) * __builtin_amdgcn_exp2f((hi ? m2 : m) - mn);
+    const float b = (hi ? l : l2) * __builtin_amdgcn_exp2f((hi ? m : m2) - mn);
+    if (hi == 0) partial[((int64_t)h * n_chunks + chunk) * LQ_ROWS + wave * 32 + lq] = make_float2(mn, a + b);
   }
 }
 
