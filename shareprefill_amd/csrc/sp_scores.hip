@@ -306,12 +306,13 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
   const sp_bf16* kh = k + (int64_t)(h / group) * sk_h;
   bf16x8 qa[8];
   lq_load_q(qh, n, sq_n, wave, lane, inv_sqrt_d, qa);
-  float rm[16], rinv[16];
+  // per row: max + log2(sum), so that a probability is exp2(logit * log2 e - rm): the normalisation rides in the
+  // exponent instead of costing a multiplication per element
+  float rm[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const float2 st = rowstat[h * LQ_ROWS + lq_row_of(wave, lane, r)];
-    rm[r] = st.x;
-    rinv[r] = st.y;
+    rm[r] = st.x - __builtin_amdgcn_logf(st.y);  // st.y = 1 / sum; v_log_f32 is log2
   }
   const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
   const int64_t first = (int64_t)blockIdx.x * tiles_per_wg;
@@ -343,7 +344,7 @@ __global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
       float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[nt][r], LQ_LOG2E, -rm[r])) * rinv[r];
+        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[nt][r], LQ_LOG2E, -rm[r]));
         P[lq_row_of(wave, lane, r) * LQ_PITCH + 32 * nt + (lane & 31)] = pv;
         part[r & 3] += pv;
       }
