@@ -7,11 +7,11 @@
 // Three kernels:
 //   stats   : per (head, key chunk) the running row max / row sum of the logits (bf16 MFMA);
 //   combine : folds the chunk partials into one (max, 1/sum) per query row, in chunk order;
-//   probs   : recomputes the logits tile by tile; the column sums (vertical) start in registers and meet in LDS,
-//             the probabilities of one 128x128 tile go to LDS and all four waves sum its anti-diagonals (slash).
-//             A slash bin receives its upper part from the previous key tile; that part is carried in registers,
-//             and each workgroup recomputes one leading tile so that no cross-workgroup accumulation (and no
-//             float atomic) is needed.
+//   probs   : recomputes the logits tile by tile; the column sums (vertical) and, through a permutation of keys and
+//             query rows, the anti-diagonal sums (slash) both start in registers, and only a 32 KiB digest of the
+//             128x128 probability tile goes through LDS.  A slash bin receives its upper part from the previous key
+//             tile; that part is carried through LDS, and each workgroup recomputes one leading tile so that no
+//             cross-workgroup accumulation (and no float atomic) is needed.
 // Every sum runs in a fixed order, so results are reproducible run to run.
 #include "sp_common.h"
 
@@ -21,21 +21,21 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define LQ_ROWS 128          // query rows (= block size)
 #define LQ_TILE 128          // keys per tile
 #define LQ_D 128             // head dim
-#define LQ_THREADS 256       // 4 waves, wave w owns query rows 32w..32w+31
-#define LQ_MIN_TILES 1       // key tiles per workgroup (probs: output tiles, plus one leading tile): a power of two, at
-#define LQ_MAX_TILES 32      // most 32 -- as many as still leave about a thousand workgroups at long sequences (32 at
-                             // 128K tokens and Llama head counts), as few as give one round of ~512 at short ones (2 at 4K)
-#define LQ_PITCH 136         // LDS row pitch (floats) of the probability tile
+#define LQ_THREADS 256       // 4 waves per head, wave w owns 32 query rows of the last block
+#define LQ_MIN_TILES 1       // key tiles per workgroup of the statistics kernel: a power of two, at most 32 -- as many as
+#define LQ_MAX_TILES 32      // still leave one round of workgroups at long sequences, as few as give one at short ones
 // Row maxima are kept in base-2 units (max logit * log2 e), so a probability is one fused multiply-add and one
 // hardware exp2.  "No logit seen yet" is a large finite negative number, not -inf: then max, difference and exp2
 // need no special case (exp2(-inf - finite) = 0 for masked logits, exp2(0) * 0 for an empty history).
 #define LQ_LOG2E 1.4426950408889634f
 #define LQ_NO_MAX (-1.0e30f)
 
-// lane's A operand: scaled last-block queries, 8 k-steps x 8 bf16
+// lane's operand: scaled last-block queries, 8 k-steps x 8 bf16; MFMA row m = lane % 32 of wave w is query 32 w + m of
+// the last block, or query 127 - (32 w + m) with REVERSED
+template <bool REVERSED>
 __device__ static __forceinline__ void lq_load_q(const sp_bf16* __restrict__ q, int64_t n, int64_t sq_n, int wave, int lane,
                                         float inv_sqrt_d, bf16x8 (&qa)[8]) {
-  const int row = wave * 32 + (lane & 31);
+  const int row = REVERSED ? LQ_ROWS - 1 - (wave * 32 + (lane & 31)) : wave * 32 + (lane & 31);
   const sp_bf16* src = q + (n - LQ_ROWS + row) * sq_n + 8 * (lane >> 5);
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
@@ -53,90 +53,12 @@ __device__ static __forceinline__ void lq_load_q(const sp_bf16* __restrict__ q, 
   }
 }
 
-// ---- K tile staging: 128 keys x 128 channels bf16 through LDS (row pitch 272 bytes), coalesced ---------------
-#define LQ_KPITCH 136  // bf16 elements per LDS row of the K tile
-
-typedef uint32_t lq_u32x4 __attribute__((ext_vector_type(4)));
-struct LqKRegs {
-  lq_u32x4 v[8];
-};
-
-// thread t fetches chunk t%16 (16 bytes) of key rows t/16, t/16+16, ...; keys past the end are clamped (masked later)
-__device__ static __forceinline__ void lq_fetch_k(const sp_bf16* __restrict__ k, int64_t n, int64_t sk_n, int64_t kb, int t,
-                                         LqKRegs& kr) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    int64_t key = kb + i * 16 + (t >> 4);
-    if (key > n - 1) key = n - 1;
-    kr.v[i] = *reinterpret_cast<const lq_u32x4*>(k + key * sk_n + (t & 15) * 8);
-  }
-}
-
-__device__ static __forceinline__ void lq_store_k(sp_bf16* Ks, int t, const LqKRegs& kr) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-    *reinterpret_cast<lq_u32x4*>(Ks + (i * 16 + (t >> 4)) * LQ_KPITCH + (t & 15) * 8) = kr.v[i];
-}
-
-// logits of this wave's 32 query rows against the 128 keys of the staged tile:
-// acc[nt][r] = S[row 32w + 8(r/4) + 4(lane/32) + r%4][key kb + 32nt + lane%32]
-__device__ static __forceinline__ void lq_tile_logits(const sp_bf16* Ks, int lane, const bf16x8 (&qa)[8], floatx16 (&acc)[4]) {
-#pragma unroll
-  for (int nt = 0; nt < 4; ++nt) {
-    const sp_bf16* src = Ks + (32 * nt + (lane & 31)) * LQ_KPITCH + 8 * (lane >> 5);
-    floatx16 c = {0};
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      const uint4 raw = *reinterpret_cast<const uint4*>(src + 16 * ks);
-      c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[ks], __builtin_bit_cast(bf16x8, raw), c, 0, 0, 0);
-    }
-    acc[nt] = c;
-  }
-}
-
 __device__ static __forceinline__ int lq_row_of(int wave, int lane, int r) {
   return wave * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
 }
 
 typedef float lq_floatx2 __attribute__((ext_vector_type(2)));
 typedef __bf16 lq_bf16x2 __attribute__((ext_vector_type(2)));
-
-// Rounds the logits to bf16 (the reference's qk tensor is bf16, attention_sharing.py:129-139) with the hardware
-// round-to-nearest-even conversion, two at a time, and masks what the last query block must not see.  Only the
-// tiles that reach into the last 128 tokens (or past the sequence end) need the mask: MASKED is tile-uniform.
-template <bool MASKED>
-__device__ static __forceinline__ void lq_finish_logits(floatx16 (&acc)[4], uint32_t flags, int64_t kb, int64_t n, int wave,
-                                               int lane) {
-  if (flags & SP_FLAG_LOGITS_BF16) {
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        lq_floatx2 f;
-        f[0] = acc[nt][r];
-        f[1] = acc[nt][r + 1];
-        const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, lq_bf16x2));
-        acc[nt][r] = __uint_as_float(pk << 16);
-        acc[nt][r + 1] = __uint_as_float(pk & 0xffff0000u);
-      }
-  }
-  if (MASKED) {
-    // key <= query position  <=>  c - row <= (n - 128) - kb;  key < n  <=>  c < n - kb   (c, row: offsets in the tile)
-    const int64_t d64 = (n - LQ_ROWS) - kb, e64 = n - kb;
-    const int dlim = d64 > 1024 ? 1024 : (int)d64, elim = e64 > 1024 ? 1024 : (int)e64;
-    int ln = lane;
-    asm volatile("" : "+v"(ln));  // keeps this rare path's lane arithmetic out of the tile loop's registers
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = lq_row_of(wave, ln, r);
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        const int c = 32 * nt + (ln & 31);
-        if (!(c - row <= dlim && c < elim)) acc[nt][r] = -INFINITY;
-      }
-    }
-  }
-}
 
 // ---- kernel 1: chunk partials of the row max / row sum ------------------------------------------
 // Built for occupancy: four workgroups per CU (16 waves) hide each other's load and barrier latencies.  That needs
@@ -146,52 +68,101 @@ __device__ static __forceinline__ void lq_finish_logits(floatx16 (&acc)[4], uint
 //   * the product is taken transposed, S^T = K . Q^T: in the 32x32 accumulators a lane then owns ONE query (column
 //     lane % 32) and 16 of the tile's keys per 32-key group, so the running max and sum are two registers, not 32,
 //     and the fold at the end is one exchange between the two lane halves.
-#define LQ_KSW_BYTES (LQ_TILE * LQ_D * 2)  // 32 KiB: [128 keys][16 chunks of 16 bytes], chunk c of row r at c ^ (r & 15)
+#define LQ_KSW_BYTES (LQ_TILE * LQ_D * 2)  // 32 KiB: [128 keys][16 chunks of 16 bytes], chunk c of row r at c ^ ((r >> SWZ) & 15)
 
 typedef __attribute__((address_space(3))) void* lq_lds_ptr;
 typedef const __attribute__((address_space(1))) void* lq_gbl_ptr;
 
-// Eight wave-instructions per wave fill the tile: instruction `it` of wave w writes the 1 KiB segment 4 * it + w
+// Both kernels put TWO query heads of a kv group into one workgroup of eight waves (waves 0-3 the first head, 4-7
+// the second, each wave 32 queries of the last block): the K tile is fetched once for both, and it is the L2 -> LDS
+// traffic of these fetches that bounds the kernels otherwise (one tile per (query head, key tile): 1 GiB per pass at
+// 128K tokens and 32 heads, about 5 TB/s when nothing else is done).  A group with an odd head count leaves the second
+// half of its last workgroup without a head: those waves fetch and synchronise, and compute nothing.
+#define LQ_WG_HEADS 2
+#define LQ_WG_THREADS (LQ_THREADS * LQ_WG_HEADS)
+static inline __host__ __device__ int lq_pairs(int group) { return (group + LQ_WG_HEADS - 1) / LQ_WG_HEADS; }
+
+// Four wave-instructions per wave fill the tile: instruction `it` of wave w (0..7) writes the 1 KiB segment 8 * it + w
 // (4 key rows); lane i writes chunk position i of the segment and fetches the global chunk that belongs there.
-__device__ static __forceinline__ void lq_issue_k_direct(const sp_bf16* __restrict__ k, int64_t n, int64_t sk_n, int64_t kb,
-                                                         char* ks, int wave, int lane) {
+// SWZ = 0 serves operand reads of 16 consecutive rows, SWZ = 2 reads of rows 4 apart.
+// The address of a lane's chunk is a tile-uniform base (scalar arithmetic) plus a 32-bit lane offset that does not
+// change from tile to tile -- row (4 w + lane / 16) * stride + swizzled chunk, computed once: with SWZ = 0 the
+// chunk is the same for all four instructions, with SWZ = 2 it takes two values (it % 2).  Only the one tile that
+// reaches past the end of the sequence clamps its rows onto the last key (masked later), lane by lane.
+template <int SWZ>
+struct LqKLane {
+  uint32_t off[SWZ == 0 ? 1 : 2];
+};
+
+template <int SWZ>
+__device__ static __forceinline__ LqKLane<SWZ> lq_k_lane(int64_t sk_n, int wave8, int lane) {
+  LqKLane<SWZ> kl;
+  const int row0 = wave8 * 4 + (lane >> 4);  // instruction `it` adds 32 rows
 #pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int seg = it * 4 + wave;
-    const int row = seg * 4 + (lane >> 4);
-    const int cl = (lane & 15) ^ (row & 15);
-    int64_t key = kb + row;
-    if (key > n - 1) key = n - 1;  // rows past the end are clamped onto the last key (masked later)
-    __builtin_amdgcn_global_load_lds((lq_gbl_ptr)(k + key * sk_n + cl * 8), (lq_lds_ptr)(ks + seg * 1024), 16, 0, 0);
+  for (int v = 0; v < (SWZ == 0 ? 1 : 2); ++v) {
+    const int cl = (lane & 15) ^ (((32 * v + row0) >> SWZ) & 15);
+    kl.off[v] = (uint32_t)(row0 * (int)sk_n * 2 + cl * 16);
+  }
+  return kl;
+}
+
+template <int SWZ>
+__device__ static __forceinline__ void lq_issue_k_direct(const sp_bf16* __restrict__ k, int64_t n, int64_t sk_n, int64_t kb,
+                                                         char* ks, int wave8, int lane, const LqKLane<SWZ>& kl) {
+  if (kb + LQ_TILE <= n) {
+    const char* base = reinterpret_cast<const char*>(k + kb * sk_n);
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const char* src = base + (int64_t)it * 32 * sk_n * 2;  // uniform
+      __builtin_amdgcn_global_load_lds((lq_gbl_ptr)(src + kl.off[SWZ == 0 ? 0 : it & 1]),
+                                       (lq_lds_ptr)(ks + (it * 8 + wave8) * 1024), 16, 0, 0);
+    }
+  } else {
+#pragma unroll 1
+    for (int it = 0; it < 4; ++it) {
+      const int seg = it * 8 + wave8;
+      const int row = seg * 4 + (lane >> 4);
+      const int cl = (lane & 15) ^ ((row >> SWZ) & 15);
+      int64_t key = kb + row;
+      if (key > n - 1) key = n - 1;
+      __builtin_amdgcn_global_load_lds((lq_gbl_ptr)(k + key * sk_n + cl * 8), (lq_lds_ptr)(ks + seg * 1024), 16, 0, 0);
+    }
   }
 }
 
-__global__ __launch_bounds__(LQ_THREADS, 4) void sp_lastq_stats_kernel(
+__global__ __launch_bounds__(LQ_WG_THREADS, 4) void sp_lastq_stats_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
     int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, int n_chunks, int tiles_per_wg,
     float2* __restrict__ partial /* [hq][n_chunks][128] */) {
   __shared__ __attribute__((aligned(1024))) char Ksw[LQ_KSW_BYTES];
-  const int h = blockIdx.y;
+  const int pairs = lq_pairs(group);
+  const int kvh = blockIdx.y / pairs;
   const int chunk = blockIdx.x;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave8 = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = wave8 & 3;                                        // query band of the wave's head
+  const int hg = (blockIdx.y % pairs) * LQ_WG_HEADS + (wave8 >> 2);  // head within the kv group
+  const bool has_head = hg < group;                                  // (wave-uniform)
+  const int h = kvh * group + (has_head ? hg : 0);
   const int lq = lane & 31, hi = lane >> 5;
   const sp_bf16* qh = q + (int64_t)h * sq_h;
-  const sp_bf16* kh = k + (int64_t)(h / group) * sk_h;
+  const sp_bf16* kh = k + (int64_t)kvh * sk_h;
   bf16x8 qa[8];  // the lane's query (row 32 wave + lq of the last block), channels 16 ks + 8 hi .. + 7
-  lq_load_q(qh, n, sq_n, wave, lane, inv_sqrt_d, qa);
+  lq_load_q<false>(qh, n, sq_n, wave, lane, inv_sqrt_d, qa);
   float m = LQ_NO_MAX, l = 0.f;
   const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
   const int64_t tile0 = (int64_t)chunk * tiles_per_wg;
   // byte offset of the lane's operand chunk inside a 32-key group: row lq, logical chunk 2 ks + hi
   const int row_off = lq * 256;
+  const LqKLane<0> kl = lq_k_lane<0>(sk_n, wave8, lane);
   for (int t = 0; t < tiles_per_wg; ++t) {
     const int64_t tile = tile0 + t;
     if (tile >= n_tiles) break;
     const int64_t kb = tile * LQ_TILE;
     __syncthreads();  // the previous tile's operand reads are done
-    lq_issue_k_direct(kh, n, sk_n, kb, Ksw, wave, lane);
+    lq_issue_k_direct<0>(kh, n, sk_n, kb, Ksw, wave8, lane, kl);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's direct loads have landed
     __syncthreads();
+    if (!has_head) continue;
     const bool masked = kb + LQ_TILE > n - LQ_ROWS;  // (tile-uniform) reaches into the last block or past the end
     // key <= query position  <=>  c - row <= (n - 128) - kb;  key < n  <=>  c < n - kb   (c, row: offsets in the tile)
     const int64_t d64 = (n - LQ_ROWS) - kb, e64 = n - kb;
@@ -200,17 +171,33 @@ __global__ __launch_bounds__(LQ_THREADS, 4) void sp_lastq_stats_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
       // S^T: acc[j][r] = logit(key kb + 64 half + 32 j + 8 (r / 4) + 4 hi + r % 4, this lane's query)
+      // (the operand reads run four MFMAs ahead: issued one by one in front of their MFMA, every MFMA waits out a
+      // whole LDS round trip)
       floatx16 acc[2];
+      {
+        const char* src = Ksw + (2 * half) * 32 * 256 + row_off;
+        uint4 ring[4];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const char* src = Ksw + (2 * half + j) * 32 * 256 + row_off;
-        floatx16 c = {0};
+        for (int i = 0; i < 4; ++i) ring[i] = *reinterpret_cast<const uint4*>(src + (((2 * i + hi) ^ (lq & 15)) << 4));
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-          const uint4 raw = *reinterpret_cast<const uint4*>(src + (((2 * ks + hi) ^ (lq & 15)) << 4));
-          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), qa[ks], c, 0, 0, 0);
+        for (int i = 0; i < 16; ++i) {
+          const int j = i >> 3, ks = i & 7;
+          const uint4 raw = ring[i & 3];
+          if (ks == 0) acc[j] = floatx16{0};
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), qa[ks], acc[j], 0, 0, 0);
+          if (i + 4 < 16) {
+            const int j2 = (i + 4) >> 3, ks2 = (i + 4) & 7;
+            ring[i & 3] = *reinterpret_cast<const uint4*>(src + j2 * 32 * 256 + (((2 * ks2 + hi) ^ (lq & 15)) << 4));
+          }
         }
-        acc[j] = c;
+        // keep that order: 4 reads, then MFMA and read in turn, then the last 4 MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int i = 0; i < 12; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
       }
       if (flags & SP_FLAG_LOGITS_BF16) {  // the reference's qk tensor is bf16 (attention_sharing.py:129-139)
 #pragma unroll
@@ -257,7 +244,7 @@ __global__ __launch_bounds__(LQ_THREADS, 4) void sp_lastq_stats_kernel(
     // (hi = 0 adds its own part first, then the other half's: one order for both lanes)
     const float a = (hi ? l2 : l) * __builtin_amdgcn_exp2f((hi ? m2 : m) - mn);
     const float b = (hi ? l : l2) * __builtin_amdgcn_exp2f((hi ? m : m2) - mn);
-    if (hi == 0) partial[((int64_t)h * n_chunks + chunk) * LQ_ROWS + wave * 32 + lq] = make_float2(mn, a + b);
+    if (hi == 0 && has_head) partial[((int64_t)h * n_chunks + chunk) * LQ_ROWS + wave * 32 + lq] = make_float2(mn, a + b);
   }
 }
 
@@ -291,125 +278,221 @@ __global__ __launch_bounds__(LQ_ROWS * LQ_COMBINE_GROUPS) void sp_lastq_combine_
 }
 
 // ---- kernel 3: probabilities -> vertical / slash ------------------------------------------------------
-__global__ __launch_bounds__(LQ_THREADS, 2) void sp_lastq_probs_kernel(
+// S = Q . K^T with the queries as the A operand, so that in the 32x32 accumulators a lane owns key columns and 16
+// query rows of each: the column (vertical) sums start in registers.  Two permutations make the anti-diagonal
+// (slash) sums start in registers too:
+//   * a lane's four accumulator sets take the four CONSECUTIVE keys 4 lq .. 4 lq + 3 (the B operand of key sub-tile
+//     nt reads K row 4 lq + nt), and
+//   * MFMA row m of wave w is query 127 - (32 w + m) of the last block, i.e. the rows run backwards.
+// Element (row i' = 32 w + 8 g + 4 hi + j, key 4 lq + nt) then belongs to slash bin  kb + 4 lq + 4 G + (nt + j)  with
+// G = 8 w + 2 g + hi: the sixteen elements of a register group g fall on seven bins of the same lane, nine additions
+// without any lane exchange, and every bin offset is a multiple of four plus (nt + j).  The lane writes the seven sums
+// as two aligned 16-byte LDS stores (offsets 0..3 to Dm[G], 4..6 to Dh[G], which is Dm shifted by one chunk), 32 KiB
+// for the whole 128 x 128 tile, and a thread collects four bins with 16-byte reads:
+// an eighth of the LDS traffic of a full probability tile, and no select between this tile's and the next tile's bins.
+// Bins 128..254 of a tile belong to the next tile's first 127 tokens: they are carried through LDS, and each
+// workgroup recomputes one leading tile so that no cross-workgroup accumulation (and no float atomic) is needed.
+// LDS of the workgroup (one per CU, two waves per SIMD): two K tiles (the next one is fetched while the current one is
+// used), and per head the diagonal digest, the column partials, the carried bins and the block-sum parts.
+#define LQP_D_FLOATS (2 * 32 * LQ_TILE)  // Dm[32][128] | Dh[32][128]
+struct LqpHeadLds {
+  float D[LQP_D_FLOATS];
+  float vpart[8][LQ_TILE];  // column sums per (wave, lane half)
+  float carry[2][LQ_TILE];  // bins 128..255 of the previous tile, by tile parity
+  float bpart[2][2][4];     // [tile parity][slash, vertical][wave] block-sum parts
+  float zero16[4];
+};
+#define LQP_LDS_BYTES (2 * LQ_KSW_BYTES + LQ_WG_HEADS * sizeof(LqpHeadLds))
+
+__global__ __launch_bounds__(LQ_WG_THREADS, 2) void sp_lastq_probs_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
     int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, const float2* __restrict__ rowstat,
     float* __restrict__ vert_tok, float* __restrict__ slash_tok, float* __restrict__ vert_blk,
     float* __restrict__ slash_blk, int64_t nb, int tiles_per_wg) {
-  extern __shared__ float lds[];
-  float* P = lds;                            // [128][LQ_PITCH] probability tile (the K tile is staged here first)
-  float* vpart = lds + LQ_ROWS * LQ_PITCH;   // [8][128] column sums per (wave, lane half)
-  float* spart = vpart + 8 * LQ_TILE;        // [6][128] lower / upper anti-diagonal and column sums per row half
-  const int h = blockIdx.y;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  extern __shared__ __attribute__((aligned(1024))) char lqp_lds[];
+  char* R2 = lqp_lds;  // [2][LQ_KSW_BYTES]
+  const int pairs = lq_pairs(group);
+  const int kvh = blockIdx.y / pairs;
+  const int wave8 = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = wave8 & 3;
+  const int hg = (blockIdx.y % pairs) * LQ_WG_HEADS + (wave8 >> 2);
+  const bool has_head = hg < group;  // (wave-uniform)
+  const int h = kvh * group + (has_head ? hg : 0);
+  LqpHeadLds& L = reinterpret_cast<LqpHeadLds*>(lqp_lds + 2 * LQ_KSW_BYTES)[wave8 >> 2];
+  const int tid = threadIdx.x & (LQ_THREADS - 1);  // thread within the head's four waves
+  const int lq = lane & 31, hi = lane >> 5;
   const sp_bf16* qh = q + (int64_t)h * sq_h;
-  const sp_bf16* kh = k + (int64_t)(h / group) * sk_h;
+  const sp_bf16* kh = k + (int64_t)kvh * sk_h;
   bf16x8 qa[8];
-  lq_load_q(qh, n, sq_n, wave, lane, inv_sqrt_d, qa);
+  lq_load_q<true>(qh, n, sq_n, wave, lane, inv_sqrt_d, qa);
   // per row: max + log2(sum), so that a probability is exp2(logit * log2 e - rm): the normalisation rides in the
   // exponent instead of costing a multiplication per element
   float rm[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const float2 st = rowstat[h * LQ_ROWS + lq_row_of(wave, lane, r)];
+    const float2 st = rowstat[h * LQ_ROWS + (LQ_ROWS - 1 - lq_row_of(wave, lane, r))];
     rm[r] = st.x - __builtin_amdgcn_logf(st.y);  // st.y = 1 / sum; v_log_f32 is log2
   }
   const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
   const int64_t first = (int64_t)blockIdx.x * tiles_per_wg;
   const float inv_rows = 1.0f / (float)LQ_ROWS;
-  float carry[2] = {0.f, 0.f};  // wave 0: upper anti-diagonal parts handed from the previous tile to its two bins
-
-  // the K tile is staged in the same LDS region the probability tile is written to afterwards
-  sp_bf16* Ks = reinterpret_cast<sp_bf16*>(lds);
   const int64_t t_begin = first > 0 ? first - 1 : 0;
   const int64_t t_end = first + tiles_per_wg < n_tiles ? first + tiles_per_wg : n_tiles;
-  LqKRegs kr;
-  if (t_begin < t_end) lq_fetch_k(kh, n, sk_n, t_begin * LQ_TILE, threadIdx.x, kr);
+  float* Dm = L.D;
+  float* Dh = Dm + 32 * LQ_TILE;
+  if (tid < LQ_TILE) L.carry[(t_begin & 1) ^ 1][tid] = 0.f;  // nothing is carried into the first tile
+  if (tid < 4) L.zero16[tid] = 0.f;
+  // B operand of key sub-tile nt, k-step ks: K row 4 lq + nt, logical 16-byte chunk 2 ks + hi (swizzled by row / 4)
+  const int b_off = lq * 1024;
+  const int b_swz = lq & 15;
+
+  const LqKLane<2> kl = lq_k_lane<2>(sk_n, wave8, lane);
+  lq_issue_k_direct<2>(kh, n, sk_n, t_begin * LQ_TILE, R2 + (t_begin & 1) * LQ_KSW_BYTES, wave8, lane, kl);
   for (int64_t tile = t_begin; tile < t_end; ++tile) {
     const int64_t kb = tile * LQ_TILE;
-    lq_store_k(Ks, threadIdx.x, kr);  // (the previous iteration ended with a barrier)
-    __syncthreads();
-    if (tile + 1 < t_end) lq_fetch_k(kh, n, sk_n, kb + LQ_TILE, threadIdx.x, kr);
-    floatx16 acc[4];
-    lq_tile_logits(Ks, lane, qa, acc);
-    __syncthreads();  // every wave has its logits: the K tile may be overwritten by P
-    if (kb + LQ_TILE <= n - LQ_ROWS)
-      lq_finish_logits<false>(acc, flags, kb, n, wave, lane);
-    else
-      lq_finish_logits<true>(acc, flags, kb, n, wave, lane);
-    // probabilities (exp2(-inf) = 0 for the masked entries): the tile goes to LDS for the anti-diagonal sums, the
-    // column sums start in registers (a lane holds 16 rows of each of its 4 columns)
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      float part[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[nt][r], LQ_LOG2E, -rm[r]));
-        P[lq_row_of(wave, lane, r) * LQ_PITCH + 32 * nt + (lane & 31)] = pv;
-        part[r & 3] += pv;
-      }
-      vpart[(2 * wave + (lane >> 5)) * LQ_TILE + 32 * nt + (lane & 31)] = (part[0] + part[1]) + (part[2] + part[3]);
+    const int par = (int)(tile & 1);
+    const char* R = R2 + par * LQ_KSW_BYTES;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's direct loads of this tile have landed
+    __syncthreads();  // ... and everyone's; the previous tile's K reads and digest reads are done
+    if (tile + 1 < t_end)  // the next K tile, into the buffer the previous tile has left
+      lq_issue_k_direct<2>(kh, n, sk_n, kb + LQ_TILE, R2 + (par ^ 1) * LQ_KSW_BYTES, wave8, lane, kl);
+    if (tid == 0 && tile > first && has_head) {  // the previous tile's block sums: its parts were complete one barrier ago
+      const float* bp = &L.bpart[par ^ 1][0][0];
+      slash_blk[(int64_t)h * nb + tile - 1] = bp[0] + bp[1];
+      vert_blk[(int64_t)h * nb + tile - 1] = (bp[4] + bp[5]) + (bp[6] + bp[7]);
     }
-    __syncthreads();
-    {
-      // anti-diagonals: element (i, c) belongs to bin kb + c - i + 127.  Thread (u, hv) walks rows 64 hv .. 64 hv + 63
-      // of the wrapped diagonal u, P[i][(u + 1 + i) mod 128]; rows i <= 126 - u lie above the tile's main diagonal
-      // and belong to bin kb + 128 + u (next tile), the others to bin kb + u.  Which of the two a row feeds is the
-      // same for all rows of wave 0 (upper) and wave 3 (lower); four independent partial sums per kind.
-      int tid = threadIdx.x;
-      asm volatile("" : "+v"(tid));  // recompute the walk's addresses per tile: hoisted out of the loop they spill
-      const int u = tid & 127, hv = tid >> 7;
-      const float* col = P + (64 * hv) * LQ_PITCH;
-      float lo[4] = {0.f, 0.f, 0.f, 0.f}, hi[4] = {0.f, 0.f, 0.f, 0.f};
-      if (wave == 0) {
-#pragma unroll 8
-        for (int j = 0; j < 64; ++j) hi[j & 3] += col[j * LQ_PITCH + ((u + 1 + j) & 127)];
-      } else if (wave == 3) {
-#pragma unroll 8
-        for (int j = 0; j < 64; ++j) lo[j & 3] += col[j * LQ_PITCH + ((u + 1 + 64 + j) & 127)];
-      } else {
-        const int split = 126 - u - 64 * hv;  // rows j <= split of this half are upper rows
-#pragma unroll 8
-        for (int j = 0; j < 64; ++j) {
-          const float pv = col[j * LQ_PITCH + ((u + 1 + 64 * hv + j) & 127)];
-          hi[j & 3] += j <= split ? pv : 0.f;
-          lo[j & 3] += j <= split ? 0.f : pv;
+    if (has_head) {
+      // acc[nt][r] = S[row i' = 32 w + 8 (r / 4) + 4 hi + r % 4][key kb + 4 lq + nt]
+      floatx16 acc[4];
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const char* src = R + b_off + nt * 256;
+        floatx16 c = {0};
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+          const uint4 raw = *reinterpret_cast<const uint4*>(src + (((2 * ks + hi) ^ b_swz) << 4));
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[ks], __builtin_bit_cast(bf16x8, raw), c, 0, 0, 0);
+        }
+        acc[nt] = c;
+      }
+      if (flags & SP_FLAG_LOGITS_BF16) {  // the reference's qk tensor is bf16 (attention_sharing.py:129-139)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            lq_floatx2 f;
+            f[0] = acc[nt][r];
+            f[1] = acc[nt][r + 1];
+            const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, lq_bf16x2));
+            acc[nt][r] = __uint_as_float(pk << 16);
+            acc[nt][r + 1] = __uint_as_float(pk & 0xffff0000u);
+          }
+      }
+      if (kb + LQ_TILE > n - LQ_ROWS) {  // (tile-uniform) the tile reaches into the last block or past the end
+        // key <= query position  <=>  c - i <= (n - 128) - kb;  key < n  <=>  c < n - kb   (c, i: offsets in the tile)
+        const int64_t d64 = (n - LQ_ROWS) - kb, e64 = n - kb;
+        const int dlim = d64 > 1024 ? 1024 : (int)d64, elim = e64 > 1024 ? 1024 : (int)e64;
+        int ln = lane;
+        asm volatile("" : "+v"(ln));  // keeps this rare path's lane arithmetic out of the tile loop's registers
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = LQ_ROWS - 1 - lq_row_of(wave, ln, r);
+#pragma unroll
+          for (int nt = 0; nt < 4; ++nt) {
+            const int c = 4 * (ln & 31) + nt;
+            if (!(c - i <= dlim && c < elim)) acc[nt][r] = -INFINITY;
+          }
         }
       }
-      spart[(0 + hv) * LQ_TILE + u] = (lo[0] + lo[1]) + (lo[2] + lo[3]);
-      spart[(2 + hv) * LQ_TILE + u] = (hi[0] + hi[1]) + (hi[2] + hi[3]);
-      // columns: fold the 8 (wave, lane half) partials, four per thread
-      const float* vp = vpart + (4 * hv) * LQ_TILE + u;
-      spart[(4 + hv) * LQ_TILE + u] = (vp[0] + vp[LQ_TILE]) + (vp[2 * LQ_TILE] + vp[3 * LQ_TILE]);
+      // probabilities (exp2(-inf) = 0 for the masked entries), column sums and the seven diagonal sums of each group
+      float vs[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float x[4][4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            x[nt][j] = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[nt][4 * g + j], LQ_LOG2E, -rm[4 * g + j]));
+            vs[nt] += x[nt][j];
+          }
+        float4 dm, dh;
+        dm.x = x[0][0];
+        dm.y = x[0][1] + x[1][0];
+        dm.z = (x[0][2] + x[1][1]) + x[2][0];
+        dm.w = (x[0][3] + x[1][2]) + (x[2][1] + x[3][0]);
+        dh.x = (x[1][3] + x[2][2]) + x[3][1];
+        dh.y = x[2][3] + x[3][2];
+        dh.z = x[3][3];
+        dh.w = 0.f;
+        const int G = 8 * wave + 2 * g + hi;
+        *reinterpret_cast<float4*>(Dm + G * LQ_TILE + 4 * lq) = dm;
+        *reinterpret_cast<float4*>(Dh + G * LQ_TILE + 4 * lq) = dh;
+      }
+      *reinterpret_cast<float4*>(&L.vpart[2 * wave + hi][4 * lq]) = make_float4(vs[0], vs[1], vs[2], vs[3]);
     }
-    __syncthreads();  // also: every wave is done with the tile, the next K tile may overwrite it
-    // Final sums, token stores and block sums: wave 0 the anti-diagonals, wave 2 the columns, two bins per lane
-    // (the tile is one 128-token block, so a wave's total is the block sum and needs no further exchange).
-    if ((wave & 1) == 0) {
+    __syncthreads();
+    if (has_head) {
       const bool emit = tile >= first;
+      // slash: thread (pg, qd) gathers bins 4 pg .. 4 pg + 3 from the eight groups G = 8 qd .. 8 qd + 7 (Dm[G] holds
+      // bins 4 G .. 4 G + 127, Dh[G] bins 4 G + 4 .. 4 G + 131), then the four lane quarters of the wave meet
       int ln = lane;
       asm volatile("" : "+v"(ln));
-      const int u0 = 2 * ln;
-      float val[2];
-      if (wave == 0) {
+      const int pg = 16 * wave + (ln & 15), qd = ln >> 4;
+      float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          val[e] = (carry[e] + (spart[u0 + e] + spart[LQ_TILE + u0 + e])) * inv_rows;
-          carry[e] = spart[2 * LQ_TILE + u0 + e] + spart[3 * LQ_TILE + u0 + e];
+      for (int gi = 0; gi < 8; ++gi) {
+        const int G = 8 * qd + gi;
+        const int cm = pg - G;  // chunk of Dm[G]; Dh[G] is one chunk behind.  Chunks outside a row read 16 zero bytes.
+        const float* am = (unsigned)cm < 32u ? Dm + G * LQ_TILE + 4 * cm : L.zero16;
+        const float* ah = (unsigned)(cm - 1) < 32u ? Dh + G * LQ_TILE + 4 * (cm - 1) : L.zero16;
+        const float4 vm = *reinterpret_cast<const float4*>(am);
+        const float4 vh = *reinterpret_cast<const float4*>(ah);
+        s.x += vm.x, s.y += vm.y, s.z += vm.z, s.w += vm.w;
+        s.x += vh.x, s.y += vh.y, s.z += vh.z, s.w += vh.w;
+      }
+      float sv[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        sv[d] += __shfl_xor(sv[d], 16, SP_WAVE);
+        sv[d] += __shfl_xor(sv[d], 32, SP_WAVE);
+      }
+      const int p0 = 4 * pg;  // 64 wave + 4 (lane % 16): waves 0, 1 hold this tile's bins, waves 2, 3 the next tile's
+      if (wave < 2) {
+        float tot = 0.f;
+        if (ln < 16) {
+          float* tok = slash_tok + (int64_t)h * n + kb + p0;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            float val = (L.carry[par ^ 1][p0 + d] + sv[d]) * inv_rows;
+            if (kb + p0 + d >= n) val = 0.f;
+            else if (emit) tok[d] = val;
+            tot += val;
+          }
         }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 2; ++e) val[e] = (spart[4 * LQ_TILE + u0 + e] + spart[5 * LQ_TILE + u0 + e]) * inv_rows;
+        tot = sp_wave_sum(tot);
+        if (ln == 0) L.bpart[par][0][wave] = tot;
+      } else if (ln < 16) {
+        *reinterpret_cast<float4*>(&L.carry[par][p0 - LQ_TILE]) = make_float4(sv[0], sv[1], sv[2], sv[3]);
       }
-      float* tok = (wave == 0 ? slash_tok : vert_tok) + (int64_t)h * n + kb;
-#pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        if (kb + u0 + e >= n) val[e] = 0.f;
-        else if (emit) tok[u0 + e] = val[e];
+      // vertical: lanes 0..31 of wave w fold the eight partials of columns 32 w .. 32 w + 31
+      float val = 0.f;
+      if (ln < 32) {
+        const int col = 32 * wave + ln;
+        val = (((L.vpart[0][col] + L.vpart[1][col]) + (L.vpart[2][col] + L.vpart[3][col])) +
+               ((L.vpart[4][col] + L.vpart[5][col]) + (L.vpart[6][col] + L.vpart[7][col]))) * inv_rows;
+        if (kb + col >= n) val = 0.f;
+        else if (emit) vert_tok[(int64_t)h * n + kb + col] = val;
       }
-      const float bsum = sp_wave_sum(val[0] + val[1]);
-      if (emit && lane == 0) (wave == 0 ? slash_blk : vert_blk)[(int64_t)h * nb + tile] = bsum;
+      val = sp_wave_sum(val);
+      if (ln == 0) L.bpart[par][1][wave] = val;
     }
+  }
+  __syncthreads();
+  if (tid == 0 && t_end > first && has_head) {  // the last tile's block sums
+    const float* bp = &L.bpart[(t_end - 1) & 1][0][0];
+    slash_blk[(int64_t)h * nb + t_end - 1] = bp[0] + bp[1];
+    vert_blk[(int64_t)h * nb + t_end - 1] = (bp[4] + bp[5]) + (bp[6] + bp[7]);
   }
 }
 
@@ -421,6 +504,20 @@ static inline int lq_tiles_per_wg(int64_t n, int32_t hq) {
   // short sequences: one round of workgroups (two per CU) rather than few long-running ones
   while (tiles > LQ_MIN_TILES && work / tiles < 512) tiles /= 2;
   return tiles;
+}
+// Output tiles per workgroup of the probabilities kernel.  A workgroup of T output tiles computes T + 1 (the leading
+// tile), and the launch runs in ceil(workgroups / 256) rounds, one workgroup per CU: take the T that minimises
+// rounds x (T + 1).
+static inline int lq_probs_tiles_per_wg(int64_t nb, int32_t wg_rows) {
+  const int64_t slots = 256;
+  int best = 1;
+  int64_t best_cost = INT64_MAX;
+  for (int t = 1; t <= 64; ++t) {
+    const int64_t wgs = sp_ceil_div(nb, t) * wg_rows;
+    const int64_t cost = sp_ceil_div(wgs, slots) * (t + (sp_ceil_div(nb, t) > 1 ? 1 : 0));
+    if (cost < best_cost) best_cost = cost, best = t;
+  }
+  return best;
 }
 // chunk count of the launch (the workspace is sized for it)
 static inline int lq_chunks(int64_t n, int32_t hq) {
@@ -461,27 +558,28 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
   const float inv_sqrt_d = 1.0f / sqrtf((float)d);
   const int group = hq / hkv;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_lastq_stats_kernel, dim3(n_chunks, hq), dim3(LQ_THREADS), 0, s, (const sp_bf16*)q,
+  const int wg_rows = hkv * lq_pairs(group);  // workgroups per key chunk: LQ_WG_HEADS heads of one kv group each
+  hipLaunchKernelGGL(sp_lastq_stats_kernel, dim3(n_chunks, wg_rows), dim3(LQ_WG_THREADS), 0, s, (const sp_bf16*)q,
                      (const sp_bf16*)k, n, hkv, group, q_stride_n, q_stride_h, k_stride_n, k_stride_h, inv_sqrt_d,
                      flags, n_chunks, tiles_per_wg, partial);
   SP_LAUNCH_CHECK();
   hipLaunchKernelGGL(sp_lastq_combine_kernel, dim3(hq), dim3(LQ_ROWS * LQ_COMBINE_GROUPS), 0, s, partial, n_chunks,
                      rowstat);
   SP_LAUNCH_CHECK();
-  const size_t lds_bytes = (LQ_ROWS * LQ_PITCH + 14 * LQ_TILE) * sizeof(float);
   static bool attr_set[64] = {false};  // per device, once (idempotent)
   int dev = 0;
   SP_HIP(hipGetDevice(&dev));
   SP_REQUIRE(dev >= 0 && dev < 64, SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: device index %d", dev);
   if (!attr_set[dev]) {
     SP_HIP(hipFuncSetAttribute((const void*)sp_lastq_probs_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)lds_bytes));
+                               (int)LQP_LDS_BYTES));
     attr_set[dev] = true;
   }
-  const int grid_x = (int)sp_ceil_div(nb, tiles_per_wg);
-  hipLaunchKernelGGL(sp_lastq_probs_kernel, dim3(grid_x, hq), dim3(LQ_THREADS), lds_bytes, s, (const sp_bf16*)q,
+  const int tiles_probs = lq_probs_tiles_per_wg(nb, wg_rows);
+  const int grid_x = (int)sp_ceil_div(nb, tiles_probs);
+  hipLaunchKernelGGL(sp_lastq_probs_kernel, dim3(grid_x, wg_rows), dim3(LQ_WG_THREADS), LQP_LDS_BYTES, s, (const sp_bf16*)q,
                      (const sp_bf16*)k, n, hkv, group, q_stride_n, q_stride_h, k_stride_n, k_stride_h, inv_sqrt_d,
-                     flags, rowstat, vert_tok, slash_tok, vert_blk, slash_blk, nb, tiles_per_wg);
+                     flags, rowstat, vert_tok, slash_tok, vert_blk, slash_blk, nb, tiles_probs);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

@@ -14,7 +14,8 @@ def _inputs(hq, hkv, n, seed):
     return q[0], k[0]  # [H, N, D] views of token-major storage
 
 
-@pytest.mark.parametrize("hq,hkv,n", [(4, 2, 1024), (8, 2, 4096), (4, 4, 1000), (2, 1, 128), (4, 1, 2304)])
+@pytest.mark.parametrize("hq,hkv,n", [(4, 2, 1024), (8, 2, 4096), (4, 4, 1000), (2, 1, 128), (4, 1, 2304),
+                                      (6, 2, 640), (7, 1, 1111)])  # odd groups: a workgroup half without a head
 @pytest.mark.parametrize("bf16_logits", [False, True])
 def test_lastq_scores_match_oracle(gpu_device, hq, hkv, n, bf16_logits):
     from shareprefill_amd import _lib, ops
