@@ -79,14 +79,18 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 // two adjacent heads (2i, 2i+1) of a kv group by sp_attn_pairing_kernel, whichever gives the smaller unions:
 //   rows  : item (h, p) = rows 2p and 2p+1 of head h (verticals are shared, slashes shift by one block);
 //   heads : item (h, p) = row 2p + (h & 1) of heads 2i and 2i+1 (heads that share a pattern keep the same columns).
-// Items are grouped in gangs of AT_GANG consecutive pairs of ONE
-// head.  Gangs are dealt statically to the 8 XCDs (queue x = gang position % 8; workgroup b serves queue b % 8
+// Items are grouped in gangs of AT_GANG consecutive pairs of ONE head (all of a head's pairs when it has fewer: a short
+// prompt's queues then hold no padding tickets, each of which would cost a workgroup an atomic and two barriers).  Gangs are dealt statically to the 8 XCDs (queue x = gang position % 8; workgroup b serves queue b % 8
 // first -- workgroups are placed on XCDs round-robin), so the 32 workgroups of an XCD start a gang together at
 // column 0 and sweep the key blocks nearly in lock-step: every K / V^T tile one of them pulls into the XCD's
 // L2 is hit by the others.  The head order inside a kv group is rotated from chunk to chunk so that every
 // queue sees every head, heavy (late) rows go first, and a workgroup whose queue is empty steals from the
 // other queues.  Pulling is by atomic tickets only: nobody ever waits for anybody, and every workgroup leaves
 // once all eight queues are exhausted.
+// Up to 32K tokens a launch has few gangs per workgroup, the heaviest of them a large part of a workgroup's whole
+// share, and every head's K / V^T fit the memory-side cache together, so the order above (one kv head after the
+// other) only makes the last kv head's heavy rows start late: there sp_attn_order_kernel ranks the gangs by the
+// number of blocks their items visit and the queues are dealt from that ranking, heaviest first.
 #define AT_GANG 32
 // The 1 KiB scheduler area (int indices): 0..127 eight queue tickets (one per 64 bytes), 128..191 the pivot slot of
 // every head (one byte each, AT_NO_SLOT = its block sums are not kept), 192..195 {shader cycles, 100 MHz ticks} of
@@ -96,32 +100,53 @@ __global__ __launch_bounds__(AT_THREADS) void sp_repack_v_kernel(const sp_bf16* 
 #define AT_SLOT_TABLE 128
 #define AT_CLOCK_SLOT 192
 #define AT_NPIV_SLOT 196
+#define AT_ORDER_SLOT 197  // 1: the gang positions of this call go through the order table (sp_attn_order_kernel)
 #define AT_PAIR_TABLE 200
 #define AT_PIVOT_TICKETS 232  // 232..239: the eight queue tickets of the pivot heads' own launch
 #define AT_NO_SLOT 255
+// Behind the 1 KiB of slots: the order table, AT_ORDER_MAX gang positions (uint16), see sp_attn_order_kernel.
+#define AT_ORDER_MAX 1024
+#define AT_SCHED_BYTES (1024 + AT_ORDER_MAX * 2)
 #define AT_MAX_HEADS 256
 #define AT_FWD_THREADS 512
 
 struct AtGeom {
-  int group, n_pairs, n_chunks, n_gangs;
+  int group, n_pairs, gang, n_chunks, n_gangs;
+  const uint16_t* order;  // gang position -> gang (nullptr: identity)
 };
 
 __device__ static inline int at_queue_items(const AtGeom& gm, int xq) {
   const int gangs = gm.n_gangs > xq ? (gm.n_gangs - xq + 7) / 8 : 0;
-  return gangs * AT_GANG;
+  return gangs * gm.gang;
+}
+
+// gang position (before any reordering) -> head and chunk of row pairs, 0 = the last (heaviest) rows
+__device__ static inline void at_gang_of(const AtGeom& gm, int pos, int& h, int& j) {
+  const int i = pos % gm.group;
+  const int rest = pos / gm.group;
+  j = rest % gm.n_chunks;
+  const int kvh = rest / gm.n_chunks;
+  h = kvh * gm.group + (i + j) % gm.group;
 }
 
 // ticket of queue xq -> (head, row pair); false for the padding slots of the last chunk
 __device__ static inline bool at_item(const AtGeom& gm, int xq, int ticket, int& h, int& pair) {
-  const int pos = (ticket / AT_GANG) * 8 + xq;  // gang position
-  const int slot = ticket % AT_GANG;
-  const int i = pos % gm.group;
-  const int rest = pos / gm.group;
-  const int j = rest % gm.n_chunks;  // chunk of pairs, 0 = the last (heaviest) rows
-  const int kvh = rest / gm.n_chunks;
-  h = kvh * gm.group + (i + j) % gm.group;
-  pair = gm.n_pairs - 1 - (j * AT_GANG + slot);
+  int pos = (ticket / gm.gang) * 8 + xq;  // gang position
+  const int slot = ticket % gm.gang;
+  if (gm.order != nullptr) pos = gm.order[pos];
+  int j;
+  at_gang_of(gm, pos, h, j);
+  pair = gm.n_pairs - 1 - (j * gm.gang + slot);
   return pair >= 0;
+}
+
+__device__ static inline void at_geometry(AtGeom& gm, int hq, int hkv, int nb) {
+  gm.group = hq / hkv;
+  gm.n_pairs = (nb + 1) / 2;
+  gm.gang = gm.n_pairs < AT_GANG ? gm.n_pairs : AT_GANG;
+  gm.n_chunks = (gm.n_pairs + gm.gang - 1) / gm.gang;
+  gm.n_gangs = hq * gm.n_chunks;
+  gm.order = nullptr;
 }
 
 // ---- LDS staging -------------------------------------------------------------------------------------------
@@ -627,10 +652,8 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
 
   const long long clk0 = clock64(), tick0 = wall_clock64();  // see sp_attn_last_launch_clocks
   AtGeom gm;
-  gm.group = hq / hkv;
-  gm.n_pairs = (nb + 1) / 2;
-  gm.n_chunks = (gm.n_pairs + AT_GANG - 1) / AT_GANG;
-  gm.n_gangs = hq * gm.n_chunks;
+  at_geometry(gm, hq, hkv, nb);
+  gm.order = sched[AT_ORDER_SLOT] != 0 ? reinterpret_cast<const uint16_t*>(sched + 256) : nullptr;
   const int xcd = blockIdx.x & 7;
   int first_try = 0;  // queues before this offset are known to be empty (used by thread 0 only)
   const int t = threadIdx.x;
@@ -970,6 +993,7 @@ __global__ void sp_attn_prep_kernel(int* __restrict__ sched, const int32_t* __re
       slots[h] = keep ? (uint8_t)cnt++ : (uint8_t)AT_NO_SLOT;
     }
     sched[AT_NPIV_SLOT] = cnt;
+    sched[AT_ORDER_SLOT] = 0;
   }
 }
 
@@ -1008,6 +1032,53 @@ __global__ __launch_bounds__(256) void sp_attn_pairing_kernel(int* __restrict__ 
   atomicAdd(&tot[1], by_heads);
   __syncthreads();
   if (threadIdx.x == 0) table[i] = tot[1] < tot[0] ? 1 : 0;
+}
+
+// After sp_attn_pairing_kernel, for launches of at most AT_ORDER_MAX gangs: ranks the gangs by the work of their items
+// -- the blocks the item's two rows visit together, plus a few blocks' worth of fixed time per item -- and writes the
+// gang positions in descending order (ties: ascending position) into the order table.  One workgroup; integer
+// weights, so the ranking does not depend on the order of anything.
+#define AT_ITEM_FIXED 6  // an item's fixed time (ticket, block list, first tiles, epilogue) in units of one block visit
+__global__ __launch_bounds__(1024) void sp_attn_order_kernel(int* __restrict__ sched, const uint64_t* __restrict__ mask,
+                                                             int hq, int hkv, int nb, int nbw) {
+  __shared__ uint32_t weight[AT_ORDER_MAX];
+  AtGeom gm;
+  at_geometry(gm, hq, hkv, nb);
+  const uint8_t* pair_table = reinterpret_cast<const uint8_t*>(sched + AT_PAIR_TABLE);
+  uint16_t* order = reinterpret_cast<uint16_t*>(sched + 256);
+  for (int pos = threadIdx.x; pos < gm.n_gangs; pos += blockDim.x) {
+    int h, j;
+    at_gang_of(gm, pos, h, j);
+    const bool by_heads = pair_table[h >> 1] != 0;
+    const int h_a = by_heads ? (h & ~1) : h, h_b = by_heads ? (h | 1) : h;
+    uint32_t wsum = 0;
+    for (int slot = 0; slot < gm.gang; ++slot) {
+      const int pair = gm.n_pairs - 1 - (j * gm.gang + slot);
+      if (pair < 0) break;
+      const int r_a = by_heads ? 2 * pair + (h & 1) : 2 * pair, r_b = by_heads ? r_a : r_a + 1;
+      if (r_a >= nb) continue;
+      const bool has_b = r_b < nb;
+      const uint64_t* ma = mask + ((int64_t)h_a * nb + r_a) * nbw;
+      const uint64_t* mb = mask + ((int64_t)h_b * nb + (has_b ? r_b : r_a)) * nbw;
+      const int wmax = (has_b ? r_b : r_a) >> 6;
+      uint32_t cnt = AT_ITEM_FIXED;
+      for (int wi = 0; wi <= wmax; ++wi)
+        cnt += __builtin_popcountll(at_trim(ma[wi], wi, r_a) | (has_b ? at_trim(mb[wi], wi, r_b) : 0ull));
+      wsum += cnt;
+    }
+    weight[pos] = wsum;
+  }
+  __syncthreads();
+  for (int pos = threadIdx.x; pos < gm.n_gangs; pos += blockDim.x) {
+    const uint32_t wp = weight[pos];
+    int rank = 0;
+    for (int o = 0; o < gm.n_gangs; ++o) {
+      const uint32_t wo = weight[o];
+      rank += (wo > wp) || (wo == wp && o < pos);
+    }
+    order[rank] = (uint16_t)pos;
+  }
+  if (threadIdx.x == 0) sched[AT_ORDER_SLOT] = 1;
 }
 
 // ---- pivot heads with a slot: block-averaged attention map from the block sums the forward kernel kept ----
@@ -1151,14 +1222,15 @@ __global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_kernel(
 }
 
 // ---- host ---------------------------------------------------------------------------------------------
-// workspace layout: [ repacked V^T : hkv*nb*128*128 bf16 | 8 queue tickets : 1 KiB | row statistics : hq*n float2 ]
+// workspace layout: [ repacked V^T : hkv*nb*128*128 bf16 | scheduler area : 1 KiB of slots + 2 KiB order table |
+//                     row statistics : hq*n float2 ]
 static size_t at_vt_bytes(int64_t n, int32_t hkv, int32_t d, int32_t bs) {
   return (size_t)hkv * (size_t)sp_ceil_div(n, bs) * bs * d * sizeof(sp_bf16);
 }
 
 extern "C" size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs) {
   if (n <= 0 || hq <= 0 || hkv <= 0 || d <= 0 || bs <= 0) return 0;
-  return at_vt_bytes(n, hkv, d, bs) + 1024 + (size_t)hq * (size_t)n * sizeof(float2);
+  return at_vt_bytes(n, hkv, d, bs) + AT_SCHED_BYTES + (size_t)hq * (size_t)n * sizeof(float2);
 }
 
 // block sums of one pivot head: fp32 [nb*(nb+1)/2 lower-triangular blocks][128 queries]
@@ -1243,7 +1315,7 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   const float scale_log2 = softmax_scale * 1.4426950408889634f;
   char* ws = (char*)workspace;
   int* counter = reinterpret_cast<int*>(ws + at_vt_bytes(n, hkv, d, bs));
-  float2* rowstat = reinterpret_cast<float2*>(ws + at_vt_bytes(n, hkv, d, bs) + 1024);
+  float2* rowstat = reinterpret_cast<float2*>(ws + at_vt_bytes(n, hkv, d, bs) + AT_SCHED_BYTES);
   const bool want_avg = decision != nullptr && avg_attn != nullptr;
   hipStream_t s = (hipStream_t)stream;
   // Workspace beyond the base size holds the block sums of pivot heads, one slab per pivot: those heads run in a
@@ -1264,6 +1336,17 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
     hipLaunchKernelGGL(sp_attn_pairing_kernel, dim3((unsigned)((hq + 1) / 2)), dim3(256), 0, s, counter, mask, (int)hq,
                        (int)(hq / hkv), (int)nb, (int)((nb + 63) / 64), max_pivots > 0 ? 1 : 0);
     SP_LAUNCH_CHECK();
+    // few gangs per workgroup and every head's K / V^T within the memory-side cache: deal the gangs heaviest first
+    // (measured on dense masks: +6 % at 16K tokens, +4 % at 32K; at 8K and below the ranking launch costs more
+    // than the better tail is worth)
+    const int64_t n_pairs = (nb + 1) / 2;
+    const int64_t gang = n_pairs < AT_GANG ? n_pairs : AT_GANG;
+    const int64_t n_gangs = hq * sp_ceil_div(n_pairs, gang);
+    if (nb > 64 && nb <= 256 && n_gangs <= AT_ORDER_MAX) {
+      hipLaunchKernelGGL(sp_attn_order_kernel, dim3(1), dim3(1024), 0, s, counter, mask, (int)hq, (int)hkv, (int)nb,
+                         (int)((nb + 63) / 64));
+      SP_LAUNCH_CHECK();
+    }
   }
   const size_t lds_bytes = AT_LDS_BYTES;
   // per device, once: the kernels' LDS allowance and the CU count (idempotent, so a race between two host threads

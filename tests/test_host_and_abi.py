@@ -47,7 +47,7 @@ def test_library_identity_and_error_string():
     # 1024 key tiles in chunks of 32 (the launch's own chunking at this size) + the folded row statistics
     assert lib.sp_lastq_scores_workspace_bytes(131072, 32, 128) == (32 * 32 * 128 + 32 * 128) * 8
     assert lib.sp_lastq_scores_workspace_bytes(4096, 32, 128) == (32 * 16 * 128 + 32 * 128) * 8  # two tiles per chunk
-    assert lib.sp_attn_workspace_bytes(131072, 32, 8, 128, 128) == 8 * 131072 * 128 * 2 + 1024 + 32 * 131072 * 8
+    assert lib.sp_attn_workspace_bytes(131072, 32, 8, 128, 128) == 8 * 131072 * 128 * 2 + 3072 + 32 * 131072 * 8
 
 
 def test_cluster_state_struct_matches_header_layout():
