@@ -238,8 +238,12 @@ class AttentionSharing:
         Returns (block bit mask [B, Hq, nb, nbw], use_dense bool [B, Hq]).  With as_ids=True the first value is the
         reference's form instead (attention_sharing.py:366): list[B][Hq] of sorted unique int64 flat block ids
         row * nb + col; building the ragged lists synchronises the stream."""
-        if gqa_interleave:
-            raise NotImplementedError("gqa_interleave=True (query head h -> kv head h % Hkv) is not supported")
+        if gqa_interleave and k.shape[2] != q.shape[2]:
+            # with un-expanded K the reference's second einsum (attention_sharing.py:141-151) gives query head h the kv
+            # head h % Hkv; its own attention function never gets here with un-expanded K (it expands first, after
+            # which the flag changes nothing), so only this direct call can ask for that mapping
+            raise NotImplementedError("gqa_interleave=True with un-expanded K (query head h -> kv head h % Hkv) is not "
+                                      "supported; with K expanded to the query head count the flag changes nothing")
         if q.shape[0] != 1:
             raise ValueError("SharePrefill keeps per-cluster state for batch size 1 only")
         plan = self.plan_layer(q[0].transpose(0, 1), k[0].transpose(0, 1), layer_idx, block_size, min_budget,

@@ -48,8 +48,12 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
     bsz, num_heads, q_len, head_dim = query_states.shape
     config = module.config
     softmax_scale = getattr(module, "scaling", 1.0 / math.sqrt(head_dim))
-    if gqa_interleave:
-        raise NotImplementedError("gqa_interleave=True (query head h -> kv head h % Hkv) is not supported")
+    # gqa_interleave is accepted and changes nothing, as in the reference: there K and V are expanded to the query
+    # head count before anything else, by repeat_interleave (True) or by expand + reshape (False) -- both give query
+    # head h the kv head h // g (shareprefill_attn.py:33-40, 77-82) -- and everything after sees one kv head per query
+    # head, so neither the selection's einsum (attention_sharing.py:128-151) nor the kernel's head mapping
+    # (shareprefill_attn.py:333-336) can tell the two settings apart.  Here K and V stay un-expanded and are indexed h // g.
+    del gqa_interleave
 
     if q_len == 1:
         # decode step (shareprefill_attn.py:146-155): one query against the whole cache, nothing is selected.

@@ -281,8 +281,13 @@ def test_reference_style_interfaces(gpu_device, tmp_path):
     assert len(dense_heads) == 2
     for h in dense_heads:  # all lower-triangular ids, attention_sharing.py:217-219
         assert ids[h].cpu().tolist() == [r * 8 + c for r in range(8) for c in range(r + 1)]
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError):  # un-expanded K: the reference would map head h to kv head h % Hkv
         sharing.get_active_blocks(qn, kn, 0, hq, 128, 8, 2 ** 24, gqa_interleave=True)
+    # K expanded to the query head count, as the reference's attention function passes it: the flag changes nothing
+    sharing.reset_state()
+    k_exp = kn.repeat_interleave(hq // kn.shape[2], dim=2)
+    mask_i, dense_i = sharing.get_active_blocks(qn, k_exp, 0, hq, 128, 8, 2 ** 24, 0.9, 0.5, 0.9, 0.1, gqa_interleave=True)
+    assert torch.equal(mask_i, mask) and torch.equal(dense_i, use_dense)
     with pytest.raises(ValueError):
         sharing.get_active_blocks(qn.expand(2, -1, -1, -1), kn.expand(2, -1, -1, -1), 0, hq, 128, 8, 2 ** 24)
     sharing.reset_state()
@@ -306,6 +311,10 @@ def test_forward_rejects_sliding_window_and_handles_short_and_decode(gpu_device,
     ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float().repeat_interleave(2, 1),
                                                            v.float().repeat_interleave(2, 1), is_causal=True)
     assert (out.transpose(1, 2).float() - ref).abs().max().item() <= MAX_ABS
+    # gqa_interleave: accepted, and (as in the reference, which expands K / V the same way under both settings)
+    # without any effect
+    out_i, _ = shareprefill_attention_forward(mod, q, k, v, None, scaling=1.0, gqa_interleave=True)
+    assert torch.equal(out_i, out)
     out1, w1 = shareprefill_attention_forward(mod, q[:, :, -1:], k, v, None, scaling=1.0)  # decode step
     assert w1 is None and out1.shape == (1, 1, 4, 128)
     assert (out1[0, 0].float() - ref[0, :, -1].float()).abs().max().item() <= MAX_ABS

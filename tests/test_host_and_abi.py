@@ -229,8 +229,9 @@ def test_attention_forward_argument_errors(tmp_path):
     k = torch.zeros(1, 1, 256, 128, dtype=torch.bfloat16)
     with pytest.raises(NotImplementedError):
         shareprefill_attention_forward(mod, q, k, k, None, scaling=0.1, sliding_window=128)
-    with pytest.raises(NotImplementedError):
-        shareprefill_attention_forward(mod, q, k, k, None, scaling=0.1, gqa_interleave=True)
+    with pytest.raises(ValueError):  # gqa_interleave is accepted (it changes nothing, as in the reference): batch 2 is what fails
+        shareprefill_attention_forward(mod, q.expand(2, -1, -1, -1), k.expand(2, -1, -1, -1), k.expand(2, -1, -1, -1),
+                                       None, scaling=0.1, gqa_interleave=True)
     with pytest.raises(ValueError):
         shareprefill_attention_forward(mod, q.expand(2, -1, -1, -1), k.expand(2, -1, -1, -1), k.expand(2, -1, -1, -1),
                                        None, scaling=0.1)
