@@ -61,8 +61,9 @@ typedef float lq_floatx2 __attribute__((ext_vector_type(2)));
 typedef __bf16 lq_bf16x2 __attribute__((ext_vector_type(2)));
 
 // ---- kernel 1: chunk partials of the row max / row sum ------------------------------------------
-// Built for occupancy: four workgroups per CU (16 waves) hide each other's load and barrier latencies.  That needs
-// <= 128 registers per lane and <= 40 KiB of LDS per workgroup, so
+// Built for occupancy: sixteen waves per CU (two workgroups of two heads) hide each other's load and barrier
+// latencies (fetching the next tile while the current one is used changes nothing on top of that).  That needs
+// <= 128 registers per lane and <= 80 KiB of LDS per workgroup, so
 //   * the K tile goes from global memory straight into LDS (128-bit direct loads, no staging registers), unpadded,
 //     with the 16-byte chunk index XOR-swizzled by the row so that the operand reads stay conflict-free;
 //   * the product is taken transposed, S^T = K . Q^T: in the 32x32 accumulators a lane then owns ONE query (column
@@ -171,33 +172,17 @@ __global__ __launch_bounds__(LQ_WG_THREADS, 4) void sp_lastq_stats_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
       // S^T: acc[j][r] = logit(key kb + 64 half + 32 j + 8 (r / 4) + 4 hi + r % 4, this lane's query)
-      // (the operand reads run four MFMAs ahead: issued one by one in front of their MFMA, every MFMA waits out a
-      // whole LDS round trip)
       floatx16 acc[2];
-      {
-        const char* src = Ksw + (2 * half) * 32 * 256 + row_off;
-        uint4 ring[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ring[i] = *reinterpret_cast<const uint4*>(src + (((2 * i + hi) ^ (lq & 15)) << 4));
+      for (int j = 0; j < 2; ++j) {
+        const char* src = Ksw + (2 * half + j) * 32 * 256 + row_off;
+        floatx16 c = {0};
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int j = i >> 3, ks = i & 7;
-          const uint4 raw = ring[i & 3];
-          if (ks == 0) acc[j] = floatx16{0};
-          acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), qa[ks], acc[j], 0, 0, 0);
-          if (i + 4 < 16) {
-            const int j2 = (i + 4) >> 3, ks2 = (i + 4) & 7;
-            ring[i & 3] = *reinterpret_cast<const uint4*>(src + j2 * 32 * 256 + (((2 * ks2 + hi) ^ (lq & 15)) << 4));
-          }
+        for (int ks = 0; ks < 8; ++ks) {
+          const uint4 raw = *reinterpret_cast<const uint4*>(src + (((2 * ks + hi) ^ (lq & 15)) << 4));
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), qa[ks], c, 0, 0, 0);
         }
-        // keep that order: 4 reads, then MFMA and read in turn, then the last 4 MFMAs
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-        for (int i = 0; i < 12; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        acc[j] = c;
       }
       if (flags & SP_FLAG_LOGITS_BF16) {  // the reference's qk tensor is bf16 (attention_sharing.py:129-139)
 #pragma unroll
