@@ -37,6 +37,30 @@ def test_lastq_scores_match_oracle(gpu_device, hq, hkv, n, bf16_logits):
     assert torch.allclose(sb, O.block_sum(st, 128), rtol=1e-5, atol=1e-9)
 
 
+def test_lastq_scores_seeded_random_shapes(gpu_device):
+    """Ragged lengths around the tile and chunk boundaries and every group size up to 8 (odd groups leave half of a
+    two-head workgroup empty), fp32 logits so that the tight tolerance holds element by element."""
+    import numpy as np
+
+    from shareprefill_amd import ops
+
+    rng = np.random.default_rng(20240607)
+    lengths = [128, 129, 255, 256, 257, 383, 640, 1000, 1111, 2049, 3000, 4097, 5000, 8191]
+    for case in range(24):
+        hkv = int(rng.choice([1, 2, 3]))
+        g = int(rng.choice([1, 2, 3, 4, 5, 7, 8]))
+        n = int(rng.choice(lengths))
+        hq = hkv * g
+        q, k = _inputs(hq, hkv, n, 1000 + case)
+        vref, sref = O.lastq_scores(q, k, 128, logits_in_input_dtype=False)
+        vt, st, vb, sb = [x.cpu() for x in ops.lastq_scores(q.to(gpu_device), k.to(gpu_device), 128, 0)]
+        tag = f"case {case}: hq {hq} hkv {hkv} n {n}"
+        assert torch.allclose(vt, vref, rtol=2e-4, atol=1e-8), tag
+        assert torch.allclose(st, sref, rtol=2e-4, atol=1e-8), tag
+        assert torch.allclose(vb, O.block_sum(vt, 128), rtol=1e-5, atol=1e-9), tag
+        assert torch.allclose(sb, O.block_sum(st, 128), rtol=1e-5, atol=1e-9), tag
+
+
 def test_lastq_scores_head_major_layout_and_determinism(gpu_device):
     from shareprefill_amd import ops
 
