@@ -644,40 +644,80 @@ extern "C" int sp_cover_select_global(const float* x, const int32_t* enable, int
 #define RS_THREADS 256
 #define RS_MAX 4096
 
-// rank[i] = position of element i in (key desc, index asc) order; keys[] in LDS
-__device__ static void rs_ranks(const uint32_t* keys, int n, uint16_t* rank) {
-  for (int i = threadIdx.x; i < n; i += RS_THREADS) {
+// ---- score_cover_idx_each_row (attn/utils.py:60-76) -------------------------------------------------
+// keep[r] = first (count(cumsum < thr) + 1) entries of the sorted row, or exactly one if thr is never reached
+// Views into the kernel's dynamic LDS, carved for rows of n entries (rs_lds_bytes(n) bytes: 14 KiB at nb = 1024
+// instead of the 58 KiB a layout for the longest supported row takes, i.e. eight workgroups per CU instead of two).
+struct RowShared {
+  uint32_t* keys;                 // [n4], 16-byte aligned
+  uint16_t* rank;                 // [n4]
+  unsigned long long* sorted_fx;  // [n4]
+  unsigned long long* chunk_sum;  // [RS_THREADS]
+  uint32_t* below;
+  int* n_eff;
+};
+__host__ __device__ static inline size_t rs_lds_bytes(int n) {
+  const size_t n4 = (size_t)((n + 3) & ~3);
+  return n4 * 8 + RS_THREADS * 8 + n4 * 4 + n4 * 2 + 16;
+}
+__device__ static inline RowShared rs_carve(char* base, int n) {
+  const size_t n4 = (size_t)((n + 3) & ~3);
+  RowShared sh;
+  sh.sorted_fx = reinterpret_cast<unsigned long long*>(base);
+  sh.chunk_sum = sh.sorted_fx + n4;
+  sh.keys = reinterpret_cast<uint32_t*>(sh.chunk_sum + RS_THREADS);
+  sh.rank = reinterpret_cast<uint16_t*>(sh.keys + n4);
+  sh.below = reinterpret_cast<uint32_t*>(base + n4 * 8 + RS_THREADS * 8 + n4 * 4 + n4 * 2);
+  sh.n_eff = reinterpret_cast<int*>(sh.below + 1);
+  return sh;
+}
+
+// rank[i] for i < m among keys[0 .. m-1], four keys per LDS read; keys[m .. (m + 3) & ~3) must be zero
+__device__ static void rs_ranks4(const uint32_t* keys, int m, uint16_t* rank) {
+  const int m4 = (m + 3) & ~3;
+  for (int i = threadIdx.x; i < m; i += RS_THREADS) {
     const uint32_t ki = keys[i];
     int r = 0;
-    for (int j = 0; j < n; ++j) {
-      const uint32_t kj = keys[j];
-      r += (kj > ki) || (kj == ki && j < i);
+    for (int j = 0; j < m4; j += 4) {
+      const uint4 kj = *reinterpret_cast<const uint4*>(keys + j);
+      r += (kj.x > ki) || (kj.x == ki && j < i);
+      r += (kj.y > ki) || (kj.y == ki && j + 1 < i);
+      r += (kj.z > ki) || (kj.z == ki && j + 2 < i);
+      r += (kj.w > ki) || (kj.w == ki && j + 3 < i);
     }
     rank[i] = (uint16_t)r;
   }
 }
 
-// ---- score_cover_idx_each_row (attn/utils.py:60-76) -------------------------------------------------
-// keep[r] = first (count(cumsum < thr) + 1) entries of the sorted row, or exactly one if thr is never reached
-struct RowShared {
-  uint32_t keys[RS_MAX];
-  uint16_t rank[RS_MAX];
-  unsigned long long sorted_fx[RS_MAX];
-  unsigned long long chunk_sum[RS_THREADS];
-  uint32_t below;
-};
-
-__device__ static int rs_row_keep(const float* __restrict__ row, int n, long long t_lt, RowShared& sh) {
-  for (int i = threadIdx.x; i < n; i += RS_THREADS) sh.keys[i] = sp_sort_key(row[i]);
-  if (threadIdx.x == 0) sh.below = 0;
+// Only the row's entries up to its last non-zero key take part in the sort: the zero keys behind it sort last in
+// index order whatever stands before them (rank[i] = i), add nothing to any cumulative mass and cannot be the
+// crossing entry, so ranks, count and the "never reached -> keep one" rule come out as over the whole row.  Row r of
+// a pivot's block-average map ends at column r: a third of the comparisons of the full square on average.
+__device__ static int rs_row_keep(const float* __restrict__ row, int n, long long t_lt, const RowShared& sh) {
+  if (threadIdx.x == 0) {
+    *sh.below = 0;
+    *sh.n_eff = 0;
+  }
   __syncthreads();
-  rs_ranks(sh.keys, n, sh.rank);
+  int last = 0;
+  for (int i = threadIdx.x; i < n; i += RS_THREADS) {
+    const uint32_t key = sp_sort_key(row[i]);
+    sh.keys[i] = key;
+    if (key) last = i + 1;
+  }
+  if (last) atomicMax(sh.n_eff, last);
   __syncthreads();
-  for (int i = threadIdx.x; i < n; i += RS_THREADS) sh.sorted_fx[sh.rank[i]] = sp_to_fixed(row[i]);
+  const int m = *sh.n_eff;
+  for (int i = m + threadIdx.x; i < ((m + 3) & ~3); i += RS_THREADS) sh.keys[i] = 0;  // (past the row's end too)
+  for (int i = m + threadIdx.x; i < n; i += RS_THREADS) sh.rank[i] = (uint16_t)i;
+  __syncthreads();
+  rs_ranks4(sh.keys, m, sh.rank);
+  __syncthreads();
+  for (int i = threadIdx.x; i < m; i += RS_THREADS) sh.sorted_fx[sh.rank[i]] = sp_to_fixed(row[i]);
   __syncthreads();
   // inclusive scan of sorted_fx in contiguous per-thread chunks
-  const int per = (n + RS_THREADS - 1) / RS_THREADS;
-  const int lo = threadIdx.x * per, hi = min(lo + per, n);
+  const int per = (m + RS_THREADS - 1) / RS_THREADS;
+  const int lo = min((int)threadIdx.x * per, m), hi = min(lo + per, m);
   unsigned long long s = 0;
   for (int i = lo; i < hi; ++i) s += sh.sorted_fx[i];
   sh.chunk_sum[threadIdx.x] = s;
@@ -691,16 +731,17 @@ __device__ static int rs_row_keep(const float* __restrict__ row, int n, long lon
       cnt += (off <= (unsigned long long)t_lt);
     }
   }
-  if (cnt) atomicAdd(&sh.below, cnt);
+  if (cnt) atomicAdd(sh.below, cnt);
   __syncthreads();
-  const int c = (int)sh.below;
-  return c < n ? c + 1 : 1;
+  const int c = (int)*sh.below;
+  return c < m ? c + 1 : 1;
 }
 
 __global__ __launch_bounds__(RS_THREADS) void sp_cover_select_rows_kernel(const float* __restrict__ x, int nb, int nbw,
                                                                           long long t_lt,
                                                                           uint64_t* __restrict__ pattern) {
-  __shared__ RowShared sh;
+  extern __shared__ __attribute__((aligned(16))) char rs_lds[];
+  const RowShared sh = rs_carve(rs_lds, nb);
   const int r = blockIdx.x;
   const int keep = rs_row_keep(x + (int64_t)r * nb, nb, t_lt, sh);
   uint32_t* prow = reinterpret_cast<uint32_t*>(pattern + (int64_t)r * nbw);
@@ -718,7 +759,7 @@ __global__ __launch_bounds__(RS_THREADS) void sp_cover_select_rows_kernel(const 
 extern "C" int sp_cover_select_rows(const float* x, int32_t nb, float thr, uint64_t* pattern, sp_stream_t stream) {
   SP_REQUIRE(x && pattern && nb > 0, SP_ERR_INVALID_ARGUMENT, "sp_cover_select_rows: bad arguments");
   SP_REQUIRE(nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_cover_select_rows: nb=%d exceeds %d", nb, RS_MAX);
-  hipLaunchKernelGGL(sp_cover_select_rows_kernel, dim3(nb), dim3(RS_THREADS), 0, (hipStream_t)stream, x, nb,
+  hipLaunchKernelGGL(sp_cover_select_rows_kernel, dim3(nb), dim3(RS_THREADS), rs_lds_bytes(nb), (hipStream_t)stream, x, nb,
                      (nb + 63) / 64, (long long)sp_thr_lt(thr), pattern);
   SP_LAUNCH_CHECK();
   return SP_OK;
@@ -1196,7 +1237,6 @@ extern "C" int sp_queryaware_select_bf16(const void* qbar, const void* kbar, con
 // pivot state update (attention_sharing.py:94-103 and the vs_ratio of :278-286, computed eagerly)
 // ------------------------------------------------------------------------------------------------
 struct PivotRowShared {
-  RowShared row;
   unsigned long long cov, tot;
   unsigned long long pad[RS_THREADS / SP_WAVE];
   int last;
@@ -1213,18 +1253,20 @@ __global__ __launch_bounds__(RS_THREADS) void sp_pivot_rows_kernel(sp_cluster_st
                                                                    int nbw, long long t_lt,
                                                                    unsigned long long* __restrict__ accum) {
   __shared__ PivotRowShared sh;
+  extern __shared__ __attribute__((aligned(16))) char rs_lds[];
+  const RowShared rsh = rs_carve(rs_lds, nb);
   const int r = blockIdx.x, h = blockIdx.y;
   if (decision[h] != SP_DEC_DENSE) return;
   const int c = head_cluster[h];
   if (!sp_slot_ok(st, c)) return;  // a dense head outside every shared cluster keeps no pattern
   const float* row = avg_attn + ((int64_t)h * nb + r) * nb;
-  const int keep = rs_row_keep(row, nb, t_lt, sh.row);
+  const int keep = rs_row_keep(row, nb, t_lt, rsh);
   uint32_t* prow = reinterpret_cast<uint32_t*>(st.pattern + ((int64_t)c * nb + r) * nbw);
   for (int w = threadIdx.x; w < nbw * 2; w += RS_THREADS) {
     uint32_t bits = 0;
     for (int b = 0; b < 32; ++b) {
       const int col = w * 32 + b;
-      if (col < nb && col <= r && sh.row.rank[col] < keep) bits |= 1u << b;
+      if (col < nb && col <= r && rsh.rank[col] < keep) bits |= 1u << b;
     }
     if (r == 0 && w == 0) bits |= 1u;
     prow[w] = bits;
@@ -1294,7 +1336,7 @@ extern "C" int sp_pivot_update(const sp_cluster_state* state, const int32_t* hea
   if (state->n_clusters == 0) return SP_OK;
   unsigned long long* accum = reinterpret_cast<unsigned long long*>(state->accum);
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_pivot_rows_kernel, dim3(nb, hq), dim3(RS_THREADS), 0, s, *state, head_cluster, decision,
+  hipLaunchKernelGGL(sp_pivot_rows_kernel, dim3(nb, hq), dim3(RS_THREADS), rs_lds_bytes(nb), s, *state, head_cluster, decision,
                      avg_attn, nb, (nb + 63) / 64, (long long)sp_thr_lt(pattern_threshold), accum);
   SP_LAUNCH_CHECK();
   return SP_OK;
