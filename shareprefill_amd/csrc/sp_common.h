@@ -33,6 +33,11 @@ void sp_set_error(const char* fmt, ...);
 
 __host__ __device__ static inline int64_t sp_ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// ---- kernels of one source file launched from another ----
+// pooled block probabilities of query-aware heads on the matrix core (sp_scores.hip), head_dim 128
+int sp_block_probs_mfma_launch(const void* qbar, const void* kbar, const int32_t* decision, int32_t hq, int32_t hkv,
+                               int32_t nb, uint32_t flags, float* probs, hipStream_t stream);
+
 // ---- bf16 <-> fp32 -------------------------------------------------------------------------------
 typedef uint16_t sp_bf16;
 

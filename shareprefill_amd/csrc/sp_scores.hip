@@ -481,6 +481,192 @@ __global__ __launch_bounds__(LQ_WG_THREADS, 2) void sp_lastq_probs_kernel(
   }
 }
 
+// ---- pooled block probabilities of query-aware heads (attention_sharing.py:350-360) -------------------------------
+// probs[h][r][c] = softmax over c <= r of  bf16(qbar[r][h] / sqrt d) . kbar[c][kv head of h],  zero for c > r.
+// The same two passes as the last-query scores, over 128-row tiles of the pooled queries against 128-row tiles of
+// the pooled keys: pass 1 the row maxima and sums (transposed product, a lane owns one query), pass 2 the logits
+// again (a lane owns key columns: coalesced rows of the output), normalised in the exponent.  One workgroup per (row
+// tile, head); the K tile goes straight from global memory into LDS, XOR-swizzled; heads that are not query-aware
+// leave at once.
+#define BPM_THREADS 256
+
+// 32 segments of 1 KiB (4 pooled-key rows each): instruction `it` of wave w (0..3) fills segment 4 it + w
+__device__ static __forceinline__ void bpm_issue_k(const sp_bf16* __restrict__ kb_head, int64_t row_stride, int nb,
+                                                   int c_tile, char* ks, int wave, int lane) {
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int seg = it * 4 + wave;
+    const int row = seg * 4 + (lane >> 4);
+    const int cl = (lane & 15) ^ (row & 15);
+    int key = c_tile * LQ_TILE + row;
+    if (key > nb - 1) key = nb - 1;  // rows past the end are clamped onto the last pooled key (masked later)
+    __builtin_amdgcn_global_load_lds((lq_gbl_ptr)(kb_head + (int64_t)key * row_stride + cl * 8),
+                                     (lq_lds_ptr)(ks + seg * 1024), 16, 0, 0);
+  }
+}
+
+// elements r, r + 1 of an accumulator rounded to bf16 (hardware conversion, round to nearest even)
+__device__ static __forceinline__ void bpm_round_pair(floatx16& v, int r) {
+  lq_floatx2 f;
+  f[0] = v[r];
+  f[1] = v[r + 1];
+  const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, lq_bf16x2));
+  v[r] = __uint_as_float(pk << 16);
+  v[r + 1] = __uint_as_float(pk & 0xffff0000u);
+}
+
+__global__ __launch_bounds__(BPM_THREADS, 2) void sp_block_probs_mfma_kernel(
+    const sp_bf16* __restrict__ qbar /* [nb][hq][128] */, const sp_bf16* __restrict__ kbar /* [nb][hkv][128] */,
+    const int32_t* __restrict__ decision, int hq, int hkv, int nb, uint32_t flags, float inv_sqrt_d,
+    float* __restrict__ probs /* [hq][nb][nb] */) {
+  __shared__ __attribute__((aligned(1024))) char Ks[LQ_KSW_BYTES];
+  __shared__ float2 rstat[LQ_ROWS];
+  const int rt = blockIdx.x, h = blockIdx.y;
+  if (decision[h] != SP_DEC_QA) return;
+  const int kvh = h / (hq / hkv);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lq = lane & 31, hi = lane >> 5;
+  const sp_bf16* kb_head = kbar + (int64_t)kvh * LQ_D;
+  const int64_t k_stride = (int64_t)hkv * LQ_D;
+  // the lane's operand row: pooled query rt * 128 + 32 wave + lq (clamped), scaled and rounded as the reference's
+  // avg_q / sqrt(d) in bf16
+  bf16x8 qa[8];
+  {
+    int row = rt * LQ_ROWS + wave * 32 + lq;
+    if (row > nb - 1) row = nb - 1;
+    const sp_bf16* src = qbar + ((int64_t)row * hq + h) * LQ_D + 8 * hi;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      uint4 raw = *reinterpret_cast<const uint4*>(src + 16 * ks);
+      uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = sp_f32_to_bf16(__uint_as_float(w[j] << 16) * inv_sqrt_d);
+        const uint32_t hi16 = sp_f32_to_bf16(__uint_as_float(w[j] & 0xffff0000u) * inv_sqrt_d);
+        w[j] = lo | (hi16 << 16);
+      }
+      raw = make_uint4(w[0], w[1], w[2], w[3]);
+      qa[ks] = __builtin_bit_cast(bf16x8, raw);
+    }
+  }
+  const int row_off = lq * 256;
+
+  // ---- pass 1: row maximum (base-2 units) and sum, transposed product: the lane's query is row 32 wave + lq ----
+  {
+    float m = LQ_NO_MAX, l = 0.f;
+    const int my_row = rt * LQ_ROWS + wave * 32 + lq;
+    for (int ct = 0; ct <= rt; ++ct) {
+      __syncthreads();
+      bpm_issue_k(kb_head, k_stride, nb, ct, Ks, wave, lane);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+#pragma unroll 1
+      for (int half = 0; half < 2; ++half) {
+        floatx16 acc[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const char* src = Ks + (2 * half + j) * 32 * 256 + row_off;
+          floatx16 c = {0};
+#pragma unroll
+          for (int ks = 0; ks < 8; ++ks) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(src + (((2 * ks + hi) ^ (lq & 15)) << 4));
+            c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), qa[ks], c, 0, 0, 0);
+          }
+          acc[j] = c;
+        }
+        if (flags & SP_FLAG_LOGITS_BF16) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) bpm_round_pair(acc[j], r);
+        }
+        if (ct == rt) {  // the diagonal tile: keys beyond the row's own block (and beyond the last block) are masked
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int key = ct * LQ_TILE + 64 * half + 32 * j + 8 * (r >> 2) + 4 * hi + (r & 3);
+              if (key > my_row || key >= nb) acc[j][r] = -INFINITY;
+            }
+        }
+        float tmax = acc[0][0];
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, acc[j][r]);
+        const float mn = fmaxf(m, tmax * LQ_LOG2E);
+        float add[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) add[r & 3] += __builtin_amdgcn_exp2f(__builtin_fmaf(acc[j][r], LQ_LOG2E, -mn));
+        l = __builtin_fmaf(l, __builtin_amdgcn_exp2f(m - mn), (add[0] + add[1]) + (add[2] + add[3]));
+        m = mn;
+      }
+    }
+    const float m2 = __shfl_xor(m, 32, SP_WAVE), l2 = __shfl_xor(l, 32, SP_WAVE);
+    const float mn = fmaxf(m, m2);
+    const float a = (hi ? l2 : l) * __builtin_amdgcn_exp2f((hi ? m2 : m) - mn);
+    const float b = (hi ? l : l2) * __builtin_amdgcn_exp2f((hi ? m : m2) - mn);
+    // max + log2(sum): a probability is then exp2(logit * log2 e - that)
+    if (hi == 0) rstat[wave * 32 + lq] = make_float2(mn + __builtin_amdgcn_logf(a + b), 0.f);
+  }
+  __syncthreads();
+  float rm[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) rm[r] = rstat[lq_row_of(wave, lane, r)].x;
+
+  // ---- pass 2: probabilities; acc[nt][r] = S[row 32 wave + 8 (r / 4) + 4 hi + r % 4][key 32 nt + lq] ----
+  for (int ct = 0; ct <= rt; ++ct) {
+    __syncthreads();
+    bpm_issue_k(kb_head, k_stride, nb, ct, Ks, wave, lane);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+#pragma unroll 1
+    for (int nt = 0; nt < 4; ++nt) {
+      const char* src = Ks + nt * 32 * 256 + row_off;
+      floatx16 c = {0};
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src + (((2 * ks + hi) ^ (lq & 15)) << 4));
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[ks], __builtin_bit_cast(bf16x8, raw), c, 0, 0, 0);
+      }
+      if (flags & SP_FLAG_LOGITS_BF16) {
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) bpm_round_pair(c, r);
+      }
+      const int key = ct * LQ_TILE + 32 * nt + lq;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = rt * LQ_ROWS + lq_row_of(wave, lane, r);
+        float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(c[r], LQ_LOG2E, -rm[r]));
+        if (key > row) pv = 0.f;
+        if (row < nb && key < nb) probs[((int64_t)h * nb + row) * nb + key] = pv;
+      }
+    }
+  }
+  // the rest of the rows: zero beyond the diagonal tile
+  {
+    const int c0 = (rt + 1) * LQ_TILE;
+    for (int i = 0; i < LQ_ROWS; ++i) {
+      const int row = rt * LQ_ROWS + i;
+      if (row >= nb) break;
+      float* out = probs + ((int64_t)h * nb + row) * nb;
+      for (int c = c0 + (int)threadIdx.x; c < nb; c += BPM_THREADS) out[c] = 0.f;
+    }
+  }
+}
+
+// launcher for sp_queryaware_select_bf16 (head_dim 128)
+int sp_block_probs_mfma_launch(const void* qbar, const void* kbar, const int32_t* decision, int32_t hq, int32_t hkv,
+                               int32_t nb, uint32_t flags, float* probs, hipStream_t stream) {
+  hipLaunchKernelGGL(sp_block_probs_mfma_kernel, dim3((unsigned)sp_ceil_div(nb, LQ_ROWS), hq), dim3(BPM_THREADS), 0, stream,
+                     (const sp_bf16*)qbar, (const sp_bf16*)kbar, decision, (int)hq, (int)hkv, (int)nb, flags,
+                     1.0f / sqrtf((float)LQ_D), probs);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
 // ---- host -------------------------------------------------------------------------------------------------
 static inline int lq_tiles_per_wg(int64_t n, int32_t hq) {
   const int64_t work = sp_ceil_div(n, LQ_TILE) * hq;  // (head, key tile) pairs

@@ -1223,10 +1223,15 @@ extern "C" int sp_queryaware_select_bf16(const void* qbar, const void* kbar, con
              "sp_queryaware_select_bf16: bad shape");
   const size_t lds = (size_t)(d + nb) * sizeof(float);
   SP_REQUIRE(lds <= 60000, SP_ERR_UNSUPPORTED, "sp_queryaware_select_bf16: nb=%d too large", nb);
-  hipLaunchKernelGGL(sp_block_probs_kernel, dim3(nb, hq), dim3(BP_THREADS), lds, (hipStream_t)stream,
-                     (const sp_bf16*)qbar, (const sp_bf16*)kbar, decision, hq, hkv, d, nb, flags,
-                     1.0f / sqrtf((float)d), probs);
-  SP_LAUNCH_CHECK();
+  if (d == 128) {  // two passes on the matrix core, 128 rows per workgroup
+    const int rc = sp_block_probs_mfma_launch(qbar, kbar, decision, hq, hkv, nb, flags, probs, (hipStream_t)stream);
+    if (rc != SP_OK) return rc;
+  } else {  // one row per workgroup, fp32 dot products
+    hipLaunchKernelGGL(sp_block_probs_kernel, dim3(nb, hq), dim3(BP_THREADS), lds, (hipStream_t)stream,
+                       (const sp_bf16*)qbar, (const sp_bf16*)kbar, decision, hq, hkv, d, nb, flags,
+                       1.0f / sqrtf((float)d), probs);
+    SP_LAUNCH_CHECK();
+  }
   // score = pattern_threshold * nb evaluated in double, then taken to fp32 as a tensor comparison would
   const float score = (float)((double)pattern_threshold * (double)nb);
   return gsel_run(probs, decision, SP_DEC_QA, hq, nb, score, mask, workspace, workspace_bytes, (hipStream_t)stream,
