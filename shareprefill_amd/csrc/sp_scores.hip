@@ -262,6 +262,32 @@ __global__ __launch_bounds__(LQ_ROWS * LQ_COMBINE_GROUPS) void sp_lastq_combine_
   }
 }
 
+// Cross-lane sums without the LDS round trip of a lane permute (each costs a wave alone on its SIMD ~120 cycles of
+// waiting, and the digest reader strings twenty of them together): lanes ^ 16 and ^ 32 through the gfx950 swaps (which
+// of the two results is the lane's own does not matter to a sum), the 16 lanes of a row through DPP.
+__device__ static __forceinline__ float lq_sum_xor16(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (uint32_t)a[0]) + __builtin_bit_cast(float, (uint32_t)a[1]);
+}
+__device__ static __forceinline__ float lq_sum_xor32(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (uint32_t)a[0]) + __builtin_bit_cast(float, (uint32_t)a[1]);
+}
+template <int CTRL>
+__device__ static __forceinline__ float lq_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// the sum over all 64 lanes, in every lane; fixed order
+__device__ static __forceinline__ float lq_wave_sum(float v) {
+  v += lq_dpp<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  v += lq_dpp<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  v += lq_dpp<0x141>(v);  // row_half_mirror
+  v += lq_dpp<0x140>(v);  // row_mirror
+  return lq_sum_xor32(lq_sum_xor16(v));
+}
+
 // ---- kernel 3: probabilities -> vertical / slash ------------------------------------------------------
 // S = Q . K^T with the queries as the A operand, so that in the 32x32 accumulators a lane owns key columns and 16
 // query rows of each: the column (vertical) sums start in registers.  Two permutations make the anti-diagonal
@@ -420,42 +446,50 @@ __global__ __launch_bounds__(LQ_WG_THREADS, 2) void sp_lastq_probs_kernel(
     if (has_head) {
       const bool emit = tile >= first;
       // slash: thread (pg, qd) gathers bins 4 pg .. 4 pg + 3 from the eight groups G = 8 qd .. 8 qd + 7 (Dm[G] holds
-      // bins 4 G .. 4 G + 127, Dh[G] bins 4 G + 4 .. 4 G + 131), then the four lane quarters of the wave meet
+      // bins 4 G .. 4 G + 127, Dh[G] bins 4 G + 4 .. 4 G + 131), then the four lane quarters of the wave meet.
+      // Every LDS read of the stage -- digest chunks, carried bins, column partials -- is issued before the first
+      // use of any: one round trip for the wave instead of a chain of them.
       int ln = lane;
       asm volatile("" : "+v"(ln));
       const int pg = 16 * wave + (ln & 15), qd = ln >> 4;
-      float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+      const int p0 = 4 * pg;  // 64 wave + 4 (lane % 16): waves 0, 1 hold this tile's bins, waves 2, 3 the next tile's
+      float4 vm[8], vh[8];
 #pragma unroll
       for (int gi = 0; gi < 8; ++gi) {
         const int G = 8 * qd + gi;
         const int cm = pg - G;  // chunk of Dm[G]; Dh[G] is one chunk behind.  Chunks outside a row read 16 zero bytes.
         const float* am = (unsigned)cm < 32u ? Dm + G * LQ_TILE + 4 * cm : L.zero16;
         const float* ah = (unsigned)(cm - 1) < 32u ? Dh + G * LQ_TILE + 4 * (cm - 1) : L.zero16;
-        const float4 vm = *reinterpret_cast<const float4*>(am);
-        const float4 vh = *reinterpret_cast<const float4*>(ah);
-        s.x += vm.x, s.y += vm.y, s.z += vm.z, s.w += vm.w;
-        s.x += vh.x, s.y += vh.y, s.z += vh.z, s.w += vh.w;
+        vm[gi] = *reinterpret_cast<const float4*>(am);
+        vh[gi] = *reinterpret_cast<const float4*>(ah);
       }
-      float sv[4] = {s.x, s.y, s.z, s.w};
+      const float4 cr = *reinterpret_cast<const float4*>(&L.carry[par ^ 1][p0 & (LQ_TILE - 1)]);  // (used by waves 0, 1)
+      const int col = 32 * wave + (ln & 31);
+      float vp[8];
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        sv[d] += __shfl_xor(sv[d], 16, SP_WAVE);
-        sv[d] += __shfl_xor(sv[d], 32, SP_WAVE);
+      for (int j = 0; j < 8; ++j) vp[j] = L.vpart[j][col];
+      float sv[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int gi = 0; gi < 8; ++gi) {
+        sv[0] += vm[gi].x, sv[1] += vm[gi].y, sv[2] += vm[gi].z, sv[3] += vm[gi].w;
+        sv[0] += vh[gi].x, sv[1] += vh[gi].y, sv[2] += vh[gi].z, sv[3] += vh[gi].w;
       }
-      const int p0 = 4 * pg;  // 64 wave + 4 (lane % 16): waves 0, 1 hold this tile's bins, waves 2, 3 the next tile's
+#pragma unroll
+      for (int d = 0; d < 4; ++d) sv[d] = lq_sum_xor32(lq_sum_xor16(sv[d]));
       if (wave < 2) {
         float tot = 0.f;
         if (ln < 16) {
           float* tok = slash_tok + (int64_t)h * n + kb + p0;
+          const float crv[4] = {cr.x, cr.y, cr.z, cr.w};
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
-            float val = (L.carry[par ^ 1][p0 + d] + sv[d]) * inv_rows;
+            float val = (crv[d] + sv[d]) * inv_rows;
             if (kb + p0 + d >= n) val = 0.f;
             else if (emit) tok[d] = val;
             tot += val;
           }
         }
-        tot = sp_wave_sum(tot);
+        tot = lq_wave_sum(tot);
         if (ln == 0) L.bpart[par][0][wave] = tot;
       } else if (ln < 16) {
         *reinterpret_cast<float4*>(&L.carry[par][p0 - LQ_TILE]) = make_float4(sv[0], sv[1], sv[2], sv[3]);
@@ -463,13 +497,11 @@ __global__ __launch_bounds__(LQ_WG_THREADS, 2) void sp_lastq_probs_kernel(
       // vertical: lanes 0..31 of wave w fold the eight partials of columns 32 w .. 32 w + 31
       float val = 0.f;
       if (ln < 32) {
-        const int col = 32 * wave + ln;
-        val = (((L.vpart[0][col] + L.vpart[1][col]) + (L.vpart[2][col] + L.vpart[3][col])) +
-               ((L.vpart[4][col] + L.vpart[5][col]) + (L.vpart[6][col] + L.vpart[7][col]))) * inv_rows;
+        val = (((vp[0] + vp[1]) + (vp[2] + vp[3])) + ((vp[4] + vp[5]) + (vp[6] + vp[7]))) * inv_rows;
         if (kb + col >= n) val = 0.f;
         else if (emit) vert_tok[(int64_t)h * n + kb + col] = val;
       }
-      val = sp_wave_sum(val);
+      val = lq_wave_sum(val);
       if (ln == 0) L.bpart[par][1][wave] = val;
     }
   }
