@@ -392,11 +392,23 @@ __device__ __forceinline__ float at_max2(float a, float b) {
 // (0: sub-tile 2b-1, 1: sub-tile 2b) and which half of it P_prev belongs to.
 // Slot order: the 8 operand slots of S_out first (channel step outermost, so that the four accumulators take turns),
 // then the 8 of O (one channel tile each) and the two row-sum MFMAs; det receives the OR of P_out's packed words.
-template <bool DO_QK, bool DO_PV, int KQ, int VB, int KT>
+// The first two operands of a stage that starts with the S product of 32-key quarter KQ, fetched ahead of the stage
+// (at the end of the one before it, or right behind the block's barrier): the stage then does not open with an LDS
+// round trip in which, the other wave of the SIMD being at the same point, nobody issues anything.
+template <int KQ>
+__device__ __forceinline__ void at_prefetch_qk(const AtAddr& ad, bf16x8 (&pre)[2]) {
+  pre[0] = at_lds128_async<(KQ >> 1) * AT_KBUF_BYTES + ((KQ & 1) * 32) * 256>(ad.ka[0]);
+  pre[1] = at_lds128_async<(KQ >> 1) * AT_KBUF_BYTES + ((KQ & 1) * 32 + 16) * 256>(ad.ka[0]);
+}
+
+// PRE: operands 0 and 1 of the stage are already in flight in `pre` (at_prefetch_qk<KQ>, and nothing else has been
+// read from LDS since).  NEXT >= 0: the stage ends by fetching the first two operands of the next one, quarter NEXT.
+template <bool DO_QK, bool DO_PV, int KQ, int VB, int KT, bool PRE, int NEXT>
 __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2],
                                          const floatx4 (&s_in)[2][2], const bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
                                          floatx4 (&o)[9][2], float sc, const float (&neg_m)[2], uint32_t (&det)[2],
-                                         const bf16x8& ones) {
+                                         const bf16x8& ones, bf16x8 (&pre)[2]) {
+  static_assert(!PRE || DO_QK, "only stages that start with the S product take prefetched operands");
   constexpr int NP = (DO_QK ? 8 : 0) + (DO_PV ? 8 : 0);  // operand slots; each holds one MFMA per query tile
   static_assert(NP == 8 || NP == 16, "a fused stage has 8 or 16 operand slots");
   constexpr int EPS = 16 / NP;  // softmax elements handled per operand slot
@@ -413,7 +425,13 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
     else  // slot i: channel tile i
       opnd[k] = at_lds128_async<i * 16 * 128>(ad.va[VB][KT]);
   };
-  at_static_for<0, AHEAD>(fetch);
+  static_assert(AHEAD == 2, "the prefetched pair is the stage's look-ahead");
+  if constexpr (PRE) {
+    opnd[0] = pre[0];
+    opnd[1] = pre[1];
+  } else {
+    at_static_for<0, AHEAD>(fetch);
+  }
   AT_PIN();
   at_static_for<0, NP>([&](auto kc) {
     constexpr int k = decltype(kc)::value;
@@ -475,6 +493,10 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
     }
     AT_PIN();
   });
+  if constexpr (NEXT >= 0) {
+    at_prefetch_qk<NEXT>(ad, pre);
+    AT_PIN();
+  }
   e[15] = __builtin_amdgcn_exp2f(x[15]);
   pk[7] = at_pack2(e[14], e[15]);
   det[1] |= pk[7];
@@ -622,15 +644,17 @@ __device__ __forceinline__ void at_commit(const floatx4 (&s_prev)[2][2], bf16x8 
 // One pipeline step.  s_in = S(j) (complete), p_prev = P(j-1) not yet applied to O (HAVE_PREV), det the OR of its
 // packed words; s_out still holds S(j-1) on entry and S(j+1) on return, p_out = P(j) with its OR in det.
 // The fused stage exists once per step: O never lives in two register sets that would have to be merged.
-template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT, bool PIVOT>
+template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT, bool PIVOT, bool PRE = false, int NEXT = -1>
 __device__ __forceinline__ void at_step(const AtAddr& ad, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2],
                                         floatx4 (&s_in)[2][2], bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
                                         floatx4 (&o)[9][2], float scale_log2, float (&m_run)[2], uint32_t (&det)[2],
-                                        const bf16x8& ones, bool diag, int key_base, int t, float (&l_mark)[2]) {
+                                        const bf16x8& ones, bool diag, int key_base, int t, float (&l_mark)[2],
+                                        bf16x8 (&pre)[2]) {
   if (HAVE_PREV) at_commit<PIVOT>(s_out, p_prev, det, o, scale_log2, m_run, l_mark);
   if (diag) at_causal(s_in, key_base, t);
   const float neg_m[2] = {-m_run[0], -m_run[1]};
-  at_fused<DO_QK, HAVE_PREV, KQ, VB, KT>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, det, ones);
+  at_fused<DO_QK, HAVE_PREV, KQ, VB, KT, PRE, NEXT>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, det, ones,
+                                                    pre);
 }
 
 // PIVOT = false: every head except the pivots that have a slot in the scheduler area's table (when skip_slotted).
@@ -816,8 +840,15 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     int c_cur = -1;
     bool mine = false;
     const uint32_t my_flag = grp ? AT_IN_B : AT_IN_A;
+    // The list is read one block ahead of its use: e_next is the entry of block b + 1, and the read of block b + 2's
+    // goes out at the top of block b, unseen by the compiler (an asynchronous LDS read like the operand fetches),
+    // to be picked up when the walk moves on.  Read where it is needed, it cost every wave an LDS round trip right
+    // behind each block's barrier, where no other wave has anything to issue either.
+    uint32_t e_next = 0u, e_ahead = 0u;
+    const uint32_t blist_addr = at_lds_addr(reinterpret_cast<const char*>(blist));
     if (n_blk > 0) {
       const uint32_t e0 = entry(0);
+      e_next = entry(1);
       c_cur = (int)(e0 & AT_COL_MASK);
       mine = (e0 & my_flag) != 0u;
       issue_k(c_cur, 0, 0);
@@ -839,7 +870,11 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       __builtin_amdgcn_s_barrier();  // ... everybody's; and every wave is past block b-1
       // (hidden loop invariance: no precomputed copies of these lane constants that could be spilled)
       asm volatile("" : "+v"(lo.k), "+v"(lo.v));
-      c_next = (int)(entry(b + 1) & AT_COL_MASK);
+      c_next = (int)(e_next & AT_COL_MASK);
+      {
+        const int ba = b + 2 < n_blk ? b + 2 : n_blk - 1;
+        asm volatile("ds_read_b32 %0, %1" : "=v"(e_ahead) : "v"(blist_addr + 4u * (uint32_t)ba));
+      }
       kb = kring + ((2 * b) & 3) * AT_KBUF_BYTES;
       vb = vring + ((2 * b + 3) & 3) * AT_VBUF_BYTES;
       vb1 = vring + ((2 * b) & 3) * AT_VBUF_BYTES;
@@ -860,16 +895,17 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       feed(2);
       feed(3);
     };
-    auto step_walk = [&]() {
+    auto step_walk = [&]() {  // (every call follows a `top` of the block that ends here)
       ++b;
       if (b < n_blk) {
-        const uint32_t e = entry(b);
-        c_cur = (int)(e & AT_COL_MASK);
-        mine = (e & my_flag) != 0u;
+        c_cur = (int)(e_next & AT_COL_MASK);
+        mine = (e_next & my_flag) != 0u;
       } else {
         c_cur = -1;
         mine = false;
       }
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e_ahead));  // long since back: issued a whole block ago
+      e_next = __builtin_amdgcn_readfirstlane(e_ahead);
     };
     bool finished = false;  // the final wait + barrier has been passed
     while (c_cur >= 0) {
@@ -881,18 +917,19 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       }
       floatx4 sa[2][2], sb[2][2];  // [key tile][query tile]
       bf16x8 pa[2], pb[2];         // [query tile]
+      bf16x8 pre[2];               // the next stage's first two LDS operands, in flight (at_prefetch_qk)
       // ---- start of a run: S of the first half-tile, nothing to overlap with yet ----
       feed(0);
       at_qk_only<0>(kb, koff, qb, sa);
       feed(1);
-      at_step<true, false, 1, 0, 0, PIVOT>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
-                                           c_cur == r, 0, tq, l_mark);
+      at_step<true, false, 1, 0, 0, PIVOT, false, 2>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
+                                                     c_cur == r, 0, tq, l_mark, pre);
       feed(2);
-      at_step<true, true, 2, 1, 0, PIVOT>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
-                                          c_cur == r, 32, tq, l_mark);
+      at_step<true, true, 2, 1, 0, PIVOT, true, 3>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
+                                                   c_cur == r, 32, tq, l_mark, pre);
       feed(3);
-      at_step<true, true, 3, 1, 1, PIVOT>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
-                                          c_cur == r, AT_SUB, tq, l_mark);
+      at_step<true, true, 3, 1, 1, PIVOT, true, -1>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
+                                                    c_cur == r, AT_SUB, tq, l_mark, pre);
       int c_prev = c_cur;
       step_walk();
       // ---- steady state: four half-tile steps per block ----
@@ -901,22 +938,23 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         // The instruction arbiter favours the older waves (the even row's), which then finish the block early and
         // idle at the barrier while the odd row's waves run alone at half the matrix-core rate: the odd row gets
         // priority for the first half of the block, which evens the two out.
+        at_prefetch_qk<0>(ad, pre);  // (the block's first operands, while the loads and the commit test are set up)
         if (grp) __builtin_amdgcn_s_setprio(1);
         feed(0);
         // S(previous block, keys 96..127) -> P;  S(keys 0..31) on the matrix core;  O += V^T(2b-1, keys 0..31) . P
-        at_step<true, true, 0, 0, 0, PIVOT>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
-                                            c_prev == r, AT_SUB + 32, tq, l_mark);
+        at_step<true, true, 0, 0, 0, PIVOT, true, 1>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
+                                                     c_prev == r, AT_SUB + 32, tq, l_mark, pre);
         feed(1);
-        at_step<true, true, 1, 0, 1, PIVOT>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
-                                            c_cur == r, 0, tq, l_mark);
+        at_step<true, true, 1, 0, 1, PIVOT, true, 2>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
+                                                     c_cur == r, 0, tq, l_mark, pre);
         emit(c_prev);  // the previous block's last half-tile went into O (and the sums) in this step
         if (grp) __builtin_amdgcn_s_setprio(0);
         feed(2);
-        at_step<true, true, 2, 1, 0, PIVOT>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
-                                            c_cur == r, 32, tq, l_mark);
+        at_step<true, true, 2, 1, 0, PIVOT, true, 3>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
+                                                     c_cur == r, 32, tq, l_mark, pre);
         feed(3);
-        at_step<true, true, 3, 1, 1, PIVOT>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
-                                            c_cur == r, AT_SUB, tq, l_mark);
+        at_step<true, true, 3, 1, 1, PIVOT, true, -1>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
+                                                      c_cur == r, AT_SUB, tq, l_mark, pre);
         c_prev = c_cur;
         step_walk();
       }
@@ -933,7 +971,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         at_block_addr(ad, kb, vb, vb, koff, voff);
       }
       at_step<false, true, 0, 0, 0, PIVOT>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
-                                           c_prev == r, AT_SUB + 32, tq, l_mark);
+                                           c_prev == r, AT_SUB + 32, tq, l_mark, pre);
       at_commit<PIVOT>(sb, pb, det, o, scale_log2, m_run, l_mark);
       at_pv_only<1>(vb, voff, pb, o, ones);
       emit(c_prev);
