@@ -940,15 +940,15 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         // priority for the first half of the block, which evens the two out.
         at_prefetch_qk<0>(ad, pre);  // (the block's first operands, while the loads and the commit test are set up)
         if (grp) __builtin_amdgcn_s_setprio(1);
-        feed(0);
         // S(previous block, keys 96..127) -> P;  S(keys 0..31) on the matrix core;  O += V^T(2b-1, keys 0..31) . P
         at_step<true, true, 0, 0, 0, PIVOT, true, 1>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                                      c_prev == r, AT_SUB + 32, tq, l_mark, pre);
-        feed(1);
+        feed(0);
         at_step<true, true, 1, 0, 1, PIVOT, true, 2>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
                                                      c_cur == r, 0, tq, l_mark, pre);
         emit(c_prev);  // the previous block's last half-tile went into O (and the sums) in this step
         if (grp) __builtin_amdgcn_s_setprio(0);
+        feed(1);
         feed(2);
         at_step<true, true, 2, 1, 0, PIVOT, true, 3>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                                      c_cur == r, 32, tq, l_mark, pre);
