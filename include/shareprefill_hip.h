@@ -262,6 +262,20 @@ int sp_cover_select_rows(const float* x, int32_t nb, float thr, uint64_t* patter
  * row_ptr[h][r+1] = number of set blocks in rows 0..r of head h; row_ptr[h][0] = 0. */
 int sp_mask_row_pointers(const uint64_t* mask, int32_t hq, int32_t nb, int32_t* row_ptr, sp_stream_t stream);
 
+/* The reference's block_idx form of a selection (the argument of triton_block_wise_prefill_attention,
+ * shareprefill_attn.py:484-486, 528-540, and the first return value of get_active_blocks, attention_sharing.py:366):
+ * block_idx[h][0..k) = flat block ids row * nb + col in any order, row stride idx_stride_h elements, padded with any
+ * value outside [0, nb * nb) (the reference pads with nb * (nb + 1)).
+ * sp_block_idx_to_mask: mask[hq][nb][ceil(nb/64)] = the bit mask the attention entry point takes; ids above the
+ *   diagonal are dropped (the reference's kernel masks every element of such a block, shareprefill_attn.py:401-406).
+ * sp_block_idx_row_pointers: triton_column_count_cumsum (shareprefill_attn.py:187-269) on the ids themselves:
+ *   row_ptr[h][r+1] = number of ids with id / nb <= r (duplicates counted, as by the reference's histogram);
+ *   row_ptr[h][0] = 0.  nb <= 4096. */
+int sp_block_idx_to_mask(const int64_t* block_idx, int64_t idx_stride_h, int64_t k, int32_t hq, int32_t nb,
+                         uint64_t* mask, sp_stream_t stream);
+int sp_block_idx_row_pointers(const int64_t* block_idx, int64_t idx_stride_h, int64_t k, int32_t hq, int32_t nb,
+                              int32_t* row_ptr, sp_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

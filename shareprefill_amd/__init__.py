@@ -10,7 +10,7 @@ include/shareprefill_hip.h), built with `python -m shareprefill_amd.build`.  The
 from .attention_sharing import AttentionSharing
 from .shareprefill_attn import shareprefill_attention_forward
 from .shareprefill_configurations import SharePrefillConfig
-from . import attention_sharing, shareprefill_attn, shareprefill_configurations, shareprefill_patch
+from . import attention_sharing, shareprefill_attn, shareprefill_configurations, shareprefill_patch, utils
 from .shareprefill_patch import SharePrefill, unpatch_model
 
 __all__ = ["SharePrefill", "SharePrefillConfig", "AttentionSharing", "shareprefill_attention_forward", "unpatch_model"]

@@ -69,6 +69,8 @@ SIGNATURES = {
     "sp_pivot_update": (_I32, [_ST, _P, _P, _P, _I32, _I32, _F, _P]),
     "sp_cover_select_rows": (_I32, [_P, _I32, _F, _P, _P]),
     "sp_mask_row_pointers": (_I32, [_P, _I32, _I32, _P, _P]),
+    "sp_block_idx_to_mask": (_I32, [_P, _I64, _I64, _I32, _I32, _P, _P]),
+    "sp_block_idx_row_pointers": (_I32, [_P, _I64, _I64, _I32, _I32, _P, _P]),
 }
 
 _lib = None

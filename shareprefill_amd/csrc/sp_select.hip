@@ -1381,3 +1381,100 @@ extern "C" int sp_mask_row_pointers(const uint64_t* mask, int32_t hq, int32_t nb
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
+
+// ------------------------------------------------------------------------------------------------
+// The reference's block_idx form of a layer's selection (shareprefill_attn.py:484-486, 528-540): per head a list
+// of flat block ids row * nb + col, in any order, padded with values outside the grid (the reference pads with
+// nb * (nb + 1)).
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void sp_fill_u64_kernel(uint64_t* __restrict__ p, int64_t n, uint64_t value) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = value;
+}
+
+__global__ __launch_bounds__(256) void sp_block_idx_to_mask_kernel(const int64_t* __restrict__ idx, int64_t stride_h,
+                                                                   int64_t k, int nb, int nbw,
+                                                                   uint64_t* __restrict__ mask) {
+  const int h = blockIdx.y;
+  const int64_t cells = (int64_t)nb * nb;
+  unsigned long long* mh = reinterpret_cast<unsigned long long*>(mask) + (int64_t)h * nb * nbw;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < k; i += (int64_t)gridDim.x * 256) {
+    const int64_t id = idx[(int64_t)h * stride_h + i];
+    if (id < 0 || id >= cells) continue;  // padding
+    const int r = (int)(id / nb), c = (int)(id % nb);
+    if (c > r) continue;  // above the diagonal: the kernel's causal mask leaves nothing of such a block
+    atomicOr(mh + (int64_t)r * nbw + (c >> 6), 1ull << (c & 63));
+  }
+}
+
+extern "C" int sp_block_idx_to_mask(const int64_t* block_idx, int64_t idx_stride_h, int64_t k, int32_t hq, int32_t nb,
+                                    uint64_t* mask, sp_stream_t stream) {
+  SP_REQUIRE(mask && hq > 0 && nb > 0 && k >= 0 && (block_idx || k == 0), SP_ERR_INVALID_ARGUMENT,
+             "sp_block_idx_to_mask: bad arguments");
+  SP_REQUIRE(hq <= 65535, SP_ERR_UNSUPPORTED, "sp_block_idx_to_mask: hq=%d exceeds 65535", hq);
+  const int nbw = (nb + 63) / 64;
+  const int64_t words = (int64_t)hq * nb * nbw;
+  // a fill kernel rather than a memset node, so that the call can be recorded into a graph
+  const unsigned fill_grid = (unsigned)(sp_ceil_div(words, 256) < 4096 ? sp_ceil_div(words, 256) : 4096);
+  hipLaunchKernelGGL(sp_fill_u64_kernel, dim3(fill_grid), dim3(256), 0, (hipStream_t)stream, mask, words,
+                     (uint64_t)0);
+  SP_LAUNCH_CHECK();
+  if (k > 0) {
+    const unsigned gx = (unsigned)(sp_ceil_div(k, 256) < 1024 ? sp_ceil_div(k, 256) : 1024);
+    hipLaunchKernelGGL(sp_block_idx_to_mask_kernel, dim3(gx, hq), dim3(256), 0, (hipStream_t)stream, block_idx,
+                       idx_stride_h, k, nb, nbw, mask);
+    SP_LAUNCH_CHECK();
+  }
+  return SP_OK;
+}
+
+// CSR row pointers of id lists (count_kernel, shareprefill_attn.py:187-223: a histogram of id / nb, then its running
+// sum).  Duplicates count as often as they occur and the order of the ids does not matter, as in the reference.
+__global__ __launch_bounds__(256) void sp_block_idx_row_pointers_kernel(const int64_t* __restrict__ idx,
+                                                                        int64_t stride_h, int64_t k, int nb,
+                                                                        int32_t* __restrict__ row_ptr) {
+  __shared__ int32_t cnt[RS_MAX];
+  __shared__ int32_t part[256];
+  const int h = blockIdx.x;
+  const int64_t cells = (int64_t)nb * nb;
+  for (int r = threadIdx.x; r < nb; r += 256) cnt[r] = 0;
+  __syncthreads();
+  for (int64_t i = threadIdx.x; i < k; i += 256) {
+    const int64_t id = idx[(int64_t)h * stride_h + i];
+    if (id >= 0 && id < cells) atomicAdd(&cnt[(int)(id / nb)], 1);
+  }
+  __syncthreads();
+  // running sum: every thread owns a contiguous run of rows
+  const int per = (nb + 255) / 256;
+  const int r0 = threadIdx.x * per, r1 = (r0 + per < nb) ? r0 + per : nb;
+  int s = 0;
+  for (int r = r0; r < r1; ++r) s += cnt[r];
+  part[threadIdx.x] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int t = 0; t < 256; ++t) {
+      const int v = part[t];
+      part[t] = acc;
+      acc += v;
+    }
+  }
+  __syncthreads();
+  int32_t* out = row_ptr + (int64_t)h * (nb + 1);
+  int acc = part[threadIdx.x];
+  for (int r = r0; r < r1; ++r) {
+    acc += cnt[r];
+    out[r + 1] = acc;
+  }
+  if (threadIdx.x == 0) out[0] = 0;
+}
+
+extern "C" int sp_block_idx_row_pointers(const int64_t* block_idx, int64_t idx_stride_h, int64_t k, int32_t hq,
+                                         int32_t nb, int32_t* row_ptr, sp_stream_t stream) {
+  SP_REQUIRE(row_ptr && hq > 0 && nb > 0 && k >= 0 && (block_idx || k == 0), SP_ERR_INVALID_ARGUMENT,
+             "sp_block_idx_row_pointers: bad arguments");
+  SP_REQUIRE(nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_block_idx_row_pointers: nb=%d exceeds %d", nb, RS_MAX);
+  hipLaunchKernelGGL(sp_block_idx_row_pointers_kernel, dim3(hq), dim3(256), 0, (hipStream_t)stream, block_idx,
+                     idx_stride_h, k, nb, row_ptr);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}

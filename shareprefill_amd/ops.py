@@ -456,6 +456,41 @@ def mask_row_pointers(mask: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def _check_block_idx(idx: torch.Tensor) -> torch.Tensor:
+    if idx.dim() != 2 or not idx.is_cuda:
+        raise ValueError("block ids must be a GPU tensor [Hq, K]")
+    if idx.dtype != torch.int64:
+        idx = idx.to(torch.int64)
+    if idx.shape[1] > 0 and idx.stride(1) != 1:
+        idx = idx.contiguous()
+    return idx
+
+
+def block_idx_to_mask(idx: torch.Tensor, nb: int) -> torch.Tensor:
+    """Flat block ids [Hq, K] (row * nb + col, any order, padded with values outside the grid) -> bit mask int64
+    [Hq, nb, nbw]: the reference's block_idx form (shareprefill_attn.py:484-486) turned into the form the attention
+    entry point takes.  Ids above the diagonal are dropped."""
+    lib = _lib.load()
+    idx = _check_block_idx(idx)
+    hq, k = idx.shape
+    mask = torch.empty(hq, nb, (nb + 63) // 64, dtype=torch.int64, device=idx.device)
+    st = lib.sp_block_idx_to_mask(_ptr(idx) if k else None, idx.stride(0), k, hq, nb, _ptr(mask), _stream(idx.device))
+    _lib.check(st, "sp_block_idx_to_mask")
+    return mask
+
+
+def block_idx_row_pointers(idx: torch.Tensor, nb: int) -> torch.Tensor:
+    """Flat block ids [Hq, K] -> CSR row pointers int32 [Hq, nb+1] (count_kernel, shareprefill_attn.py:187-223)."""
+    lib = _lib.load()
+    idx = _check_block_idx(idx)
+    hq, k = idx.shape
+    out = torch.empty(hq, nb + 1, dtype=torch.int32, device=idx.device)
+    st = lib.sp_block_idx_row_pointers(_ptr(idx) if k else None, idx.stride(0), k, hq, nb, _ptr(out),
+                                       _stream(idx.device))
+    _lib.check(st, "sp_block_idx_row_pointers")
+    return out
+
+
 # ---- mask format helpers (host side, synchronising; for tests and inspection) ---------------------------
 def mask_to_bool(mask: torch.Tensor, nb: int) -> torch.Tensor:
     """bit mask int64 [..., nb, nbw] -> bool [..., nb, nb]."""

@@ -37,6 +37,80 @@ def _dense_causal_mask(hq: int, nb: int, device) -> torch.Tensor:
     return m
 
 
+def triton_column_count_cumsum(x: torch.Tensor, num_columns: int) -> torch.Tensor:
+    """The reference's helper of this name (shareprefill_attn.py:226-269), here a HIP kernel: x [B, H, K] flat block
+    ids of an num_columns x num_columns grid -> int32 [B, H, num_columns + 1], the running count of ids per grid row
+    (ids outside the grid are padding).  Its docstring example: ids [0, 5, 8, 9, 13, 14] in a 4 x 4 grid ->
+    [0, 1, 2, 4, 6]."""
+    if x.dim() != 3:
+        raise ValueError("x must be [batch_size, num_heads, activated_block_num]")
+    return torch.stack([ops.block_idx_row_pointers(x[b], num_columns) for b in range(x.shape[0])])
+
+
+def _pad_block_idx(block_idx, batch_size: int, num_heads: int, pad: int, device) -> torch.Tensor:
+    """list[B][H] of id tensors -> [B, H, K] padded with `pad` (shareprefill_attn.py:528-540)."""
+    if isinstance(block_idx, torch.Tensor):
+        assert block_idx.dim() == 3 and block_idx.shape[0] == batch_size and block_idx.shape[1] == num_heads
+        return block_idx
+    assert (isinstance(block_idx, list) and isinstance(block_idx[0], list)
+            and isinstance(block_idx[0][0], torch.Tensor))
+    assert len(block_idx) == batch_size and len(block_idx[0]) == num_heads
+    flat = [t.reshape(-1).to(device=device, dtype=torch.int64) for row in block_idx for t in row]
+    out = torch.nn.utils.rnn.pad_sequence(flat, batch_first=True, padding_value=pad)
+    return out.view(batch_size, num_heads, -1)
+
+
+def triton_block_wise_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, block_idx,
+                                        heads_need_blockwise_attn_mask: torch.Tensor, block_size: int,
+                                        grid_offset: int = 0, softmax_scale: Optional[float] = None,
+                                        gqa_interleave: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The reference's kernel wrapper under its own name and arguments (shareprefill_attn.py:474-620), served by the
+    HIP block-sparse attention kernel (nothing here is Triton).
+
+    q [B, N, Hq, D], k / v [B, N, Hkv, D] bf16 (any strides with a contiguous head_dim axis); block_idx the
+    activated blocks as flat ids row * nb + col, either list[B][Hq] of tensors or one padded tensor [B, Hq, K];
+    heads_need_blockwise_attn_mask bool [B, Hq]: the heads whose block-average attention map is wanted.
+    Returns (out [B, N, Hq, D] bf16, avg_attn fp32 [B, Hq, nb, nb], zero for the other heads).
+    gqa_interleave: query head h reads kv head h % Hkv instead of h // (Hq / Hkv) (shareprefill_attn.py:333-336).
+    Only grid_offset == 0, block_size 128 and head_dim 128 are built."""
+    batch_size, q_len, num_q_heads, head_dim = q.shape
+    _, k_len, num_kv_heads, _ = k.shape
+    assert q.dtype == torch.bfloat16
+    assert q_len == k_len
+    assert num_q_heads % num_kv_heads == 0
+    if grid_offset != 0:
+        raise NotImplementedError("grid_offset != 0 is not supported (the SharePrefill path never sets it)")
+    nb = -(-q_len // block_size)
+    dev = q.device
+    idx = _pad_block_idx(block_idx, batch_size, num_q_heads, nb * (nb + 1), dev)
+    need = heads_need_blockwise_attn_mask.to(device=dev).reshape(batch_size, num_q_heads) != 0
+    scale = 1.0 / math.sqrt(head_dim) if softmax_scale is None else float(softmax_scale)
+    g = num_q_heads // num_kv_heads
+    interleave = bool(gqa_interleave) and 1 < num_kv_heads < num_q_heads
+    # room for the block sums of every head that may want its map (at most 2 GiB of it; the rest recompute)
+    slab = _lib.load().sp_attn_pivot_scratch_bytes(q_len, block_size)
+    max_pivots = max(1, min(num_q_heads, (2 << 30) // slab))
+    outs, avgs = [], []
+    for b in range(batch_size):
+        qb, idx_b, need_b = q[b].transpose(0, 1), idx[b], need[b]
+        if interleave:
+            # the kernel gives query head h the kv head h // g: put the heads of kv head j (j, j + Hkv, ...) side by side
+            qb = qb.reshape(g, num_kv_heads, q_len, head_dim).transpose(0, 1).reshape(num_q_heads, q_len, head_dim)
+            idx_b = idx_b.reshape(g, num_kv_heads, -1).transpose(0, 1).reshape(num_q_heads, -1)
+            need_b = need_b.reshape(g, num_kv_heads).transpose(0, 1).reshape(num_q_heads)
+        mask = ops.block_idx_to_mask(idx_b, nb)
+        decision = torch.where(need_b, _lib.SP_DEC_DENSE, _lib.SP_DEC_VS).to(torch.int32)
+        avg = torch.zeros(num_q_heads, nb, nb, dtype=torch.float32, device=dev)
+        out = ops.block_sparse_attention(qb, k[b].transpose(0, 1), v[b].transpose(0, 1), mask, block_size, scale,
+                                         decision=decision, avg_attn=avg, max_pivots=max_pivots)
+        if interleave:
+            out = out.reshape(q_len, num_kv_heads, g, head_dim).transpose(1, 2).reshape(q_len, num_q_heads, head_dim)
+            avg = avg.reshape(num_kv_heads, g, nb, nb).transpose(0, 1).reshape(num_q_heads, nb, nb)
+        outs.append(out)
+        avgs.append(avg)
+    return torch.stack(outs), torch.stack(avgs)
+
+
 def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: torch.Tensor,
                                 value_states: torch.Tensor, *, gqa_interleave: bool = False
                                 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
