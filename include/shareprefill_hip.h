@@ -43,6 +43,10 @@ extern "C" {
 
 /* flags */
 #define SP_FLAG_LOGITS_BF16 1u /* round pooled / last-block logits to bf16 as the reference's bf16 einsum does */
+/* Bits 8..15 of flags: the head_dim, in units of 8, that the selection's 1/sqrt(head_dim) scale
+ * (attention_sharing.py:127, 197, 357) is formed from, for q / k whose head_dim axis has been zero-padded to a width
+ * the kernels are built for (the padding changes no dot product).  0 = the tensors' own d. */
+#define SP_FLAG_SCALE_DIM(head_dim) ((((uint32_t)(head_dim)) / 8u) << 8)
 
 /* tail handling of sp_pool_avg_bf16 */
 #define SP_POOL_TAIL_TRUE_LENGTH 0 /* divide the ragged last block by its length (attn/utils.py:171,187) */

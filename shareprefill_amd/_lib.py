@@ -15,6 +15,13 @@ LIB_PATH = os.environ.get("SHAREPREFILL_HIP_LIB") or os.path.join(os.path.dirnam
 
 SP_DEC_VS, SP_DEC_DENSE, SP_DEC_SHARE, SP_DEC_QA = 0, 1, 2, 3
 SP_FLAG_LOGITS_BF16 = 1
+
+
+def SP_FLAG_SCALE_DIM(head_dim: int) -> int:
+    """flags bits 8..15: the head_dim the selection's 1/sqrt(head_dim) is formed from when q / k are zero-padded."""
+    return (head_dim // 8) << 8
+
+
 SP_POOL_TAIL_TRUE_LENGTH, SP_POOL_TAIL_RESCALE = 0, 1
 SP_ATTN_V_REPACKED = 1
 SP_ATTN_PAIR_ROWS = 2

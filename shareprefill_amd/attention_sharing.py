@@ -177,8 +177,11 @@ class AttentionSharing:
     # ---- per-layer selection --------------------------------------------------------------------------
     def plan_layer(self, q: torch.Tensor, k: torch.Tensor, layer_idx: int, block_size: int, min_budget: int,
                    max_budget: int, pattern_threshold: float = 0.9, similarity_threshold: float = 0.5,
-                   fallback_threshold: float = 0.9, queryaware_threshold: float = 0.1) -> LayerPlan:
-        """q [Hq, N, D], k [Hkv, N, D] bf16 views; budgets in blocks.  Enqueues the whole selection."""
+                   fallback_threshold: float = 0.9, queryaware_threshold: float = 0.1,
+                   scale_dim: Optional[int] = None) -> LayerPlan:
+        """q [Hq, N, D], k [Hkv, N, D] bf16 views; budgets in blocks.  Enqueues the whole selection.
+        scale_dim: the model's head_dim when q / k have been zero-padded to D (the scores then scale by
+        1/sqrt(scale_dim), attention_sharing.py:127 of the reference)."""
         hq, n, d = q.shape
         nb = -(-n // block_size)
         maxb = min(max_budget, nb)
@@ -187,16 +190,17 @@ class AttentionSharing:
         state = self._ensure_state(nb, dev)
         hc = self._head_cluster_tensor(layer_idx, hq, dev)
 
-        vert_tok, slash_tok, vert_blk, slash_blk = ops.lastq_scores(q, k, block_size, self.flags)
+        flags = self.flags | (_lib.SP_FLAG_SCALE_DIM(scale_dim) if scale_dim and scale_dim != d else 0)
+        vert_tok, slash_tok, vert_blk, slash_blk = ops.lastq_scores(q, k, block_size, flags)
         nv, ns = ops.cover_budgets(vert_tok, slash_tok, block_size, pattern_threshold, minb, maxb)
         kbar = ops.pool_avg(k, block_size)
-        avg_qk, js_qa, use_qa = ops.queryaware_test(q, kbar, vert_blk, block_size, queryaware_threshold, self.flags)
+        avg_qk, js_qa, use_qa = ops.queryaware_test(q, kbar, vert_blk, block_size, queryaware_threshold, flags)
         decision, js_v, js_s, nv_f, ns_f = ops.share_decide(state, hc, layer_idx, vert_blk, slash_blk, use_qa, nv, ns,
                                                             minb, similarity_threshold, fallback_threshold)
         mask = ops.build_mask(state, hc, decision, vert_blk, slash_blk, nv_f, ns_f)
         # query-aware heads: pooled Q only for them (head_enable), selection skipped on device for the others
         qbar = ops.pool_avg(q, block_size, tail_mode=_lib.SP_POOL_TAIL_RESCALE, head_enable=use_qa)
-        qa_probs = ops.queryaware_select(qbar, kbar, decision, mask, pattern_threshold, self.flags,
+        qa_probs = ops.queryaware_select(qbar, kbar, decision, mask, pattern_threshold, flags,
                                          probs=self._qa_scratch(hq, nb, dev))
         plan = LayerPlan(layer_idx, nb, mask, decision, nv, ns, nv_f, ns_f)
         plan.max_pivots = self.max_pivots(layer_idx, hq)
@@ -246,9 +250,12 @@ class AttentionSharing:
                                       "supported; with K expanded to the query head count the flag changes nothing")
         if q.shape[0] != 1:
             raise ValueError("SharePrefill keeps per-cluster state for batch size 1 only")
+        model_dim = q.shape[-1]
+        if model_dim in (16, 32, 64):  # the kernels are built for head_dim 128: zero-padded q / k give the same scores
+            q, k = (torch.nn.functional.pad(t, (0, 128 - model_dim)) for t in (q, k))
         plan = self.plan_layer(q[0].transpose(0, 1), k[0].transpose(0, 1), layer_idx, block_size, min_budget,
                                max_budget, pattern_threshold, similarity_threshold, fallback_threshold,
-                               queryaware_threshold)
+                               queryaware_threshold, scale_dim=model_dim)
         if as_ids:
             return plan.block_idx(), plan.use_dense
         return plan.mask.unsqueeze(0), plan.use_dense

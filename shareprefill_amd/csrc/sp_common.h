@@ -33,6 +33,13 @@ void sp_set_error(const char* fmt, ...);
 
 __host__ __device__ static inline int64_t sp_ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// 1/sqrt(head_dim) of the selection: from the head_dim named in bits 8..15 of flags (units of 8) when the tensors'
+// head_dim axis is zero-padded, else from the tensors' own d
+static inline float sp_inv_sqrt_dim(uint32_t flags, int d) {
+  const int named = (int)((flags >> 8) & 0xffu) * 8;
+  return 1.0f / sqrtf((float)(named ? named : d));
+}
+
 // ---- kernels of one source file launched from another ----
 // pooled block probabilities of query-aware heads on the matrix core (sp_scores.hip), head_dim 128
 int sp_block_probs_mfma_launch(const void* qbar, const void* kbar, const int32_t* decision, int32_t hq, int32_t hkv,

@@ -694,7 +694,7 @@ int sp_block_probs_mfma_launch(const void* qbar, const void* kbar, const int32_t
                                int32_t nb, uint32_t flags, float* probs, hipStream_t stream) {
   hipLaunchKernelGGL(sp_block_probs_mfma_kernel, dim3((unsigned)sp_ceil_div(nb, LQ_ROWS), hq), dim3(BPM_THREADS), 0, stream,
                      (const sp_bf16*)qbar, (const sp_bf16*)kbar, decision, (int)hq, (int)hkv, (int)nb, flags,
-                     1.0f / sqrtf((float)LQ_D), probs);
+                     sp_inv_sqrt_dim(flags, LQ_D), probs);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
@@ -758,7 +758,7 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
   const int64_t nb = sp_ceil_div(n, bs);
   float2* partial = (float2*)workspace;
   float2* rowstat = partial + (size_t)hq * lq_chunks(n, hq) * LQ_ROWS;
-  const float inv_sqrt_d = 1.0f / sqrtf((float)d);
+  const float inv_sqrt_d = sp_inv_sqrt_dim(flags, d);
   const int group = hq / hkv;
   hipStream_t s = (hipStream_t)stream;
   const int wg_rows = hkv * lq_pairs(group);  // workgroups per key chunk: LQ_WG_HEADS heads of one kv group each

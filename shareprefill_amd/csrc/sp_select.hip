@@ -910,7 +910,7 @@ extern "C" int sp_queryaware_test_bf16(const void* q, const void* kbar, const fl
   SP_REQUIRE(lds <= 60000, SP_ERR_UNSUPPORTED, "sp_queryaware_test_bf16: nb=%d too large", nb);
   hipLaunchKernelGGL(sp_queryaware_test_kernel, dim3(hq), dim3(QA_THREADS), lds, (hipStream_t)stream,
                      (const sp_bf16*)q, (const sp_bf16*)kbar, vert_blk, n, hq, hkv, d, q_stride_n, q_stride_h, bs, nb,
-                     flags, 1.0f / sqrtf((float)d), queryaware_threshold, avg_qk, js_qa, use_qa);
+                     flags, sp_inv_sqrt_dim(flags, d), queryaware_threshold, avg_qk, js_qa, use_qa);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
@@ -1229,7 +1229,7 @@ extern "C" int sp_queryaware_select_bf16(const void* qbar, const void* kbar, con
   } else {  // one row per workgroup, fp32 dot products
     hipLaunchKernelGGL(sp_block_probs_kernel, dim3(nb, hq), dim3(BP_THREADS), lds, (hipStream_t)stream,
                        (const sp_bf16*)qbar, (const sp_bf16*)kbar, decision, hq, hkv, d, nb, flags,
-                       1.0f / sqrtf((float)d), probs);
+                       sp_inv_sqrt_dim(flags, d), probs);
     SP_LAUNCH_CHECK();
   }
   // score = pattern_threshold * nb evaluated in double, then taken to fp32 as a tensor comparison would

@@ -24,6 +24,19 @@ LOGGER = logging.getLogger(__name__)
 
 _dense_masks = {}
 
+KERNEL_HEAD_DIM = 128
+PADDED_HEAD_DIMS = (16, 32, 64)  # the reference's other head sizes (shareprefill_attn.py:503-508)
+
+
+def pad_head_dim(*tensors: torch.Tensor):
+    """The kernels are built for head_dim 128.  The reference's smaller head sizes run on them with the head_dim axis
+    zero-padded: no dot product changes (q.k gains exact zeros, the extra output channels are P.0 = 0 and are cut
+    off again), the softmax scale and the selection's 1/sqrt(head_dim) keep the model's head_dim.  Costs a copy of
+    q / k / v and 128 / head_dim times the arithmetic."""
+    d = tensors[0].shape[-1]
+    return tuple(torch.nn.functional.pad(t, (0, KERNEL_HEAD_DIM - d)) for t in tensors)
+
+
 
 def _dense_causal_mask(hq: int, nb: int, device) -> torch.Tensor:
     """Bit mask with every lower-triangular block set, cached per shape (short prompts ask for it in every layer)."""
@@ -72,19 +85,23 @@ def triton_block_wise_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: tor
     heads_need_blockwise_attn_mask bool [B, Hq]: the heads whose block-average attention map is wanted.
     Returns (out [B, N, Hq, D] bf16, avg_attn fp32 [B, Hq, nb, nb], zero for the other heads).
     gqa_interleave: query head h reads kv head h % Hkv instead of h // (Hq / Hkv) (shareprefill_attn.py:333-336).
-    Only grid_offset == 0, block_size 128 and head_dim 128 are built."""
-    batch_size, q_len, num_q_heads, head_dim = q.shape
+    Only grid_offset == 0 and block_size 128 are built; head_dim 16 / 32 / 64 run zero-padded to 128 (pad_head_dim)."""
+    batch_size, q_len, num_q_heads, model_dim = q.shape
     _, k_len, num_kv_heads, _ = k.shape
     assert q.dtype == torch.bfloat16
     assert q_len == k_len
     assert num_q_heads % num_kv_heads == 0
+    assert model_dim in PADDED_HEAD_DIMS + (KERNEL_HEAD_DIM,), "only support head_dim in {16, 32, 64, 128}"
+    if model_dim != KERNEL_HEAD_DIM:
+        q, k, v = pad_head_dim(q, k, v)
+    head_dim = q.shape[-1]
     if grid_offset != 0:
         raise NotImplementedError("grid_offset != 0 is not supported (the SharePrefill path never sets it)")
     nb = -(-q_len // block_size)
     dev = q.device
     idx = _pad_block_idx(block_idx, batch_size, num_q_heads, nb * (nb + 1), dev)
     need = heads_need_blockwise_attn_mask.to(device=dev).reshape(batch_size, num_q_heads) != 0
-    scale = 1.0 / math.sqrt(head_dim) if softmax_scale is None else float(softmax_scale)
+    scale = 1.0 / math.sqrt(model_dim) if softmax_scale is None else float(softmax_scale)
     g = num_q_heads // num_kv_heads
     interleave = bool(gqa_interleave) and 1 < num_kv_heads < num_q_heads
     # room for the block sums of every head that may want its map (at most 2 GiB of it; the rest recompute)
@@ -106,7 +123,7 @@ def triton_block_wise_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: tor
         if interleave:
             out = out.reshape(q_len, num_kv_heads, g, head_dim).transpose(1, 2).reshape(q_len, num_q_heads, head_dim)
             avg = avg.reshape(num_kv_heads, g, nb, nb).transpose(0, 1).reshape(num_q_heads, nb, nb)
-        outs.append(out)
+        outs.append(out[..., :model_dim])
         avgs.append(avg)
     return torch.stack(outs), torch.stack(avgs)
 
@@ -119,9 +136,12 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
     Prefill (N != 1): vertical/slash estimation, block selection and sharing, block-sparse attention,
     pivot update (shareprefill_attn.py:110-144).  Decode (N == 1): dense attention of the one query over
     all keys (:146-155)."""
-    bsz, num_heads, q_len, head_dim = query_states.shape
+    bsz, num_heads, q_len, model_dim = query_states.shape
     config = module.config
-    softmax_scale = getattr(module, "scaling", 1.0 / math.sqrt(head_dim))
+    softmax_scale = getattr(module, "scaling", 1.0 / math.sqrt(model_dim))
+    if model_dim in PADDED_HEAD_DIMS:
+        query_states, key_states, value_states = pad_head_dim(query_states, key_states, value_states)
+    head_dim = query_states.shape[-1]
     # gqa_interleave is accepted and changes nothing, as in the reference: there K and V are expanded to the query
     # head count before anything else, by repeat_interleave (True) or by expand + reshape (False) -- both give query
     # head h the kv head h // g (shareprefill_attn.py:33-40, 77-82) -- and everything after sees one kv head per query
@@ -137,7 +157,7 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
             raise AssertionError(f"SharePrefill attention expects bfloat16 q/k/v, got {query_states.dtype}")
         outs = [ops.decode_attention(query_states[b, :, 0], key_states[b], value_states[b], softmax_scale)
                 for b in range(bsz)]
-        return torch.stack(outs).unsqueeze(2), None
+        return torch.stack(outs).unsqueeze(2)[..., :model_dim], None
 
     if bsz != 1:
         raise ValueError("SharePrefill prefill keeps per-cluster state for batch size 1 only")
@@ -165,7 +185,7 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
         out = ops.block_sparse_attention(q, k, v, mask, block_size, softmax_scale, pair_rows=True)
         if q_len >= block_size:
             sharing.note_dense_layer(module.layer_idx, num_heads, nb)
-        return out.unsqueeze(0).transpose(1, 2), avg_attn
+        return out.unsqueeze(0).transpose(1, 2)[..., :model_dim], avg_attn
 
     # Room for the block sums of this layer's possible pivots (at most 16 GiB of it; pivots beyond that take the
     # recomputing pass).  How many heads can become pivots is known from the table alone.
@@ -176,11 +196,12 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
     ops.repack_v(v, block_size, ws[0])
     avg_attn.zero_()
     plan = sharing.plan_layer(q, k, module.layer_idx, block_size, minb, maxb, config.pattern_threshold,
-                              config.similarity_threshold, config.fallback_threshold, config.queryaware_threshold)
+                              config.similarity_threshold, config.fallback_threshold, config.queryaware_threshold,
+                              scale_dim=model_dim)
     out = ops.block_sparse_attention(q, k, v, plan.mask, block_size, softmax_scale, decision=plan.decision,
                                      avg_attn=avg_attn[0], max_pivots=max_pivots, workspace=ws)
     sharing.update_pivotal_attns(module.layer_idx, avg_attn, plan.decision, config.pattern_threshold)
-    return out.unsqueeze(0).transpose(1, 2), avg_attn
+    return out.unsqueeze(0).transpose(1, 2)[..., :model_dim], avg_attn
 
 
 def shareprefill_attention_forward(module, query_states: torch.Tensor, key_states: torch.Tensor,

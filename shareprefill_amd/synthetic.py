@@ -72,13 +72,14 @@ def planted_qkv(hq: int, hkv: int, n: int, d: int, seed: int, device="cpu", dtyp
     k[:SINK_TOKENS] *= SINK_SCALE
     fgen = torch.Generator(device="cpu")
     fgen.manual_seed(seed + 7919)
-    omega = (torch.rand(BAND_PAIRS, generator=fgen) * (math.pi / (BAND_WIDTH / 2))).to(device)
+    pairs = min(BAND_PAIRS, d // 2)  # head sizes below 32 channels carry as many band features as fit
+    omega = (torch.rand(BAND_PAIRS, generator=fgen)[:pairs] * (math.pi / (BAND_WIDTH / 2))).to(device)
     pos = torch.arange(n, device=device, dtype=torch.float32)
     ang = pos[:, None] * omega[None, :]
     feat = torch.cat([torch.cos(ang), torch.sin(ang)], dim=-1) * BAND_BETA  # [n, 2P]
     gain = 1.0 + q_head_gain * torch.arange(hq, device=device, dtype=torch.float32) / hq
-    q[:, :, : 2 * BAND_PAIRS] = feat[:, None, :] * gain[None, :, None]
-    k[:, :, : 2 * BAND_PAIRS] = feat[:, None, :]
+    q[:, :, : 2 * pairs] = feat[:, None, :] * gain[None, :, None]
+    k[:, :, : 2 * pairs] = feat[:, None, :]
     q, k, v = (t.to(dtype) for t in (q, k, v))
     return (q.unsqueeze(0).transpose(1, 2), k.unsqueeze(0).transpose(1, 2), v.unsqueeze(0).transpose(1, 2))
 

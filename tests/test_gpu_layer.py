@@ -39,7 +39,8 @@ class FakeAttention:
         self.attention_dropout = 0.0
 
 
-def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_free=True, with_forced=True, **thr):
+def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_free=True, with_forced=True, d=128,
+               **thr):
     from shareprefill_amd import AttentionSharing, shareprefill_attention_forward, ops
 
     # dense_short_prompts off: these tests compare the selection itself, also where the prompt is so short that every
@@ -49,7 +50,7 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_fre
     kw.update(thr)
     table = synthetic.random_cluster_table(hq, n_clusters, n_layers, seed)
     path = synthetic.write_cluster_table(table, str(tmp_path / "table.json"))
-    q, k, v = synthetic.planted_qkv(hq, hkv, n, 128, seed, q_head_gain=1.0)
+    q, k, v = synthetic.planted_qkv(hq, hkv, n, d, seed, q_head_gain=1.0)
     sharing = AttentionSharing(path)
     sharing.keep_debug = True
     cfg = types.SimpleNamespace(**kw)
@@ -59,10 +60,10 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_fre
     nb = -(-n // 128)
     results = []
     for layer in range(n_layers):
-        mod = FakeAttention(cfg, sharing, layer, 128, hq, hkv)
+        mod = FakeAttention(cfg, sharing, layer, d, hq, hkv)
         out, avg = shareprefill_attention_forward(mod, qg, kg, vg, None, scaling=mod.scaling)
         plan = sharing.plans[-1]
-        assert out.shape == (1, n, hq, 128) and out.is_contiguous() and out.dtype == torch.bfloat16
+        assert out.shape == (1, n, hq, d) and out.is_contiguous() and out.dtype == torch.bfloat16
         assert avg.shape == (1, hq, nb, nb) and avg.dtype == torch.float32
         gpu_mask = ops.mask_to_bool(plan.mask, nb).cpu().numpy()
         dec = plan.decision.cpu().numpy()
@@ -84,7 +85,7 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_fre
         results.append(dict(layer=layer, out=out.cpu(), avg=avg.cpu(), plan=plan, mask=gpu_mask, dec=dec,
                             forced=forced, free=free))
     return dict(q=q[0], k=k[0], v=v[0], table=table, sharing=sharing, oracle_forced=oracle_forced,
-                oracle_free=oracle_free, layers=results, nb=nb, kw=kw)
+                oracle_free=oracle_free, layers=results, nb=nb, kw=kw, d=d)
 
 
 def check_forced(run):
@@ -146,7 +147,7 @@ def check_outputs(run):
     q, k, v = run["q"], run["k"], run["v"]
     for L in run["layers"]:
         want = L["dec"] == O.DEC_DENSE
-        ref, avg_ref = O.masked_attention(q, k, v, L["mask"], 128, 128 ** -0.5, want_avg=want)
+        ref, avg_ref = O.masked_attention(q, k, v, L["mask"], 128, run["d"] ** -0.5, want_avg=want)
         out = L["out"][0].transpose(0, 1).float()
         assert (out - ref).abs().max().item() <= MAX_ABS
         assert ((out - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL
@@ -164,6 +165,21 @@ def test_layer_default_thresholds_small(gpu_device, tmp_path):
     check_outputs(run)
     d0 = run["layers"][0]["dec"]
     assert (d0 == O.DEC_DENSE).sum() == 2  # one pivot per shared cluster in the first layer
+
+
+@pytest.mark.parametrize("d,n", [(64, 2048), (32, 1100), (16, 1536)])
+def test_layer_small_head_dims(gpu_device, tmp_path, d, n):
+    """The reference's other head sizes (shareprefill_attn.py:503-508) run zero-padded to 128 on the same kernels: the
+    oracle works on the unpadded tensors with 1/sqrt(d), so every comparison below also checks that the padding
+    changes nothing (kbar is compared on the model's d channels, the padded ones must be zero)."""
+    run = run_layers(gpu_device, tmp_path, hq=8, hkv=2, n=n, seed=100 + d, n_clusters=2, d=d, min_budget=512)
+    for L in run["layers"]:
+        kbar = L["plan"].kbar
+        assert kbar.shape[-1] == 128 and float(kbar[..., d:].abs().max()) == 0.0
+        L["plan"].kbar = kbar[..., :d]
+    check_forced(run)
+    check_free(run)
+    check_outputs(run)
 
 
 def test_layer_c1_shape(gpu_device, tmp_path):

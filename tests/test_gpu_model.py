@@ -9,11 +9,12 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def small_llama(layers=2, hq=4, hkv=2):
+def small_llama(layers=2, hq=4, hkv=2, head_dim=128):
     from transformers import LlamaConfig, LlamaForCausalLM
 
-    cfg = LlamaConfig(hidden_size=hq * 128, intermediate_size=1024, num_hidden_layers=layers, num_attention_heads=hq,
-                      num_key_value_heads=hkv, head_dim=128, vocab_size=512, max_position_embeddings=8192)
+    cfg = LlamaConfig(hidden_size=hq * head_dim, intermediate_size=1024, num_hidden_layers=layers,
+                      num_attention_heads=hq, num_key_value_heads=hkv, head_dim=head_dim, vocab_size=512,
+                      max_position_embeddings=8192)
     torch.manual_seed(0)
     return LlamaForCausalLM(cfg)
 
@@ -73,6 +74,33 @@ def test_patched_model_sparse_prefill_and_generate(gpu_device, tmp_path):
     with torch.no_grad():
         gen = model.generate(ids[:, :300], max_new_tokens=4, do_sample=False)
     assert gen.shape == (1, 304)
+
+
+def test_patched_model_with_head_dim_64(gpu_device, tmp_path):
+    """Llama-3.2-1B-style heads (head_dim 64, one of the reference's head sizes, shareprefill_attn.py:503-508): prefill
+    with every block kept matches the eager model, a sparse prefill runs the selection, and decode works."""
+    from shareprefill_amd import SharePrefill
+
+    ids = torch.randint(0, 512, (1, 1536), generator=torch.Generator().manual_seed(6)).to(gpu_device)
+    ref_model = small_llama(head_dim=64).to(gpu_device, torch.bfloat16)
+    ref_model.config._attn_implementation = "eager"
+    with torch.no_grad():
+        ref = ref_model(ids).logits.float()
+    model = SharePrefill(sharing_lookup_path=table(tmp_path, 2, 4), min_budget=8192, dense_short_prompts=False)(
+        small_llama(head_dim=64).to(gpu_device, torch.bfloat16))
+    with torch.no_grad():
+        out = model(ids, use_cache=False).logits.float()
+    assert (out - ref).abs().max().item() < 0.15 and ((out - ref).abs().mean() / ref.abs().mean()).item() < 2e-2
+    assert sum(model.attention_sharing.decision_histogram().values()) == 8
+    sparse = SharePrefill(sharing_lookup_path=table(tmp_path, 2, 4), pattern_threshold=0.9, min_budget=256)(
+        small_llama(head_dim=64).to(gpu_device, torch.bfloat16))
+    with torch.no_grad():
+        logits = sparse(ids, use_cache=False, logits_to_keep=1).logits
+        gen = sparse.generate(ids[:, :300], max_new_tokens=3, do_sample=False)
+        want = ref_model.generate(ids[:, :300], max_new_tokens=3, do_sample=False)
+    assert torch.isfinite(logits).all() and gen.shape == (1, 303)
+    # 300 tokens lie within the minimum budget (dense prefill), decode is dense: the greedy tokens are the eager model's
+    assert torch.equal(gen, want)
 
 
 def test_patched_qwen2_model_prefill_and_generate(gpu_device, tmp_path):

@@ -223,3 +223,30 @@ def test_score_cover_topk_reference_signature(gpu_device):
     assert got.shape == (2, 3) and got.dtype == torch.int64
     want = [[O.cover_count(x[i, j].numpy(), 0.9) for j in range(3)] for i in range(2)]
     assert got.cpu().tolist() == want
+
+
+@pytest.mark.parametrize("d", [64, 32, 16])
+def test_block_wise_prefill_attention_small_head_dims(gpu_device, d):
+    """head_dim 16 / 32 / 64 (shareprefill_attn.py:503-508) run zero-padded on the head_dim-128 kernel; the default
+    softmax scale stays 1/sqrt(d)."""
+    from shareprefill.attn.shareprefill_attn import triton_block_wise_prefill_attention
+
+    hq, hkv, n = 4, 2, 900
+    g = torch.Generator().manual_seed(d)
+    mk = lambda h: torch.randn(1, n, h, d, generator=g).to(torch.bfloat16)
+    q, k, v = mk(hq), mk(hkv), mk(hkv)
+    nb = -(-n // 128)
+    mask = _random_mask(hq, nb, d, 0.5)
+    need = torch.tensor([[True, False, False, True]])
+    block_idx = [[t.to(gpu_device) for t in _ids_from_mask(mask)]]
+    out, avg = triton_block_wise_prefill_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), block_idx,
+                                                   need.to(gpu_device), 128)
+    assert out.shape == (1, n, hq, d)
+    qh, kh, vh = (t[0].transpose(0, 1) for t in (q, k, v))
+    ref, ref_avg = O.masked_attention(qh, kh, vh, mask, 128, 1.0 / math.sqrt(d), want_avg=need[0].numpy())
+    o = out[0].cpu().float().transpose(0, 1)
+    assert (o - ref).abs().max().item() <= 2e-2
+    assert ((o - ref).abs().mean() / ref.abs().mean()).item() <= 2.5e-3
+    for h in range(hq):
+        if need[0, h]:
+            assert (avg[0, h].cpu() - ref_avg[h]).abs().max().item() <= 2e-3
