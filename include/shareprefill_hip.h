@@ -71,6 +71,9 @@ typedef struct sp_cluster_state {
   uint64_t* pattern; /* [C][nb][nbw] pivot block pattern */
   uint64_t* accum;   /* [C][2]  scratch of sp_pivot_update (covered / total mass, fixed point); zero on entry, and
                         every completed call leaves it zero again: allocate it zero-filled */
+  float* avg_map;    /* [C][nb][nb] or NULL: the pivot's block-average attention map, kept by sp_pivot_update for
+                        AttentionSharing.get_pivotal_attn (attention_sharing.py:87-99); valid once has_pattern
+                        (since library version 2) */
 } sp_cluster_state;
 
 /* ---- library info ------------------------------------------------------------------------- */

@@ -35,6 +35,7 @@ class ClusterStateStruct(C.Structure):
         ("n_clusters", C.c_int32), ("nb", C.c_int32), ("nbw", C.c_int32), ("reserved", C.c_int32),
         ("info", C.c_void_p), ("ratio", C.c_void_p), ("vert", C.c_void_p), ("slash", C.c_void_p),
         ("cols", C.c_void_p), ("dists", C.c_void_p), ("pattern", C.c_void_p), ("accum", C.c_void_p),
+        ("avg_map", C.c_void_p),
     ]
 
 

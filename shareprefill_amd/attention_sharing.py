@@ -88,8 +88,10 @@ class AttentionSharing:
                 self._slot[cid] = len(self._slot)
         self._state: Optional[ops.ClusterState] = None
         self._head_cluster: Dict[Tuple[int, int, str], torch.Tensor] = {}
-        self._layer_avg: Dict[int, torch.Tensor] = {}
-        self.keep_pivot_maps = False  # keep every layer's avg_attn alive so get_pivotal_attn can return it
+        # keep every pivot's block-average map in the device state for get_pivotal_attn (fp32 [nb, nb] per shared
+        # cluster), unless all of them together exceed pivot_map_limit_bytes
+        self.keep_pivot_maps = True
+        self.pivot_map_limit_bytes = 4 << 30
         self.keep_debug = False   # keep every float intermediate of every layer (tests)
         self.keep_plans = False   # keep every layer's block mask (64 MiB per layer at 512K tokens) until the reset
         # one LayerPlan per layer planned since the last reset; unless keep_plans / keep_debug is set only the
@@ -129,15 +131,15 @@ class AttentionSharing:
         """Forget every pivot (attention_sharing.py:41-78); called at the start of each model forward."""
         if self._state is not None:
             self._state.reset()
-        self._layer_avg = {}
         self.plans = []
         self.dense_layers = 0
         self._dense_heads = 0
 
     def _ensure_state(self, nb: int, device) -> ops.ClusterState:
         st = self._state
-        if st is None or st.nb != nb or st.device != device:
-            st = ops.ClusterState(len(self._slot), nb, device)
+        keep = self.keep_pivot_maps and max(len(self._slot), 1) * nb * nb * 4 <= self.pivot_map_limit_bytes
+        if st is None or st.nb != nb or st.device != device or (st.avg_map is not None) != keep:
+            st = ops.ClusterState(len(self._slot), nb, device, keep_maps=keep)
             self._state = st
         return st
 
@@ -152,16 +154,17 @@ class AttentionSharing:
         return self._state.pattern[s]
 
     def get_pivotal_attn(self, layer_idx: int, b: int, h: int) -> Optional[torch.Tensor]:
-        """The pivot's [nb, nb] block-average map of the head's cluster (synchronises).  Only available with
-        keep_pivot_maps=True: which layer elected a pivot is known on the device only, so every layer's
-        avg_attn tensor has to be kept alive for this lookup."""
+        """The pivot's [nb, nb] block-average attention map of the head's cluster, or None while the cluster has no
+        pivot (attention_sharing.py:87-92; synchronises).  The maps live in the device state ([nb, nb] fp32 per
+        shared cluster, written by the pivot update); with keep_pivot_maps = False, or when they would exceed
+        pivot_map_limit_bytes, they are not kept and this returns None."""
         cid = self.find_cluster_id(layer_idx, h)
-        if self._state is None or cid not in self._slot:
+        if self._state is None or self._state.avg_map is None or cid not in self._slot:
             return None
-        info = self._state.info[self._slot[cid]].cpu()
-        if int(info[1]) == 0 or int(info[4]) not in self._layer_avg:
+        s = self._slot[cid]
+        if int(self._state.info[s, 1]) == 0:
             return None
-        return self._layer_avg[int(info[4])][b, int(info[0])]
+        return self._state.avg_map[s]
 
     def pivot_summary(self) -> Dict[str, dict]:
         """Host copy of the per-cluster state (synchronises); for logging and tests."""
@@ -274,8 +277,6 @@ class AttentionSharing:
         else:
             decision = use_dense.reshape(-1)
         ops.pivot_update(self._state, hc, decision, avg_attn[0], pattern_threshold)
-        if self.keep_pivot_maps:
-            self._layer_avg[layer_idx] = avg_attn
 
     def note_dense_layer(self, layer_idx: int, hq: int, nb: int) -> None:
         """A layer whose prompt is no longer than the minimum budget ran on the dense causal mask without any

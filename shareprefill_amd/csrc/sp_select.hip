@@ -1285,8 +1285,11 @@ __global__ __launch_bounds__(RS_THREADS) void sp_pivot_rows_kernel(sp_cluster_st
   const uint8_t* cols = st.cols + (int64_t)c * nb;
   const uint8_t* dists = st.dists + (int64_t)c * nb;
   unsigned long long cov = 0, tot = 0;
+  float* keep_row = st.avg_map ? st.avg_map + ((int64_t)c * nb + r) * nb : nullptr;
   for (int col = threadIdx.x; col < nb; col += RS_THREADS) {
-    const unsigned long long fx = sp_to_fixed(row[col]);
+    const float val = row[col];
+    if (keep_row) keep_row[col] = val;  // the pivot's map itself, for get_pivotal_attn
+    const unsigned long long fx = sp_to_fixed(val);
     tot += fx;
     if (col <= r) cov += fx * (unsigned long long)((cols[col] ? 1 : 0) + (dists[r - col] ? 1 : 0));
   }

@@ -160,9 +160,11 @@ def queryaware_test(q, kbar, vert_blk, block_size, queryaware_threshold, flags=_
 class ClusterState:
     """Device slabs of the cross-layer sharing state for C shared clusters (struct sp_cluster_state)."""
 
-    def __init__(self, n_clusters: int, nb: int, device):
+    def __init__(self, n_clusters: int, nb: int, device, keep_maps: bool = False):
         self.n_clusters, self.nb, self.nbw, self.device = n_clusters, nb, (nb + 63) // 64, device
         c = max(n_clusters, 1)
+        # the pivots' block-average maps themselves (fp32 [C, nb, nb]), only when asked for
+        self.avg_map = torch.empty(c, nb, nb, dtype=torch.float32, device=device) if keep_maps else None
         self.info = torch.zeros(c, 8, dtype=torch.int32, device=device)
         self.ratio = torch.zeros(c, dtype=torch.float64, device=device)
         self.vert = torch.zeros(c, nb, dtype=torch.float32, device=device)
@@ -173,7 +175,8 @@ class ClusterState:
         self.accum = torch.zeros(c, 2, dtype=torch.int64, device=device)
         self.struct = ClusterStateStruct(n_clusters, nb, self.nbw, 0, self.info.data_ptr(), self.ratio.data_ptr(),
                                          self.vert.data_ptr(), self.slash.data_ptr(), self.cols.data_ptr(),
-                                         self.dists.data_ptr(), self.pattern.data_ptr(), self.accum.data_ptr())
+                                         self.dists.data_ptr(), self.pattern.data_ptr(), self.accum.data_ptr(),
+                                         self.avg_map.data_ptr() if keep_maps else None)
         self.reset()
 
     def reset(self):

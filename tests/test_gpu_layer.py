@@ -113,6 +113,16 @@ def check_forced(run):
             pat = ops.mask_to_bool(state.pattern[sharing._slot[cid]], run["nb"]).cpu().numpy()
             assert np.array_equal(pat, st.pattern), f"cluster {cid}: pattern differs"
             assert got["vs_ratio"] == O.vs_ratio(st.avg, st.cols, st.dists), f"cluster {cid}: vs_ratio"
+            # the reference's getters (attention_sharing.py:80-92), asked through any member (layer, head) of the cluster
+            layer_m, head_m = run["table"]["clusters"][cid][-1]
+            kept = sharing.get_pivotal_attn(layer_m, 0, head_m)
+            assert kept is not None and np.array_equal(kept.cpu().numpy(), st.avg), f"cluster {cid}: pivot map"
+            kept_pat = sharing.get_pivotal_pattern(layer_m, 0, head_m)
+            assert np.array_equal(ops.mask_to_bool(kept_pat, run["nb"]).cpu().numpy(), st.pattern)
+        else:
+            layer_m, head_m = run["table"]["clusters"][cid][-1]
+            assert sharing.get_pivotal_attn(layer_m, 0, head_m) is None
+            assert sharing.get_pivotal_pattern(layer_m, 0, head_m) is None
 
 
 def check_free(run, expect_same_masks=True):

@@ -53,9 +53,15 @@ def test_library_identity_and_error_string():
 def test_cluster_state_struct_matches_header_layout():
     from shareprefill_amd._lib import ClusterStateStruct
 
-    assert ctypes.sizeof(ClusterStateStruct) == 16 + 8 * 8
+    assert ctypes.sizeof(ClusterStateStruct) == 16 + 9 * 8
     assert [f[0] for f in ClusterStateStruct._fields_][4:] == ["info", "ratio", "vert", "slash", "cols", "dists",
-                                                              "pattern", "accum"]
+                                                              "pattern", "accum", "avg_map"]
+    # the header declares the same members in the same order
+    header = open(os.path.join(os.path.dirname(__file__), "..", "include", "shareprefill_hip.h")).read()
+    body = header[header.index("typedef struct sp_cluster_state {"):header.index("} sp_cluster_state;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = re.findall(r"(\w+);", body)
+    assert names == [f[0] for f in ClusterStateStruct._fields_]
 
 
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):
