@@ -250,3 +250,29 @@ def test_block_wise_prefill_attention_small_head_dims(gpu_device, d):
     for h in range(hq):
         if need[0, h]:
             assert (avg[0, h].cpu() - ref_avg[h]).abs().max().item() <= 2e-3
+
+
+def test_ctypes_binding_for_the_reference(gpu_device):
+    """shareprefill_amd/reference_binding.py -- the self-contained ctypes stub a maintainer of the reference would add
+    -- gives the results of the package's own front ends."""
+    from shareprefill_amd import ops, reference_binding as rb
+
+    hq, hkv, n = 4, 2, 1100
+    g = torch.Generator().manual_seed(8)
+    mk = lambda h: torch.randn(1, n, h, 128, generator=g).to(torch.bfloat16).to(gpu_device)
+    q, k, v = mk(hq), mk(hkv), mk(hkv)
+    nb = -(-n // 128)
+    mask = _random_mask(hq, nb, 8, 0.5)
+    pooled = rb.hip_bnhd_pool(k, 128)
+    assert torch.equal(pooled[0], ops.pool_avg(k[0].transpose(0, 1), 128))
+    block_idx = [[t.to(gpu_device) for t in _ids_from_mask(mask)]]
+    use_dense = torch.tensor([[False, True, False, False]], device=gpu_device)
+    out, avg = rb.hip_block_wise_prefill_attention(q, k, v, block_idx, use_dense, 128, 128 ** -0.5)
+    mg = ops.bool_to_mask(torch.from_numpy(mask)).to(gpu_device)
+    assert torch.equal(rb.ids_to_mask(block_idx, nb), mg)
+    dec = use_dense[0].to(torch.int32)
+    avg_want = torch.zeros(hq, nb, nb, dtype=torch.float32, device=gpu_device)
+    want = ops.block_sparse_attention(q[0].transpose(0, 1), k[0].transpose(0, 1), v[0].transpose(0, 1), mg, 128,
+                                      128 ** -0.5, decision=dec, avg_attn=avg_want)
+    assert torch.equal(out[0], want)
+    assert torch.equal(avg[0], avg_want) and float(avg[0, 1].sum()) > 0
