@@ -106,7 +106,7 @@ def triton_block_wise_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: tor
     interleave = bool(gqa_interleave) and 1 < num_kv_heads < num_q_heads
     # room for the block sums of every head that may want its map (at most 2 GiB of it; the rest recompute)
     slab = _lib.load().sp_attn_pivot_scratch_bytes(q_len, block_size)
-    max_pivots = max(1, min(num_q_heads, (2 << 30) // slab))
+    max_pivots = min(num_q_heads, (2 << 30) // slab)
     outs, avgs = [], []
     for b in range(batch_size):
         qb, idx_b, need_b = q[b].transpose(0, 1), idx[b], need[b]
