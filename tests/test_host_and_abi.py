@@ -368,3 +368,55 @@ def test_plans_release_older_masks_unless_asked_to_keep_them(tmp_path):
     with pytest.raises(RuntimeError, match="keep_plans"):
         sharing.plans[0].block_idx()
     assert sharing.decision_histogram()["vertical_slash"] == 6  # the per-head decisions are kept
+
+
+# ---- host helpers of the reference-named kernel wrappers (no GPU needed) ----------------------------------------
+def test_pad_block_idx_list_and_tensor_forms():
+    """list[B][H] of id tensors -> [B, H, K] padded with the reference's value (shareprefill_attn.py:528-540)."""
+    from shareprefill_amd.shareprefill_attn import _pad_block_idx
+
+    nb = 4
+    pad = nb * (nb + 1)
+    lists = [[torch.tensor([0, 5, 8]), torch.tensor([0])], [torch.tensor([], dtype=torch.int64), torch.tensor([0, 15])]]
+    out = _pad_block_idx(lists, 2, 2, pad, torch.device("cpu"))
+    assert out.shape == (2, 2, 3) and out.dtype == torch.int64
+    assert out.tolist() == [[[0, 5, 8], [0, pad, pad]], [[pad, pad, pad], [0, 15, pad]]]
+    t = torch.zeros(2, 2, 5, dtype=torch.int64)
+    assert _pad_block_idx(t, 2, 2, pad, torch.device("cpu")) is t
+    with pytest.raises(AssertionError):
+        _pad_block_idx(lists, 1, 2, pad, torch.device("cpu"))
+
+
+def test_pad_head_dim_appends_zero_channels():
+    from shareprefill_amd.shareprefill_attn import KERNEL_HEAD_DIM, PADDED_HEAD_DIMS, pad_head_dim
+
+    assert KERNEL_HEAD_DIM == 128 and PADDED_HEAD_DIMS == (16, 32, 64)
+    x = torch.randn(1, 2, 5, 64).to(torch.bfloat16)
+    y = torch.randn(1, 1, 5, 64).to(torch.bfloat16)
+    px, py = pad_head_dim(x, y)
+    assert px.shape == (1, 2, 5, 128) and py.shape == (1, 1, 5, 128)
+    assert torch.equal(px[..., :64], x) and float(px[..., 64:].abs().max()) == 0.0
+    # a zero-padded dot product is the dot product (fp64 holds these sums of bf16 products exactly, in any order)
+    assert torch.equal((px.double() @ px.double().transpose(-1, -2)), (x.double() @ x.double().transpose(-1, -2)))
+
+
+def test_scale_dim_flag_field():
+    from shareprefill_amd import _lib
+
+    assert _lib.SP_FLAG_SCALE_DIM(64) == 8 << 8 and _lib.SP_FLAG_SCALE_DIM(16) == 2 << 8
+    assert (_lib.SP_FLAG_SCALE_DIM(32) & _lib.SP_FLAG_LOGITS_BF16) == 0
+    header = open(os.path.join(os.path.dirname(__file__), "..", "include", "shareprefill_hip.h")).read()
+    assert "#define SP_FLAG_SCALE_DIM(head_dim) ((((uint32_t)(head_dim)) / 8u) << 8)" in header
+
+
+def test_reference_import_paths_resolve_to_the_package():
+    import shareprefill
+    from shareprefill.attn import utils as ref_utils
+    from shareprefill.attn.shareprefill_attn import (shareprefill_attention_forward, triton_block_wise_prefill_attention,
+                                                     triton_column_count_cumsum)
+    import shareprefill_amd
+
+    assert shareprefill.SharePrefill is shareprefill_amd.SharePrefill
+    assert ref_utils.triton_bnhd_pool is shareprefill_amd.utils.triton_bnhd_pool
+    assert triton_block_wise_prefill_attention is shareprefill_amd.shareprefill_attn.triton_block_wise_prefill_attention
+    assert callable(triton_column_count_cumsum) and callable(shareprefill_attention_forward)
