@@ -5,7 +5,8 @@ query blocks against a plain fp32 torch computation of the same rows.
 Properties used: softmax mass conservation of the last-query scores (vertical and slash vectors each sum to 1),
 block sums equal to sums of tokens, budget bounds and monotonicity, masks lower-triangular with sink column and
 diagonal kept, row pointers equal to popcounts, the id-list view round-tripping to the mask, rows of a pivot's
-block-average map summing to 1, linearity of attention in V, run-to-run bit reproducibility.
+block-average map summing to 1, linearity of attention in V, run-to-run bit reproducibility, and the closed form of
+every output row for zero queries (the mean of the kept values).
 """
 
 import math
@@ -153,6 +154,47 @@ def test_attention_is_linear_in_v_and_reproducible(c3):
     assert ((lhs - rhs).abs() <= 2.0 ** -7 * scale_of + 5e-2).all()
     assert ((lhs - rhs).abs().mean() / rhs.abs().mean()).item() <= 1e-2
     assert torch.equal(o1, c3.outs[1][0])  # the layer call produced exactly this
+
+
+def test_zero_queries_give_the_mean_of_the_kept_values_in_every_row(c3):
+    """With q = 0 every logit is 0, every probability 1 (exact in bf16), so each output row is the plain mean of V over
+    the keys its mask keeps and causality allows -- a closed form for ALL 131072 x 32 rows of the full-size masks, from
+    block sums of V: out[i] = (sum of V over kept blocks left of the diagonal + sum of V[128 r .. i]) / their count.
+    What it pins at full size: which blocks every row visits (a skipped or doubled block changes the mean by 1 / count),
+    the causal edge inside the diagonal block, the row sums, the head -> kv head mapping and the output layout."""
+    from shareprefill_amd import ops
+
+    w, nb = c3.w, c3.nb
+    g = w.hq // w.hkv
+    vf = c3.v[0].float()                                   # [Hkv, N, D]
+    blk = vf.view(w.hkv, nb, 128, 128).sum(2)              # [Hkv, nb, D] block sums
+    within = vf.view(w.hkv, nb, 128, 128).cumsum(2)        # [Hkv, nb, 128, D] running sums inside each block
+    pos = torch.arange(1, 129, device=vf.device, dtype=torch.float32)
+    for layer in (0, 1):
+        mask = c3.plans[layer].mask
+        q0 = torch.zeros_like(c3.q[0])
+        out = ops.block_sparse_attention(q0, c3.k[0], c3.v[0], mask, 128, 128 ** -0.5).float()  # [N, Hq, D]
+        mb = ops.mask_to_bool(mask, nb)
+        assert bool(mb.diagonal(dim1=1, dim2=2).all())  # the closed form below counts the diagonal block of every row
+        left = torch.tril(mb, -1).float()                  # [Hq, nb, nb] kept blocks left of the diagonal
+        worst = 0.0
+        for h in range(w.hq):
+            kv = h // g
+            num = (left[h] @ blk[kv])[:, None, :] + within[kv]          # [nb, 128, D]
+            cnt = left[h].sum(1)[:, None] * 128.0 + pos[None, :]        # [nb, 128]
+            want = (num / cnt[:, :, None]).reshape(w.seq_len, 128)
+            got = out[:, h]
+            # the output's own bf16 rounding (2^-9 relative) and fp32 summation order over up to 131072 values
+            err = (got - want).abs()
+            assert (err <= 2.0 ** -8 * want.abs() + 2e-4).all(), f"layer {layer} head {h}: {err.max().item():.3e}"
+            worst = max(worst, (err.mean() / want.abs().mean()).item())
+            if h == 3:  # negative control: the closed form with one kept block of row 700 dropped must NOT pass
+                r = 700
+                c = int(torch.nonzero(left[h, r])[0])
+                num_bad = num[r] - blk[kv][c][None, :]
+                bad = num_bad / (cnt[r] - 128.0)[:, None]
+                assert not ((got[r * 128:(r + 1) * 128] - bad).abs() <= 2.0 ** -8 * bad.abs() + 2e-4).all()
+        assert worst <= 2.5e-3
 
 
 def test_maximum_supported_length_selection_bit_exact_and_rows_within_tolerance(gpu_device, tmp_path):
