@@ -197,6 +197,36 @@ def test_zero_queries_give_the_mean_of_the_kept_values_in_every_row(c3):
         assert worst <= 2.5e-3
 
 
+@pytest.mark.parametrize("max_pivots", [8, 0])
+def test_zero_queries_give_closed_form_block_average_maps(c3, max_pivots):
+    """Same inputs (q = 0, every probability 1): a dense pivot's block-average map is known in closed form for all
+    1024 x 1024 entries -- query i of block r spreads its mass evenly over its 128 r + i + 1 keys, so
+    avg[r, c < r] = mean_i 128 / (128 r + i + 1) and avg[r, r] = mean_i (i + 1) / (128 r + i + 1).
+    max_pivots = 8: the maps come from the block sums kept during the forward pass; 0: from the recomputing pass."""
+    from shareprefill_amd import ops
+
+    w, nb = c3.w, c3.nb
+    plan = c3.plans[0]
+    dense = torch.nonzero(plan.decision == 1).reshape(-1).tolist()
+    assert len(dense) == w.n_clusters
+    avg = torch.zeros(w.hq, nb, nb, dtype=torch.float32, device=c3.q.device)
+    ops.block_sparse_attention(torch.zeros_like(c3.q[0]), c3.k[0], c3.v[0], plan.mask, 128, 128 ** -0.5,
+                               decision=plan.decision, avg_attn=avg, max_pivots=max_pivots)
+    i = torch.arange(1, 129, device=avg.device, dtype=torch.float64)
+    r = torch.arange(nb, device=avg.device, dtype=torch.float64)
+    cnt = 128.0 * r[:, None] + i[None, :]                       # [nb, 128] keys seen by query i of block r
+    off = (128.0 / cnt).mean(1)                                 # value of every block left of the diagonal in row r
+    diag = (i[None, :] / cnt).mean(1)
+    want = torch.tril(off[:, None].expand(nb, nb), -1) + torch.diag(diag)
+    for h in range(w.hq):
+        if h in dense:
+            got = avg[h].double()
+            assert (got - want).abs().max().item() <= 2e-6, f"head {h}"
+            assert torch.allclose(got.sum(1), torch.ones(nb, dtype=torch.float64, device=avg.device), atol=1e-5)
+        else:
+            assert float(avg[h].abs().max()) == 0.0
+
+
 def test_maximum_supported_length_selection_bit_exact_and_rows_within_tolerance(gpu_device, tmp_path):
     """524288 tokens = 4096 key blocks, the longest sequence the block lists and rank tables are sized for (two query
     heads on one kv head, one shared cluster, two layers): budgets, decisions, masks and the pivot's pattern
