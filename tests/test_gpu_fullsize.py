@@ -69,6 +69,24 @@ def test_scores_conserve_mass_and_block_sums(c3):
         prev = (nv, ns)
 
 
+def test_scores_match_the_oracle_at_full_size_on_sampled_heads(c3):
+    """The oracle's last-query scores finish for single heads at 131072 tokens (a 128 x N product each): four heads
+    element by element, with fp32 logits (only exp / sum rounding left) and with the reference's bf16 logits."""
+    from oracle import shareprefill_oracle as O
+    from shareprefill_amd import ops
+
+    w = c3.w
+    g = w.hq // w.hkv
+    for flags, bf16_logits, rtol, atol in ((0, False, 5e-4, 1e-9), (1, True, 3e-2, 1e-7)):
+        vt, st, _, _ = ops.lastq_scores(c3.q[0], c3.k[0], 128, flags)
+        for h in (0, 5, 17, w.hq - 1):
+            qh = c3.q[0][h:h + 1].cpu()
+            kh = c3.k[0][h // g:h // g + 1].cpu()
+            vref, sref = O.lastq_scores(qh, kh, 128, logits_in_input_dtype=bf16_logits)
+            assert torch.allclose(vt[h].cpu(), vref[0], rtol=rtol, atol=atol), f"vertical, head {h}, bf16 {bf16_logits}"
+            assert torch.allclose(st[h].cpu(), sref[0], rtol=rtol, atol=atol), f"slash, head {h}, bf16 {bf16_logits}"
+
+
 def test_masks_are_causal_keep_sink_and_diagonal_and_match_their_views(c3):
     from shareprefill_amd import ops
 
@@ -326,3 +344,20 @@ def test_sharing_and_query_aware_heads_at_full_size_bit_exact(gpu_device, tmp_pa
             got = out[r * 128:(r + 1) * 128, h].float()
             assert (got - ref).abs().max().item() <= MAX_ABS
             assert ((got - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL
+    # the float stages of the query-aware path at this size against the oracle's own evaluation (they are cheap for
+    # the oracle: pooled rows, the last query block, one [nb, nb] product per head)
+    plan = L["plan"]
+    g = w.hq // w.hkv
+    kref = O.pool_avg(run["k"].transpose(0, 1).contiguous(), 128)                  # [nb, Hkv, D]
+    kb = plan.kbar.cpu().float()
+    assert (kb - kref.float()).abs().max().item() <= 2 ** -8 * max(1.0, kref.float().abs().max().item())
+    avg_ref = O.pooled_qk_probs(run["q"], kref, 128)
+    assert torch.allclose(plan.avg_qk.cpu(), avg_ref, rtol=2e-2, atol=1e-7)
+    js_ref = O.sqrt_js(avg_ref, plan.vert_blk.cpu())
+    assert torch.allclose(plan.js_qa.cpu(), js_ref, rtol=2e-2, atol=1e-4)
+    for h in [int(x) for x in np.nonzero(d1 == O.DEC_QA)[0][:2]]:
+        want = O.block_probs(O.pool_q_head(run["q"][h], 128), kref[:, h // g])
+        got = plan.qa_probs[h].cpu()
+        assert torch.allclose(got.sum(-1), torch.ones(nb), atol=1e-5) and bool((torch.triu(got, 1) == 0).all())
+        assert torch.allclose(got, want, rtol=6e-2, atol=1e-6), f"head {h}: block probabilities"
+        assert ((got - want).abs().sum() / want.abs().sum()).item() <= 5e-3
