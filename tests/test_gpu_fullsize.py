@@ -215,6 +215,26 @@ def test_zero_queries_give_the_mean_of_the_kept_values_in_every_row(c3):
         assert worst <= 2.5e-3
 
 
+def test_one_hot_values_make_every_output_row_a_distribution(c3):
+    """V[j] = unit vector of channel j mod 128 (exact in bf16): an output row is then the row's probability mass by
+    in-block key offset, so with the real queries and keys every one of the 131072 x 32 rows must be non-negative and
+    sum to 1 -- the normalisation (running maximum, rescales, row sums, the causal edge) checked on every row."""
+    from shareprefill_amd import ops
+
+    w = c3.w
+    eye = torch.eye(128, dtype=torch.bfloat16, device=c3.q.device)
+    v1 = eye.repeat(w.seq_len // 128, 1)[None].expand(w.hkv, -1, -1)           # [Hkv, N, D] view, nothing copied per head
+    for layer in (0, 1):
+        out = ops.block_sparse_attention(c3.q[0], c3.k[0], v1, c3.plans[layer].mask, 128, 128 ** -0.5).float()
+        assert bool((out >= 0).all())
+        rows = out.sum(-1)                                                      # [N, Hq]
+        # 128 bf16 roundings (unit roundoff 2^-8) of the non-negative parts of a sum that is 1: at most 2^-8 of it when
+        # every rounding goes the same way (rows with a handful of keys come close), far less on average
+        dev = (rows - 1.0).abs()
+        assert dev.max().item() <= 2.0 ** -8 + 1e-4, f"layer {layer}: {dev.max().item():.3e}"
+        assert dev.mean().item() <= 5e-4 and abs(rows.mean().item() - 1.0) <= 2e-5
+
+
 @pytest.mark.parametrize("max_pivots", [8, 0])
 def test_zero_queries_give_closed_form_block_average_maps(c3, max_pivots):
     """Same inputs (q = 0, every probability 1): a dense pivot's block-average map is known in closed form for all
