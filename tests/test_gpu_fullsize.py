@@ -22,14 +22,13 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, MEAN_REL = 2e-2, 2.5e-3  # see tests/test_gpu_attention.py for the mean-rel floor of a bf16 result
 
 
-@pytest.fixture(scope="module")
-def c3(gpu_device, tmp_path_factory):
+def _two_layers(gpu_device, tmp_path_factory, name):
     from shareprefill_amd import AttentionSharing, shareprefill_attention_forward
 
-    w = synthetic.WORKLOADS["C3"]
+    w = synthetic.WORKLOADS[name]
     q, k, v = synthetic.workload_inputs(w, device=gpu_device)
     table = synthetic.random_cluster_table(w.hq, w.n_clusters, 2, w.seed)
-    path = synthetic.write_cluster_table(table, str(tmp_path_factory.mktemp("c3") / "table.json"))
+    path = synthetic.write_cluster_table(table, str(tmp_path_factory.mktemp(name.lower()) / "table.json"))
     sharing = AttentionSharing(path)
     sharing.keep_plans = True  # both layers' masks are inspected below
     cfg = types.SimpleNamespace(block_size=128, min_budget=w.min_budget, max_budget=None,
@@ -44,6 +43,23 @@ def c3(gpu_device, tmp_path_factory):
         plans.append(sharing.plans[-1])
     torch.cuda.synchronize()
     return types.SimpleNamespace(w=w, q=q, k=k, v=v, outs=outs, plans=plans, avgs=avgs, nb=w.seq_len // 128)
+
+
+@pytest.fixture(scope="module")
+def c3(gpu_device, tmp_path_factory):
+    return _two_layers(gpu_device, tmp_path_factory, "C3")
+
+
+@pytest.fixture(scope="module")
+def c5(gpu_device, tmp_path_factory):
+    """Qwen2.5-7B head shapes at 262144 tokens: 28 query heads on 4 kv heads (groups of 7: an odd head per group is
+    paired by rows, and head pairs never cross kv heads), nb 2048."""
+    return _two_layers(gpu_device, tmp_path_factory, "C5")
+
+
+@pytest.fixture
+def full_size_case(request):
+    return request.getfixturevalue(request.param)
 
 
 def test_scores_conserve_mass_and_block_sums(c3):
@@ -174,14 +190,17 @@ def test_attention_is_linear_in_v_and_reproducible(c3):
     assert torch.equal(o1, c3.outs[1][0])  # the layer call produced exactly this
 
 
-def test_zero_queries_give_the_mean_of_the_kept_values_in_every_row(c3):
+@pytest.mark.parametrize("full_size_case", ["c3", "c5"], indirect=True)
+def test_zero_queries_give_the_mean_of_the_kept_values_in_every_row(full_size_case):
     """With q = 0 every logit is 0, every probability 1 (exact in bf16), so each output row is the plain mean of V over
-    the keys its mask keeps and causality allows -- a closed form for ALL 131072 x 32 rows of the full-size masks, from
+    the keys its mask keeps and causality allows -- a closed form for ALL rows of the full-size masks (131072 x 32 at
+    C3, 262144 x 28 at C5), from
     block sums of V: out[i] = (sum of V over kept blocks left of the diagonal + sum of V[128 r .. i]) / their count.
     What it pins at full size: which blocks every row visits (a skipped or doubled block changes the mean by 1 / count),
     the causal edge inside the diagonal block, the row sums, the head -> kv head mapping and the output layout."""
     from shareprefill_amd import ops
 
+    c3 = full_size_case  # (either full-size fixture)
     w, nb = c3.w, c3.nb
     g = w.hq // w.hkv
     vf = c3.v[0].float()                                   # [Hkv, N, D]
@@ -202,7 +221,7 @@ def test_zero_queries_give_the_mean_of_the_kept_values_in_every_row(c3):
             cnt = left[h].sum(1)[:, None] * 128.0 + pos[None, :]        # [nb, 128]
             want = (num / cnt[:, :, None]).reshape(w.seq_len, 128)
             got = out[:, h]
-            # the output's own bf16 rounding (2^-9 relative) and fp32 summation order over up to 131072 values
+            # the output's own bf16 rounding (unit roundoff 2^-8) and fp32 summation order over up to 262144 values
             err = (got - want).abs()
             assert (err <= 2.0 ** -8 * want.abs() + 2e-4).all(), f"layer {layer} head {h}: {err.max().item():.3e}"
             worst = max(worst, (err.mean() / want.abs().mean()).item())
@@ -215,12 +234,14 @@ def test_zero_queries_give_the_mean_of_the_kept_values_in_every_row(c3):
         assert worst <= 2.5e-3
 
 
-def test_one_hot_values_make_every_output_row_a_distribution(c3):
+@pytest.mark.parametrize("full_size_case", ["c3", "c5"], indirect=True)
+def test_one_hot_values_make_every_output_row_a_distribution(full_size_case):
     """V[j] = unit vector of channel j mod 128 (exact in bf16): an output row is then the row's probability mass by
-    in-block key offset, so with the real queries and keys every one of the 131072 x 32 rows must be non-negative and
+    in-block key offset, so with the real queries and keys every one of the rows (all heads, all tokens) must be non-negative and
     sum to 1 -- the normalisation (running maximum, rescales, row sums, the causal edge) checked on every row."""
     from shareprefill_amd import ops
 
+    c3 = full_size_case  # (either full-size fixture)
     w = c3.w
     eye = torch.eye(128, dtype=torch.bfloat16, device=c3.q.device)
     v1 = eye.repeat(w.seq_len // 128, 1)[None].expand(w.hkv, -1, -1)           # [Hkv, N, D] view, nothing copied per head
