@@ -103,6 +103,34 @@ def test_scores_match_the_oracle_at_full_size_on_sampled_heads(c3):
             assert torch.allclose(st[h].cpu(), sref[0], rtol=rtol, atol=atol), f"slash, head {h}, bf16 {bf16_logits}"
 
 
+@pytest.mark.parametrize("full_size_case", ["c3", "c5"], indirect=True)
+def test_decode_and_pooling_at_full_size(full_size_case):
+    """The two HBM-bound steps at the benchmark lengths against plain fp32 evaluations on the device: the decode step
+    of the last token over the whole cache (131072 / 262144 keys) with the real queries, with zero queries (the mean
+    of V) and with one-hot values (a distribution), and the block means of K."""
+    from shareprefill_amd import ops
+
+    c = full_size_case
+    w, nb = c.w, c.nb
+    g = w.hq // w.hkv
+    k, v = c.k[0], c.v[0]                                   # [Hkv, N, D]
+    scale = 128 ** -0.5
+    for q1 in (c.q[0][:, -1], torch.zeros(w.hq, 128, dtype=torch.bfloat16, device=k.device)):
+        out = ops.decode_attention(q1.contiguous(), k, v, scale).float()
+        logits = torch.einsum("hgd,hnd->hgn", q1.float().view(w.hkv, g, 128), k.float()) * scale
+        ref = torch.einsum("hgn,hnd->hgd", torch.softmax(logits, -1), v.float()).reshape(w.hq, 128)
+        assert (out - ref).abs().max().item() <= MAX_ABS
+        assert ((out - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL
+    eye = torch.eye(128, dtype=torch.bfloat16, device=k.device)
+    v1 = eye.repeat(w.seq_len // 128, 1)[None].expand(w.hkv, -1, -1)
+    rows = ops.decode_attention(c.q[0][:, -1].contiguous(), k, v1, scale).float()
+    assert bool((rows >= 0).all()) and (rows.sum(-1) - 1.0).abs().max().item() <= 2.0 ** -8 + 1e-4
+    kbar = ops.pool_avg(k, 128).float()                     # [nb, Hkv, D]
+    want = k.float().view(w.hkv, nb, 128, 128).mean(2).transpose(0, 1)
+    assert (kbar - want).abs().max().item() <= 2.0 ** -8 * max(1.0, want.abs().max().item())
+    assert ((kbar - want).abs() <= 2.0 ** -8 * want.abs() + 1e-6).all()
+
+
 def test_masks_are_causal_keep_sink_and_diagonal_and_match_their_views(c3):
     from shareprefill_amd import ops
 
