@@ -186,6 +186,9 @@ int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec,
 #define SP_ATTN_V_REPACKED 1u
 #define SP_ATTN_PAIR_ROWS 2u /* skip the per-call analysis of how to pair query blocks into work items and pair rows
                                 2p, 2p+1 of every head: what a dense mask wants; the result never depends on it */
+#define SP_ATTN_HALF_CHANNELS 4u /* q, k and v are zero beyond channel 64 (a head_dim of 16 / 32 / 64 zero-padded to the
+                                    kernel's 128, shareprefill_attn.py:503-508): the products skip those channels and
+                                    channels 64..127 of out are NOT written */
 size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs);
 /* Optional extra workspace per pivot head (decision == SP_DEC_DENSE with avg_attn requested): with
  * sp_attn_workspace_bytes rounded up to 256 bytes + p * sp_attn_pivot_scratch_bytes(n, bs) bytes of workspace, the

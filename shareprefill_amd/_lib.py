@@ -25,6 +25,7 @@ def SP_FLAG_SCALE_DIM(head_dim: int) -> int:
 SP_POOL_TAIL_TRUE_LENGTH, SP_POOL_TAIL_RESCALE = 0, 1
 SP_ATTN_V_REPACKED = 1
 SP_ATTN_PAIR_ROWS = 2
+SP_ATTN_HALF_CHANNELS = 4
 SP_DECODE_STATIC_SCRATCH_BYTES = 8 << 20
 
 

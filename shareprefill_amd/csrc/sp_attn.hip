@@ -403,14 +403,18 @@ __device__ __forceinline__ void at_prefetch_qk(const AtAddr& ad, bf16x8 (&pre)[2
 
 // PRE: operands 0 and 1 of the stage are already in flight in `pre` (at_prefetch_qk<KQ>, and nothing else has been
 // read from LDS since).  NEXT >= 0: the stage ends by fetching the first two operands of the next one, quarter NEXT.
-template <bool DO_QK, bool DO_PV, int KQ, int VB, int KT, bool PRE, int NEXT>
+// HALF: q, k and v are zero beyond channel 64 (a head_dim of at most 64 padded to the tiles' 128): the S product takes the
+// first two of its four channel steps and O the first four of its eight channel tiles -- half the operand slots.
+template <bool DO_QK, bool DO_PV, int KQ, int VB, int KT, bool PRE, int NEXT, bool HALF>
 __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2],
                                          const floatx4 (&s_in)[2][2], const bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
                                          floatx4 (&o)[9][2], float sc, const float (&neg_m)[2], uint32_t (&det)[2],
                                          const bf16x8& ones, bf16x8 (&pre)[2]) {
   static_assert(!PRE || DO_QK, "only stages that start with the S product take prefetched operands");
-  constexpr int NP = (DO_QK ? 8 : 0) + (DO_PV ? 8 : 0);  // operand slots; each holds one MFMA per query tile
-  static_assert(NP == 8 || NP == 16, "a fused stage has 8 or 16 operand slots");
+  constexpr int QS = DO_QK ? (HALF ? 4 : 8) : 0;  // operand slots of the S product: (channel step, key tile) pairs
+  constexpr int PS = DO_PV ? (HALF ? 4 : 8) : 0;  // operand slots of the P.V product: channel tiles
+  constexpr int NP = QS + PS;                     // each slot holds one MFMA per query tile
+  static_assert(NP == 4 || NP == 8 || NP == 16, "a fused stage has 4, 8 or 16 operand slots");
   constexpr int EPS = 16 / NP;  // softmax elements handled per operand slot
   constexpr int AHEAD = 2;      // LDS operands are fetched this many slots before their MFMAs
   bf16x8 opnd[NP];
@@ -418,8 +422,8 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
   uint32_t pk[8];
   auto fetch = [&](auto kc) {
     constexpr int k = decltype(kc)::value;
-    constexpr bool qk = DO_QK && k < 8;
-    constexpr int i = k & 7;
+    constexpr bool qk = k < QS;
+    constexpr int i = qk ? k : k - QS;
     if constexpr (qk)  // slot i: channel step i / 2, key tile i % 2
       opnd[k] = at_lds128_async<(KQ >> 1) * AT_KBUF_BYTES + ((KQ & 1) * 32 + (i & 1) * 16) * 256>(ad.ka[i >> 1]);
     else  // slot i: channel tile i
@@ -435,8 +439,8 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
   AT_PIN();
   at_static_for<0, NP>([&](auto kc) {
     constexpr int k = decltype(kc)::value;
-    constexpr bool qk = DO_QK && k < 8;
-    constexpr int i = k & 7;
+    constexpr bool qk = k < QS;
+    constexpr int i = qk ? k : k - QS;
     constexpr int in_flight_after = (NP - 1 - k) < (AHEAD - 1) ? (NP - 1 - k) : (AHEAD - 1);
     AT_WAIT_LGKM(in_flight_after);  // operand k has landed
     AT_PIN();
@@ -514,15 +518,16 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
 }
 
 // MFMA-only stages (no vector work to hide): first S of a run, last P.V of a run
-template <int KH>
+template <int KH, bool HALF>
 __device__ __forceinline__ void at_qk_only(const char* kb, int koff, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2]) {
+  constexpr int QS = HALF ? 4 : 8;
   bf16x8 a[8];  // slot i: channel step i / 2, key tile i % 2
 #pragma unroll
   for (int i = 0; i < 4; ++i) a[i] = at_lds128(kb + (koff ^ ((i >> 1) << 6)) + (KH * 32 + (i & 1) * 16) * 256);
   AT_PIN();
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    if (i + 4 < 8) a[i + 4] = at_lds128(kb + (koff ^ (((i + 4) >> 1) << 6)) + (KH * 32 + (i & 1) * 16) * 256);
+  for (int i = 0; i < QS; ++i) {
+    if (i + 4 < QS) a[i + 4] = at_lds128(kb + (koff ^ (((i + 4) >> 1) << 6)) + (KH * 32 + (i & 1) * 16) * 256);
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
       if ((i >> 1) == 0)
@@ -535,16 +540,17 @@ __device__ __forceinline__ void at_qk_only(const char* kb, int koff, const bf16x
   at_settle_s(s_out);
 }
 
-template <int KT>
+template <int KT, bool HALF>
 __device__ __forceinline__ void at_pv_only(const char* vb, int voff, const bf16x8 (&p)[2], floatx4 (&o)[9][2],
                                            const bf16x8& ones) {
+  constexpr int PS = HALF ? 4 : 8;
   bf16x8 a[8];  // slot i: channel tile i
 #pragma unroll
   for (int i = 0; i < 4; ++i) a[i] = at_lds128(vb + (voff ^ (KT << 6)) + i * 16 * 128);
   AT_PIN();
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    if (i + 4 < 8) a[i + 4] = at_lds128(vb + (voff ^ (KT << 6)) + (i + 4) * 16 * 128);
+  for (int i = 0; i < PS; ++i) {
+    if (i + 4 < PS) a[i + 4] = at_lds128(vb + (voff ^ (KT << 6)) + (i + 4) * 16 * 128);
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) at_mfma_acc(o[i][qt], a[i], p[qt]);
     AT_PIN();
@@ -604,10 +610,12 @@ __device__ __forceinline__ float at_groupmax(float mx) {
 // s_prev = S(j-1) (causal predicate applied), p = P(j-1), det = OR of its packed words.  On return p is safe to use.
 // PIVOT: l_mark (the row sums at the start of the current key block, see the block sums of pivot heads in the
 // kernel) follows every rescale.
-template <bool PIVOT>
+// MODE: bit 0 = PIVOT, bit 1 = HALF (see at_fused)
+template <int MODE>
 __device__ __forceinline__ void at_commit(const floatx4 (&s_prev)[2][2], bf16x8 (&p)[2], uint32_t (&det)[2],
                                           floatx4 (&o)[9][2], float scale_log2, float (&m_run)[2],
                                           float (&l_mark)[2]) {
+  constexpr bool PIVOT = (MODE & 1) != 0, HALF = (MODE & 2) != 0;
   if (__builtin_amdgcn_ballot_w64(((det[0] | det[1]) & AT_P_TOO_LARGE) != 0u) != 0ull) {
     float mx[2];  // (S(j-1) is a whole stage old: no wait states needed before reading it)
     at_lanemax(s_prev, mx);
@@ -621,9 +629,11 @@ __device__ __forceinline__ void at_commit(const floatx4 (&s_prev)[2][2], bf16x8 
     for (int qt = 0; qt < 2; ++qt) {
       if constexpr (PIVOT) l_mark[qt] *= alpha[qt];
 #pragma unroll
-      for (int dt = 0; dt < 9; ++dt)
+      for (int dt = 0; dt < 9; ++dt) {
+        if (HALF && dt >= 4 && dt < 8) continue;  // channel tiles nobody accumulates into
 #pragma unroll
         for (int j = 0; j < 4; ++j) o[dt][qt][j] *= alpha[qt];
+      }
       float e[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j)
@@ -644,24 +654,25 @@ __device__ __forceinline__ void at_commit(const floatx4 (&s_prev)[2][2], bf16x8 
 // One pipeline step.  s_in = S(j) (complete), p_prev = P(j-1) not yet applied to O (HAVE_PREV), det the OR of its
 // packed words; s_out still holds S(j-1) on entry and S(j+1) on return, p_out = P(j) with its OR in det.
 // The fused stage exists once per step: O never lives in two register sets that would have to be merged.
-template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT, bool PIVOT, bool PRE = false, int NEXT = -1>
+template <bool DO_QK, bool HAVE_PREV, int KQ, int VB, int KT, int MODE, bool PRE = false, int NEXT = -1>
 __device__ __forceinline__ void at_step(const AtAddr& ad, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2],
                                         floatx4 (&s_in)[2][2], bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
                                         floatx4 (&o)[9][2], float scale_log2, float (&m_run)[2], uint32_t (&det)[2],
                                         const bf16x8& ones, bool diag, int key_base, int t, float (&l_mark)[2],
                                         bf16x8 (&pre)[2]) {
-  if (HAVE_PREV) at_commit<PIVOT>(s_out, p_prev, det, o, scale_log2, m_run, l_mark);
+  if (HAVE_PREV) at_commit<MODE>(s_out, p_prev, det, o, scale_log2, m_run, l_mark);
   if (diag) at_causal(s_in, key_base, t);
   const float neg_m[2] = {-m_run[0], -m_run[1]};
-  at_fused<DO_QK, HAVE_PREV, KQ, VB, KT, PRE, NEXT>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2, neg_m, det, ones,
-                                                    pre);
+  at_fused<DO_QK, HAVE_PREV, KQ, VB, KT, PRE, NEXT, (MODE & 2) != 0>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2,
+                                                                      neg_m, det, ones, pre);
 }
 
 // PIVOT = false: every head except the pivots that have a slot in the scheduler area's table (when skip_slotted).
 // PIVOT = true: only those pivots; besides the output it leaves, per (query, key block), the softmax mass of the
 // block relative to the running max at that time as u = log2(sum) + max, from which at_avg_from_block_sums (sp_attn_avg_kernel) makes
 // the block-average map without recomputing any logit.  pivot_u: fp32 [slot][r*(r+1)/2 + c][128 queries].
-template <bool PIVOT>
+// HALF: q, k and v are zero beyond channel 64 (see at_fused); channels 64..127 of out are then not written.
+template <bool PIVOT, bool HALF>
 __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ vt,
     const uint64_t* __restrict__ mask, const int32_t* __restrict__ decision, sp_bf16* __restrict__ out,
@@ -670,6 +681,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     float* __restrict__ pivot_u) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // K ring (4 x 16 KiB) | V^T ring (4 x 16 KiB)
   __shared__ int s_queue, s_ticket;
+  constexpr int MODE = (PIVOT ? 1 : 0) | (HALF ? 2 : 0);
   if (PIVOT && sched[AT_NPIV_SLOT] == 0) return;  // no pivot in this layer
   const uint8_t* const slots = reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE);
   const uint8_t* const pair_table = reinterpret_cast<const uint8_t*>(sched + AT_PAIR_TABLE);
@@ -783,7 +795,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         if (qrow > n - 1) qrow = n - 1;
         const sp_bf16* src = q + (int64_t)h * sq_h + qrow * sq_n + 8 * g;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
+        for (int ks = 0; ks < (HALF ? 2 : 4); ++ks)
           qb[qt][ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 32 * ks));
       }
     }
@@ -920,15 +932,15 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       bf16x8 pre[2];               // the next stage's first two LDS operands, in flight (at_prefetch_qk)
       // ---- start of a run: S of the first half-tile, nothing to overlap with yet ----
       feed(0);
-      at_qk_only<0>(kb, koff, qb, sa);
+      at_qk_only<0, HALF>(kb, koff, qb, sa);
       feed(1);
-      at_step<true, false, 1, 0, 0, PIVOT, false, 2>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
+      at_step<true, false, 1, 0, 0, MODE, false, 2>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
                                                      c_cur == r, 0, tq, l_mark, pre);
       feed(2);
-      at_step<true, true, 2, 1, 0, PIVOT, true, 3>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
+      at_step<true, true, 2, 1, 0, MODE, true, 3>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                                    c_cur == r, 32, tq, l_mark, pre);
       feed(3);
-      at_step<true, true, 3, 1, 1, PIVOT, true, -1>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
+      at_step<true, true, 3, 1, 1, MODE, true, -1>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
                                                     c_cur == r, AT_SUB, tq, l_mark, pre);
       int c_prev = c_cur;
       step_walk();
@@ -941,19 +953,19 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         at_prefetch_qk<0>(ad, pre);  // (the block's first operands, while the loads and the commit test are set up)
         if (grp) __builtin_amdgcn_s_setprio(1);
         // S(previous block, keys 96..127) -> P;  S(keys 0..31) on the matrix core;  O += V^T(2b-1, keys 0..31) . P
-        at_step<true, true, 0, 0, 0, PIVOT, true, 1>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
+        at_step<true, true, 0, 0, 0, MODE, true, 1>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                                      c_prev == r, AT_SUB + 32, tq, l_mark, pre);
         feed(0);
-        at_step<true, true, 1, 0, 1, PIVOT, true, 2>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
+        at_step<true, true, 1, 0, 1, MODE, true, 2>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
                                                      c_cur == r, 0, tq, l_mark, pre);
         emit(c_prev);  // the previous block's last half-tile went into O (and the sums) in this step
         if (grp) __builtin_amdgcn_s_setprio(0);
         feed(1);
         feed(2);
-        at_step<true, true, 2, 1, 0, PIVOT, true, 3>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
+        at_step<true, true, 2, 1, 0, MODE, true, 3>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                                      c_cur == r, 32, tq, l_mark, pre);
         feed(3);
-        at_step<true, true, 3, 1, 1, PIVOT, true, -1>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
+        at_step<true, true, 3, 1, 1, MODE, true, -1>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
                                                       c_cur == r, AT_SUB, tq, l_mark, pre);
         c_prev = c_cur;
         step_walk();
@@ -970,10 +982,10 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         vb = vring + ((2 * b + 3) & 3) * AT_VBUF_BYTES;
         at_block_addr(ad, kb, vb, vb, koff, voff);
       }
-      at_step<false, true, 0, 0, 0, PIVOT>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
+      at_step<false, true, 0, 0, 0, MODE>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
                                            c_prev == r, AT_SUB + 32, tq, l_mark, pre);
-      at_commit<PIVOT>(sb, pb, det, o, scale_log2, m_run, l_mark);
-      at_pv_only<1>(vb, voff, pb, o, ones);
+      at_commit<MODE>(sb, pb, det, o, scale_log2, m_run, l_mark);
+      at_pv_only<1, HALF>(vb, voff, pb, o, ones);
       emit(c_prev);
     }
     if (!finished) {
@@ -1006,7 +1018,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
           const float inv_l = 1.0f / l_tot[qt];
           sp_bf16* dst = out + (qrow * hq + h) * AT_D + 4 * g;
 #pragma unroll
-          for (int dt = 0; dt < 8; ++dt)
+          for (int dt = 0; dt < (HALF ? 4 : 8); ++dt)
             *reinterpret_cast<uint2*>(dst + dt * 16) =
                 make_uint2(at_pack2(o[dt][qt][0] * inv_l, o[dt][qt][1] * inv_l),
                            at_pack2(o[dt][qt][2] * inv_l, o[dt][qt][3] * inv_l));
@@ -1396,26 +1408,33 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   if (cu_of_device[dev] == 0) {
     hipDeviceProp_t prop;
     SP_HIP(hipGetDeviceProperties(&prop, dev));
-    SP_HIP(hipFuncSetAttribute((const void*)sp_attn_fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)lds_bytes));
-    SP_HIP(hipFuncSetAttribute((const void*)sp_attn_fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)lds_bytes));
+    const void* fwd_kernels[4] = {(const void*)sp_attn_fwd_kernel<false, false>, (const void*)sp_attn_fwd_kernel<true, false>,
+                                  (const void*)sp_attn_fwd_kernel<false, true>, (const void*)sp_attn_fwd_kernel<true, true>};
+    for (const void* f : fwd_kernels)
+      SP_HIP(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     cu_of_device[dev] = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
   const int n_cu = cu_of_device[dev];
   const int64_t total = ((nb + 1) / 2) * hq;  // row pairs
   const int grid = (int)(total < (int64_t)n_cu ? ((total + 7) / 8) * 8 : (int64_t)n_cu);
   float2* stats = want_avg ? rowstat : (float2*)nullptr;
-  hipLaunchKernelGGL(sp_attn_fwd_kernel<false>, dim3(grid), dim3(AT_FWD_THREADS), lds_bytes, s, (const sp_bf16*)q,
-                     (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out, stats, n, hq, hkv,
-                     q_stride_n, q_stride_h, k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2,
-                     counter, max_pivots > 0 ? 1 : 0, (float*)nullptr);
+  const bool half = (flags & SP_ATTN_HALF_CHANNELS) != 0;
+  auto launch_fwd = [&](auto kernel, int skip_slotted, float* block_sums) {
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(AT_FWD_THREADS), lds_bytes, s, (const sp_bf16*)q, (const sp_bf16*)k,
+                       (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out, stats, n, hq, hkv, q_stride_n,
+                       q_stride_h, k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, counter,
+                       skip_slotted, block_sums);
+  };
+  if (half)
+    launch_fwd(sp_attn_fwd_kernel<false, true>, max_pivots > 0 ? 1 : 0, (float*)nullptr);
+  else
+    launch_fwd(sp_attn_fwd_kernel<false, false>, max_pivots > 0 ? 1 : 0, (float*)nullptr);
   SP_LAUNCH_CHECK();
   if (max_pivots > 0) {
-    hipLaunchKernelGGL(sp_attn_fwd_kernel<true>, dim3(grid), dim3(AT_FWD_THREADS), lds_bytes, s, (const sp_bf16*)q,
-                       (const sp_bf16*)k, (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out, stats, n, hq,
-                       hkv, q_stride_n, q_stride_h, k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64),
-                       scale_log2, counter, 0, pivot_u);
+    if (half)
+      launch_fwd(sp_attn_fwd_kernel<true, true>, 0, pivot_u);
+    else
+      launch_fwd(sp_attn_fwd_kernel<true, false>, 0, pivot_u);
     SP_LAUNCH_CHECK();
   }
   if (want_avg) {

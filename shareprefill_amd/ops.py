@@ -274,7 +274,7 @@ def repack_v(v: torch.Tensor, block_size: int, ws: torch.Tensor) -> None:
 
 
 def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=None, avg_attn=None, max_pivots=0,
-                           workspace=None, pair_rows=False):
+                           workspace=None, pair_rows=False, half_channels=False):
     """q [Hq,N,D], k/v [Hkv,N,D] views, mask int64 [Hq,nb,nbw] -> out bf16 [N,Hq,D] contiguous.
 
     Reference: triton_block_wise_prefill_attention (shareprefill_attn.py:474-620).  avg_attn (fp32 [Hq,nb,nb],
@@ -283,7 +283,9 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
     sums during the forward pass, which saves the second pass over Q.K^T.
     workspace: (buffer, bytes) from attention_workspace into which repack_v has ALREADY put this v (and the current
     stream has been made to wait for that); by default the call takes the buffer and repacks itself.
-    pair_rows: skip the per-call analysis of which query blocks share a work item (a dense mask has no use for it)."""
+    pair_rows: skip the per-call analysis of which query blocks share a work item (a dense mask has no use for it).
+    half_channels: q, k and v are zero beyond channel 64 (a smaller head_dim zero-padded to 128): the kernel skips
+    those channels and leaves channels 64.. of out unwritten."""
     lib = _lib.load()
     _check_hnd(q, "q")
     _check_hnd(k, "k")
@@ -307,7 +309,8 @@ def block_sparse_attention(q, k, v, mask, block_size, softmax_scale, decision=No
                                            k.stride(1), k.stride(0), v.stride(1), v.stride(0), block_size,
                                            softmax_scale, _ptr(mask), _ptr(decision), _ptr(out), _ptr(avg_attn),
                                            _ptr(ws), need,
-                                           _lib.SP_ATTN_V_REPACKED | (_lib.SP_ATTN_PAIR_ROWS if pair_rows else 0),
+                                           _lib.SP_ATTN_V_REPACKED | (_lib.SP_ATTN_PAIR_ROWS if pair_rows else 0)
+                                           | (_lib.SP_ATTN_HALF_CHANNELS if half_channels else 0),
                                            _stream(dev))
     if timer is not None:
         timer.stop("attn")

@@ -32,7 +32,8 @@ def pad_head_dim(*tensors: torch.Tensor):
     """The kernels are built for head_dim 128.  The reference's smaller head sizes run on them with the head_dim axis
     zero-padded: no dot product changes (q.k gains exact zeros, the extra output channels are P.0 = 0 and are cut
     off again), the softmax scale and the selection's 1/sqrt(head_dim) keep the model's head_dim.  Costs a copy of
-    q / k / v and 128 / head_dim times the arithmetic."""
+    q / k / v; the attention kernel is told that channels 64.. are zero and skips their products (SP_ATTN_HALF_CHANNELS),
+    so its arithmetic is that of head_dim 64."""
     d = tensors[0].shape[-1]
     return tuple(torch.nn.functional.pad(t, (0, KERNEL_HEAD_DIM - d)) for t in tensors)
 
@@ -119,7 +120,8 @@ def triton_block_wise_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: tor
         decision = torch.where(need_b, _lib.SP_DEC_DENSE, _lib.SP_DEC_VS).to(torch.int32)
         avg = torch.zeros(num_q_heads, nb, nb, dtype=torch.float32, device=dev)
         out = ops.block_sparse_attention(qb, k[b].transpose(0, 1), v[b].transpose(0, 1), mask, block_size, scale,
-                                         decision=decision, avg_attn=avg, max_pivots=max_pivots)
+                                         decision=decision, avg_attn=avg, max_pivots=max_pivots,
+                                         half_channels=model_dim != KERNEL_HEAD_DIM)
         if interleave:
             out = out.reshape(q_len, num_kv_heads, g, head_dim).transpose(1, 2).reshape(q_len, num_q_heads, head_dim)
             avg = avg.reshape(num_kv_heads, g, nb, nb).transpose(0, 1).reshape(num_q_heads, nb, nb)
@@ -182,7 +184,8 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
         # full path instead.
         avg_attn = torch.zeros(1, num_heads, nb, nb, dtype=torch.float32, device=q.device)
         mask = _dense_causal_mask(num_heads, nb, q.device)
-        out = ops.block_sparse_attention(q, k, v, mask, block_size, softmax_scale, pair_rows=True)
+        out = ops.block_sparse_attention(q, k, v, mask, block_size, softmax_scale, pair_rows=True,
+                                         half_channels=model_dim != head_dim)
         if q_len >= block_size:
             sharing.note_dense_layer(module.layer_idx, num_heads, nb)
         return out.unsqueeze(0).transpose(1, 2)[..., :model_dim], avg_attn
@@ -199,7 +202,8 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
                               config.similarity_threshold, config.fallback_threshold, config.queryaware_threshold,
                               scale_dim=model_dim)
     out = ops.block_sparse_attention(q, k, v, plan.mask, block_size, softmax_scale, decision=plan.decision,
-                                     avg_attn=avg_attn[0], max_pivots=max_pivots, workspace=ws)
+                                     avg_attn=avg_attn[0], max_pivots=max_pivots, workspace=ws,
+                                     half_channels=model_dim != head_dim)
     sharing.update_pivotal_attns(module.layer_idx, avg_attn, plan.decision, config.pattern_threshold)
     return out.unsqueeze(0).transpose(1, 2)[..., :model_dim], avg_attn
 
