@@ -475,8 +475,12 @@ __global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_emit_ranked_kernel(const
 }
 
 // ---- score_cover_topk (attn/utils.py:47-50) on flat vectors: the same descent, the count instead of the set ----
+// (its own launch shape: a flat vector is cut into FLAT_SPLIT strided shares of FLAT_THREADS-wide rows; few fat workgroups,
+// all resident at once, instead of 64 x 256 threads: every workgroup pays for clearing and flushing 2048 bins)
+#define FLAT_SPLIT 16
+#define FLAT_THREADS 1024
 template <int LEVEL>
-__global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_hist_flat_kernel(const float* __restrict__ x0,
+__global__ __launch_bounds__(FLAT_THREADS) void sp_gsel_hist_flat_kernel(const float* __restrict__ x0,
                                                                          const float* __restrict__ x1, int n0,
                                                                          int64_t len,
                                                                          const GselState* __restrict__ st,
@@ -490,13 +494,13 @@ __global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_hist_flat_kernel(const f
   constexpr int shift = LEVEL == 0 ? 21 : (LEVEL == 1 ? 10 : 0);
   constexpr int width = LEVEL == 2 ? 10 : 11;
   constexpr int pshift = LEVEL == 0 ? 32 : (LEVEL == 1 ? 21 : 10);
-  for (int i = threadIdx.x; i < SEL_BINS; i += GSEL_THREADS) {
+  for (int i = threadIdx.x; i < SEL_BINS; i += FLAT_THREADS) {
     lsum[i] = 0;
     lcnt[i] = 0;
   }
   __syncthreads();
   const float* xv = v < n0 ? x0 + (int64_t)v * len : x1 + (int64_t)(v - n0) * len;  // vectors n0.. live in x1
-  for (int64_t i0 = (int64_t)blockIdx.x * GSEL_THREADS; i0 < len; i0 += (int64_t)GSEL_SPLIT * GSEL_THREADS) {
+  for (int64_t i0 = (int64_t)blockIdx.x * FLAT_THREADS; i0 < len; i0 += (int64_t)FLAT_SPLIT * FLAT_THREADS) {
     const int64_t i = i0 + threadIdx.x;
     bool live = i < len;
     uint32_t b = 0;
@@ -514,7 +518,7 @@ __global__ __launch_bounds__(GSEL_THREADS) void sp_gsel_hist_flat_kernel(const f
     }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < (1 << width); i += GSEL_THREADS) {
+  for (int i = threadIdx.x; i < (1 << width); i += FLAT_THREADS) {
     if (lcnt[i]) atomicAdd(&gcnt[(int64_t)v * SEL_BINS + i], lcnt[i]);
     if (lsum[i]) atomicAdd(&gsum[(int64_t)v * SEL_BINS + i], lsum[i]);
   }
@@ -601,12 +605,12 @@ static int gsel_count_run(const float* x0, const float* x1, int n0, int n_vec, i
   hipLaunchKernelGGL(sp_gsel_init_kernel, dim3(n_vec), dim3(256), 0, s, st, gcnt, gsum, (const int32_t*)nullptr, -1,
                      n_vec, t_le, (uint64_t*)nullptr, 0, 0);
   SP_LAUNCH_CHECK();
-  const dim3 hgrid(GSEL_SPLIT, n_vec);
-  hipLaunchKernelGGL(sp_gsel_hist_flat_kernel<0>, hgrid, dim3(GSEL_THREADS), 0, s, x0, x1, n0, len, st, gcnt, gsum);
+  const dim3 hgrid(FLAT_SPLIT, n_vec);
+  hipLaunchKernelGGL(sp_gsel_hist_flat_kernel<0>, hgrid, dim3(FLAT_THREADS), 0, s, x0, x1, n0, len, st, gcnt, gsum);
   hipLaunchKernelGGL(sp_gsel_pick_kernel<0>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
-  hipLaunchKernelGGL(sp_gsel_hist_flat_kernel<1>, hgrid, dim3(GSEL_THREADS), 0, s, x0, x1, n0, len, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_hist_flat_kernel<1>, hgrid, dim3(FLAT_THREADS), 0, s, x0, x1, n0, len, st, gcnt, gsum);
   hipLaunchKernelGGL(sp_gsel_pick_kernel<1>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
-  hipLaunchKernelGGL(sp_gsel_hist_flat_kernel<2>, hgrid, dim3(GSEL_THREADS), 0, s, x0, x1, n0, len, st, gcnt, gsum);
+  hipLaunchKernelGGL(sp_gsel_hist_flat_kernel<2>, hgrid, dim3(FLAT_THREADS), 0, s, x0, x1, n0, len, st, gcnt, gsum);
   hipLaunchKernelGGL(sp_gsel_pick_kernel<2>, dim3(n_vec), dim3(SEL_THREADS), 0, s, st, gcnt, gsum);
   hipLaunchKernelGGL(sp_gsel_count_kernel, dim3((n_vec + 63) / 64), dim3(64), 0, s, st, n_vec, t_le, len, out0, out1, n0,
                      bs, minb, maxb);
