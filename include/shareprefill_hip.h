@@ -221,7 +221,8 @@ int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const void* v, i
 /* ---- decode step -------------------------------------------------------------------------------
  * Replaces the flash_attn_func call of the decode branch (shareprefill_attn.py:146-155): one query token per
  * head against the whole KV cache, no mask.  q: bf16 [hq][d] (head stride in elements), k / v: bf16
- * [hkv][n][d] with token and head strides, out: bf16 [hq][d] contiguous.  d = 128, hq / hkv <= 32; q, k, v
+ * [hkv][n][d] with token and head strides, out: bf16 [hq][d] contiguous.  d a multiple of 8 up to 128 (built for
+ * 128; a smaller head is zero-padded to 128 on its way into LDS and reads only its own bytes), hq / hkv <= 32; q, k, v
  * 16-byte aligned with strides that are multiples of 8 elements.
  * workspace: sp_decode_workspace_bytes(n, hq, hkv) bytes of device scratch, 8-byte aligned. */
 size_t sp_decode_workspace_bytes(int64_t n, int32_t hq, int32_t hkv);

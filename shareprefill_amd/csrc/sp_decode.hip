@@ -36,14 +36,18 @@ __device__ static __forceinline__ uint32_t dc_pack2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, dc_bf16x2));
 }
 
-// thread t fetches chunk t%16 (16 bytes) of rows t/16, t/16+16, ... of a 128-row tile; rows past the end are clamped
+// thread t fetches chunk t%16 (16 bytes) of rows t/16, t/16+16, ... of a 128-row tile; rows past the end are clamped.
+// d < 128 (a smaller head): the chunks beyond the row's d channels are zeros made here, not read -- the tile in LDS is
+// the row zero-padded to 128 channels, which changes no product.
 __device__ static __forceinline__ void dc_fetch(const sp_bf16* __restrict__ x, int64_t n, int64_t stride_n, int64_t kb,
-                                               int t, dc_u32x4 (&r)[8]) {
+                                               int t, int d, dc_u32x4 (&r)[8]) {
+  const bool real = (t & 15) * 8 < d;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     int64_t key = kb + i * 16 + (t >> 4);
     if (key > n - 1) key = n - 1;
-    r[i] = *reinterpret_cast<const dc_u32x4*>(x + key * stride_n + (t & 15) * 8);
+    r[i] = (dc_u32x4){0, 0, 0, 0};
+    if (real) r[i] = *reinterpret_cast<const dc_u32x4*>(x + key * stride_n + (t & 15) * 8);
   }
 }
 
@@ -57,8 +61,8 @@ __device__ static __forceinline__ void dc_store(sp_bf16* tile, int t, const dc_u
 template <int G8>
 __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ v, int64_t n, int g,
-    int64_t sq_h, int64_t sk_n, int64_t sk_h, int64_t sv_n, int64_t sv_h, float scale_log2, int64_t keys_per_split,
-    float* __restrict__ o_part, float2* __restrict__ ml_part) {
+    int d, int64_t sq_h, int64_t sk_n, int64_t sk_h, int64_t sv_n, int64_t sv_h, float scale_log2,
+    int64_t keys_per_split, float* __restrict__ o_part, float2* __restrict__ ml_part) {
   __shared__ __attribute__((aligned(16))) sp_bf16 Ks[DC_TILE * DC_PITCH];
   __shared__ __attribute__((aligned(16))) sp_bf16 Vs[DC_TILE * DC_PITCH];
   constexpr int GM = 8 * G8;
@@ -76,7 +80,8 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
     dc_u32x4 raw = {0, 0, 0, 0};
-    if (head_ok) raw = *reinterpret_cast<const dc_u32x4*>(q + (int64_t)(kvh * g + lh) * sq_h + 16 * ks + 8 * hi);
+    if (head_ok && 16 * ks + 8 * hi < d)
+      raw = *reinterpret_cast<const dc_u32x4*>(q + (int64_t)(kvh * g + lh) * sq_h + 16 * ks + 8 * hi);
     qb[ks] = __builtin_bit_cast(dc_bf16x8, raw);
   }
 
@@ -88,8 +93,8 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
   float m_run = -INFINITY, l_run = 0.f;  // of head lh (every wave keeps the same copy)
   dc_u32x4 kr[8], vr[8];
   if (key_begin < key_end) {
-    dc_fetch(kh, n, sk_n, key_begin, t, kr);
-    dc_fetch(vh, n, sv_n, key_begin, t, vr);
+    dc_fetch(kh, n, sk_n, key_begin, t, d, kr);
+    dc_fetch(vh, n, sv_n, key_begin, t, d, vr);
   }
   for (int64_t kb = key_begin; kb < key_end; kb += DC_TILE) {
     __syncthreads();  // the previous tile's operand reads are done
@@ -97,8 +102,8 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
     dc_store(Vs, t, vr);
     __syncthreads();
     if (kb + DC_TILE < key_end) {  // next tile on its way while this one is used
-      dc_fetch(kh, n, sk_n, kb + DC_TILE, t, kr);
-      dc_fetch(vh, n, sv_n, kb + DC_TILE, t, vr);
+      dc_fetch(kh, n, sk_n, kb + DC_TILE, t, d, kr);
+      dc_fetch(vh, n, sv_n, kb + DC_TILE, t, d, vr);
     }
     // ---- S^T for this wave's 32 keys: acc[r] = logit(key 32*wave + 8(r/4) + 4hi + r%4, head lh) ----
     dc_floatx16 acc = {0};
@@ -189,7 +194,7 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
 #define DC_MAX_SPLITS 512
 __global__ __launch_bounds__(DC_D) void sp_decode_combine_kernel(const float* __restrict__ o_part,
                                                                  const float2* __restrict__ ml_part, int g, int splits,
-                                                                 sp_bf16* __restrict__ out) {
+                                                                 int d, sp_bf16* __restrict__ out) {
   __shared__ float w_s[DC_MAX_SPLITS];  // weight of chunk s: exp2(m_s - m), 0 for an empty chunk
   __shared__ float red[2];
   const int hq_idx = blockIdx.x, kvh = hq_idx / g, h = hq_idx % g, c = threadIdx.x;
@@ -212,7 +217,7 @@ __global__ __launch_bounds__(DC_D) void sp_decode_combine_kernel(const float* __
     l += ml[(int64_t)s * g].y * w_s[s];
     o += op[(int64_t)s * g * DC_D] * w_s[s];
   }
-  out[(int64_t)hq_idx * DC_D + c] = sp_f32_to_bf16(o / l);
+  if (c < d) out[(int64_t)hq_idx * d + c] = sp_f32_to_bf16(o / l);
 }
 
 // ---- host -------------------------------------------------------------------------------------------------
@@ -238,7 +243,8 @@ static int dc_check(const char* who, const void* q, const void* k, const void* v
   SP_REQUIRE(n > 0 && hq > 0 && hkv > 0 && hq % hkv == 0, SP_ERR_INVALID_ARGUMENT, "%s: bad shape n=%lld hq=%d hkv=%d",
              who, (long long)n, hq, hkv);
   SP_REQUIRE(softmax_scale > 0.f, SP_ERR_INVALID_ARGUMENT, "%s: softmax_scale must be > 0", who);
-  SP_REQUIRE(d == DC_D, SP_ERR_UNSUPPORTED, "%s: head_dim %d unsupported (only 128)", who, d);
+  SP_REQUIRE(d >= 8 && d <= DC_D && d % 8 == 0, SP_ERR_UNSUPPORTED,
+             "%s: head_dim %d unsupported (a multiple of 8 up to 128)", who, d);
   SP_REQUIRE(hq / hkv <= DC_GMAX, SP_ERR_UNSUPPORTED, "%s: more than %d query heads per kv head", who, DC_GMAX);
   // q, k and v are read with 16-byte loads
   SP_REQUIRE(q_stride_h % 8 == 0 && ((uintptr_t)q % 16) == 0, SP_ERR_UNSUPPORTED,
@@ -251,7 +257,7 @@ static int dc_check(const char* who, const void* q, const void* k, const void* v
 
 // both kernels; `partials` holds sp_decode_workspace_bytes(n, hq, hkv) bytes, every one of which the first kernel
 // writes before the second reads it (nothing has to be cleared)
-static int dc_launch(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,
+static int dc_launch(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv, int32_t d,
                      int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
                      float softmax_scale, void* out, void* partials, hipStream_t s) {
   const int g = hq / hkv;
@@ -262,8 +268,8 @@ static int dc_launch(const void* q, const void* k, const void* v, int64_t n, int
   const float scale_log2 = softmax_scale * 1.4426950408889634f;
 #define DC_LAUNCH_PARTIAL(G8)                                                                                         \
   hipLaunchKernelGGL(sp_decode_partial_kernel<G8>, dim3(splits, hkv), dim3(DC_THREADS), 0, s, (const sp_bf16*)q,      \
-                     (const sp_bf16*)k, (const sp_bf16*)v, n, g, q_stride_h, k_stride_n, k_stride_h, v_stride_n,      \
-                     v_stride_h, scale_log2, keys_per_split, o_part, ml_part)
+                     (const sp_bf16*)k, (const sp_bf16*)v, n, g, (int)d, q_stride_h, k_stride_n, k_stride_h,          \
+                     v_stride_n, v_stride_h, scale_log2, keys_per_split, o_part, ml_part)
   if (g <= 8) {
     DC_LAUNCH_PARTIAL(1);
   } else if (g <= 16) {
@@ -273,7 +279,8 @@ static int dc_launch(const void* q, const void* k, const void* v, int64_t n, int
   }
 #undef DC_LAUNCH_PARTIAL
   SP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sp_decode_combine_kernel, dim3(hq), dim3(DC_D), 0, s, o_part, ml_part, g, splits, (sp_bf16*)out);
+  hipLaunchKernelGGL(sp_decode_combine_kernel, dim3(hq), dim3(DC_D), 0, s, o_part, ml_part, g, splits, (int)d,
+                     (sp_bf16*)out);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
@@ -288,7 +295,7 @@ extern "C" int sp_decode_attn_bf16(const void* q, const void* k, const void* v, 
   SP_REQUIRE(workspace != nullptr, SP_ERR_INVALID_ARGUMENT, "sp_decode_attn_bf16: null workspace");
   SP_REQUIRE(workspace_bytes >= sp_decode_workspace_bytes(n, hq, hkv) && ((uintptr_t)workspace % 8) == 0,
              SP_ERR_WORKSPACE, "sp_decode_attn_bf16: workspace too small or misaligned");
-  return dc_launch(q, k, v, n, hq, hkv, q_stride_h, k_stride_n, k_stride_h, v_stride_n, v_stride_h, softmax_scale, out,
+  return dc_launch(q, k, v, n, hq, hkv, d, q_stride_h, k_stride_n, k_stride_h, v_stride_n, v_stride_h, softmax_scale, out,
                    workspace, (hipStream_t)stream);
 }
 
@@ -333,6 +340,6 @@ extern "C" int sp_decode_attn_static_bf16(const void* q, const void* k, const vo
   void* partials = nullptr;
   rc = dc_static_scratch(&partials);
   if (rc) return rc;
-  return dc_launch(q, k, v, n, hq, hkv, q_stride_h, k_stride_n, k_stride_h, v_stride_n, v_stride_h, softmax_scale, out,
+  return dc_launch(q, k, v, n, hq, hkv, d, q_stride_h, k_stride_n, k_stride_h, v_stride_n, v_stride_h, softmax_scale, out,
                    partials, (hipStream_t)stream);
 }

@@ -141,9 +141,6 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
     bsz, num_heads, q_len, model_dim = query_states.shape
     config = module.config
     softmax_scale = getattr(module, "scaling", 1.0 / math.sqrt(model_dim))
-    if model_dim in PADDED_HEAD_DIMS:
-        query_states, key_states, value_states = pad_head_dim(query_states, key_states, value_states)
-    head_dim = query_states.shape[-1]
     # gqa_interleave is accepted and changes nothing, as in the reference: there K and V are expanded to the query
     # head count before anything else, by repeat_interleave (True) or by expand + reshape (False) -- both give query
     # head h the kv head h // g (shareprefill_attn.py:33-40, 77-82) -- and everything after sees one kv head per query
@@ -153,16 +150,20 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
 
     if q_len == 1:
         # decode step (shareprefill_attn.py:146-155): one query against the whole cache, nothing is selected.
-        # The HIP kernel is the only path (bf16, head_dim 128, at most 32 query heads per kv head, 16-byte aligned
-        # rows); anything else raises from the entry point's own checks, as every other unsupported shape does.
+        # The HIP kernel is the only path (bf16, head_dim a multiple of 8 up to 128 -- smaller heads are padded inside
+        # the kernel, the cache is read as it is -- at most 32 query heads per kv head, 16-byte aligned rows); anything
+        # else raises from the entry point's own checks, as every other unsupported shape does.
         if query_states.dtype != torch.bfloat16:
             raise AssertionError(f"SharePrefill attention expects bfloat16 q/k/v, got {query_states.dtype}")
         outs = [ops.decode_attention(query_states[b, :, 0], key_states[b], value_states[b], softmax_scale)
                 for b in range(bsz)]
-        return torch.stack(outs).unsqueeze(2)[..., :model_dim], None
+        return torch.stack(outs).unsqueeze(2), None
 
     if bsz != 1:
         raise ValueError("SharePrefill prefill keeps per-cluster state for batch size 1 only")
+    if model_dim in PADDED_HEAD_DIMS:
+        query_states, key_states, value_states = pad_head_dim(query_states, key_states, value_states)
+    head_dim = query_states.shape[-1]
     assert query_states.dtype == torch.bfloat16, "SharePrefill attention expects bfloat16 q/k/v"
     assert key_states.shape[2] == q_len, "prefill expects q_len == k_len (no cached prefix)"
     _lib.load()
