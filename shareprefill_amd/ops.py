@@ -8,7 +8,6 @@ head-major q/k/v given as [H, N, D] views with arbitrary token / head strides an
 from __future__ import annotations
 
 import ctypes as C
-import math
 from typing import Optional
 
 import torch

@@ -9,8 +9,6 @@ Two comparisons per layer:
 Attention outputs are checked against the fp32 masked-attention oracle on the GPU's mask.
 """
 
-import json
-import math
 import types
 
 import numpy as np

@@ -1,6 +1,5 @@
 """GPU parity: block average pooling (HIP) against the CPU oracle, through the C ABI."""
 
-import numpy as np
 import pytest
 import torch
 
