@@ -299,3 +299,34 @@ def test_attention_rejects_unsupported(gpu_device):
     q = torch.zeros(257, 128, 128, dtype=torch.bfloat16, device=gpu_device)  # one query head too many
     with pytest.raises(NotImplementedError):
         ops.block_sparse_attention(q, q, q, torch.ones(257, 1, 1, dtype=torch.int64, device=gpu_device), 128, 1.0)
+
+
+@pytest.mark.parametrize("max_pivots", [0, 2])
+def test_half_channel_mode_gives_the_bits_of_the_full_kernel_on_padded_inputs(gpu_device, max_pivots):
+    """q, k, v with zeros beyond channel 64 (a head_dim-64 model padded to the kernel's 128): the instantiation that
+    skips those channels must give the first 64 output channels and the pivots' block-average maps of the full kernel
+    bit for bit -- at 32768 tokens, with a random mask, two pivot heads, and both ways the maps are made."""
+    from shareprefill_amd import ops
+
+    hq, hkv, n = 8, 2, 32768
+    nb = n // 128
+    g = torch.Generator(device=gpu_device).manual_seed(64)
+    mk = lambda h: torch.nn.functional.pad(
+        torch.randn(n, h, 64, device=gpu_device, generator=g).to(torch.bfloat16), (0, 64)).transpose(0, 1)
+    q, k, v = mk(hq), mk(hkv), mk(hkv)
+    mask = ops.bool_to_mask(torch.from_numpy(_random_mask(hq, nb, 64, density=0.3))).to(gpu_device)
+    mask[1] = ops.bool_to_mask(torch.tril(torch.ones(nb, nb, dtype=torch.bool)))  # the pivots attend densely
+    mask[6] = mask[1]
+    decision = torch.zeros(hq, dtype=torch.int32, device=gpu_device)
+    decision[1] = decision[6] = 1
+    res = []
+    for half in (False, True):
+        avg = torch.zeros(hq, nb, nb, dtype=torch.float32, device=gpu_device)
+        out = ops.block_sparse_attention(q, k, v, mask, 128, 0.125, decision=decision, avg_attn=avg,
+                                         max_pivots=max_pivots, half_channels=half)
+        res.append((out, avg))
+    (full, avg_full), (half_out, avg_half) = res
+    assert float(full[..., 64:].abs().max()) == 0.0
+    assert torch.equal(half_out[..., :64], full[..., :64])
+    assert torch.equal(avg_half, avg_full)
+    assert torch.allclose(avg_full[1].sum(-1), torch.ones(nb, device=gpu_device), atol=2e-3)
