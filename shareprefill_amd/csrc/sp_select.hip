@@ -924,41 +924,96 @@ extern "C" int sp_queryaware_test_bf16(const void* q, const void* kbar, const fl
 // cols[c] = 1 for the nv best columns (column 0 forced), dists[dd] = 1 for the ns best distances
 // (distance 0 forced); slash index i holds distance nb-1-i.
 // ------------------------------------------------------------------------------------------------
-// rank of element i in the order (key descending, index ascending) = #{j < i: key_j >= key_i} + #{j > i: key_j > key_i};
-// keys [nbp] in LDS, padded with zeros to a multiple of 4 (a zero key never outranks anything but zeros behind i)
-__device__ static inline int vs_rank(const uint32_t* keys, int nb, int i) {
-  const uint32_t ki = keys[i];
-  int r = 0;
-  const int i4 = i & ~3;
-  for (int j = 0; j < i4; j += 4) {
-    const uint4 k4 = *reinterpret_cast<const uint4*>(keys + j);
-    r += (k4.x >= ki) + (k4.y >= ki) + (k4.z >= ki) + (k4.w >= ki);
+// Membership in the top k of the order (key descending, index ascending), for every element at once, by selection
+// instead of ranking: four 8-bit radix passes over the keys find the k-th key T (a 256-bin histogram in LDS and one
+// wave that walks it from the top), then an element is in iff key > T, or key == T and fewer than `take` equal keys
+// have a lower index (ballots and per-wave counts give that index order).  O(nb) per workgroup where ranking every
+// element against every other was O(nb^2 / threads) -- 50 us of a 1024-thread workgroup at nb = 1024.
+// Every thread of the workgroup calls it (nthreads = blockDim.x, a multiple of 64); flags[map(i)] = 1 / 0 for i < nb
+// with map(i) = reverse ? nb - 1 - i : i.
+__device__ static void vs_topk_flags(const uint32_t* keys, int nb, int k, uint8_t* flags, bool reverse, int nthreads) {
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t wave_cnt[16];
+  __shared__ uint32_t s_prefix, s_take, s_base;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = nthreads >> 6;
+  if (k >= nb || k <= 0) {  // (uniform) everything or nothing
+    for (int i = threadIdx.x; i < nb; i += nthreads) flags[reverse ? nb - 1 - i : i] = k > 0;
+    __syncthreads();
+    return;
   }
-  for (int j = i4; j < i; ++j) r += keys[j] >= ki;
-  const int e4 = (i + 4) & ~3;
-  for (int j = i + 1; j < e4 && j < nb; ++j) r += keys[j] > ki;
-  for (int j = e4; j < nb; j += 4) {  // reads up to 3 padding zeros past nb: they never count (0 > ki is false)
-    const uint4 k4 = *reinterpret_cast<const uint4*>(keys + j);
-    r += (k4.x > ki) + (k4.y > ki) + (k4.z > ki) + (k4.w > ki);
+  if (threadIdx.x == 0) {
+    s_prefix = 0u;
+    s_take = (uint32_t)k;
   }
-  return r;
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    for (int b = threadIdx.x; b < 256; b += nthreads) hist[b] = 0u;
+    __syncthreads();
+    const uint32_t prefix = s_prefix;
+    for (int i = threadIdx.x; i < nb; i += nthreads) {
+      const uint32_t key = keys[i];
+      if (pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8))) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (wave == 0) {  // the bin where the running count from the top reaches the number still to take
+      uint32_t c[4], tot = 0;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        c[u] = hist[255 - (4 * lane + u)];  // lane 0 holds the four top bins
+        tot += c[u];
+      }
+      uint32_t incl = tot;  // inclusive scan over lanes
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t o = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += o;
+      }
+      uint32_t above = incl - tot;
+      const uint32_t take = s_take;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (above < take && above + c[u] >= take) {  // exactly one (lane, u) satisfies this
+          s_prefix = prefix | ((uint32_t)(255 - (4 * lane + u)) << shift);
+          s_take = take - above;
+        }
+        above += c[u];
+      }
+    }
+    __syncthreads();
+  }
+  const uint32_t T = s_prefix, take = s_take;  // take >= 1 keys equal to T belong, lowest indices first
+  if (threadIdx.x == 0) s_base = 0u;
+  __syncthreads();
+  for (int i0 = 0; i0 < nb; i0 += nthreads) {  // (uniform trip count: every lane votes)
+    const int i = i0 + threadIdx.x;
+    const uint32_t key = i < nb ? keys[i] : 0u;
+    const bool eq = i < nb && key == T;
+    const unsigned long long bal = __ballot(eq);
+    if (lane == 0) wave_cnt[wave] = __popcll(bal);
+    __syncthreads();
+    uint32_t before = s_base, tot = 0;
+    for (int w = 0; w < nwaves; ++w) {
+      if (w < wave) before += wave_cnt[w];
+      tot += wave_cnt[w];
+    }
+    before += __popcll(bal & ((1ull << lane) - 1ull));
+    if (i < nb) flags[reverse ? nb - 1 - i : i] = key > T || (eq && before < take);
+    __syncthreads();  // counts and base have been read
+    if (threadIdx.x == 0) s_base += tot;
+    __syncthreads();
+  }
 }
 
 __device__ static void vs_sets(const float* __restrict__ vert, const float* __restrict__ slash, int nb, int nv,
                                int ns, uint32_t* keys /* LDS [RS_MAX], 16-byte aligned */, uint8_t* cols,
                                uint8_t* dists, int nthreads) {
   const uint32_t inf_key = 0x7f800000u;
-  const int nbp = (nb + 3) & ~3;
-  for (int i = threadIdx.x; i < nbp; i += nthreads)
-    keys[i] = i >= nb ? 0u : ((i == 0) ? inf_key : sp_sort_key(vert[i]));
+  for (int i = threadIdx.x; i < nb; i += nthreads) keys[i] = (i == 0) ? inf_key : sp_sort_key(vert[i]);
   __syncthreads();
-  for (int i = threadIdx.x; i < nb; i += nthreads) cols[i] = vs_rank(keys, nb, i) < nv;
+  vs_topk_flags(keys, nb, nv, cols, false, nthreads);
+  for (int i = threadIdx.x; i < nb; i += nthreads) keys[i] = (i == nb - 1) ? inf_key : sp_sort_key(slash[i]);
   __syncthreads();
-  for (int i = threadIdx.x; i < nbp; i += nthreads)
-    keys[i] = i >= nb ? 0u : ((i == nb - 1) ? inf_key : sp_sort_key(slash[i]));
-  __syncthreads();
-  for (int i = threadIdx.x; i < nb; i += nthreads) dists[nb - 1 - i] = vs_rank(keys, nb, i) < ns;
-  __syncthreads();
+  vs_topk_flags(keys, nb, ns, dists, true, nthreads);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1114,18 +1169,41 @@ __global__ __launch_bounds__(MASK_THREADS) void sp_build_mask_kernel(
   // a SHARE decision without a valid slot (only a caller's own decision vector can hold one) adds no pattern
   if (dec == SP_DEC_SHARE && sp_slot_ok(st, head_cluster[h])) pat = st.pattern + (int64_t)head_cluster[h] * nb * nbw;
   uint64_t* mh = mask + (int64_t)h * nb * nbw;
+  // Both sets as bit strings: colw = the columns, dstw = the distances in the order of the slash index i = nb - 1 - d.
+  // Row r, columns c0 .. c0 + 63 then want distance bits i = nb - 1 - r + c0 .. + 63: a 64-bit window of dstw, so a mask
+  // word is two shifts and an OR instead of 64 pairs of byte look-ups.
+  __shared__ uint64_t colw[RS_MAX / 64], dstw[RS_MAX / 64 + 1];
+  if (dec != SP_DEC_DENSE) {
+    const int lane = threadIdx.x & 63;
+    for (int i0 = 0; i0 < nbw * 64; i0 += MASK_THREADS) {  // (uniform trip count: every lane votes)
+      const int i = i0 + threadIdx.x;
+      const unsigned long long cb = __ballot(i < nb && s_cols[i] != 0);
+      const unsigned long long db = __ballot(i < nb && s_dists[nb - 1 - i] != 0);
+      if (lane == 0 && i < nbw * 64) {
+        colw[i >> 6] = cb;
+        dstw[i >> 6] = db;
+      }
+    }
+    if (threadIdx.x == 0) dstw[nbw] = 0ull;
+    __syncthreads();
+  }
   const int rows_per = (nb + MASK_SPLIT - 1) / MASK_SPLIT;
   const int r_begin = blockIdx.y * rows_per, r_end = min(nb, r_begin + rows_per);
   for (int idx = r_begin * nbw + threadIdx.x; idx < r_end * nbw; idx += MASK_THREADS) {
     const int r = idx / nbw, w = idx - r * nbw;
-    uint64_t bits = 0;
     const int c0 = w * 64;
     const int cend = min(c0 + 64, r + 1);
-    if (dec == SP_DEC_DENSE) {
-      if (cend > c0) bits = (cend - c0 == 64) ? ~0ull : ((1ull << (cend - c0)) - 1ull);
-    } else {
-      for (int c = c0; c < cend; ++c) {
-        if (s_cols[c] | s_dists[r - c]) bits |= 1ull << (c - c0);
+    // the causal part of the word: columns c0 .. cend - 1
+    const uint64_t causal = cend <= c0 ? 0ull : ((cend - c0 == 64) ? ~0ull : ((1ull << (cend - c0)) - 1ull));
+    uint64_t bits = causal;
+    if (dec != SP_DEC_DENSE) {
+      bits = 0ull;
+      if (causal) {
+        const int start = nb - 1 - r + c0;  // >= 0; bits past nb - 1 belong to columns beyond r
+        const int k = start >> 6, sh = start & 63;
+        uint64_t win = dstw[k] >> sh;
+        if (sh) win |= dstw[k + 1] << (64 - sh);
+        bits = (colw[w] | win) & causal;
       }
       if (pat) bits |= pat[idx];
     }
