@@ -788,7 +788,7 @@ __device__ static float wave_sqrt_js(const float* __restrict__ p, const float* _
 // ------------------------------------------------------------------------------------------------
 // query-aware test (attention_sharing.py:193-202)
 // ------------------------------------------------------------------------------------------------
-#define QA_THREADS 256
+#define QA_THREADS 1024
 __global__ __launch_bounds__(QA_THREADS) void sp_queryaware_test_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ kbar, const float* __restrict__ vert_blk, int64_t n,
     int hq, int hkv, int d, int64_t sq_n, int64_t sq_h, int bs, int nb, uint32_t flags, float inv_sqrt_d, float thr,
