@@ -39,15 +39,21 @@ __device__ static __forceinline__ uint32_t dc_pack2(float a, float b) {
 // thread t fetches chunk t%16 (16 bytes) of rows t/16, t/16+16, ... of a 128-row tile; rows past the end are clamped.
 // d < 128 (a smaller head): the chunks beyond the row's d channels are zeros made here, not read -- the tile in LDS is
 // the row zero-padded to 128 channels, which changes no product.
+// (FULL: d == 128, nothing to pad -- the plain loads of the kernel's own head size)
+template <bool FULL>
 __device__ static __forceinline__ void dc_fetch(const sp_bf16* __restrict__ x, int64_t n, int64_t stride_n, int64_t kb,
                                                int t, int d, dc_u32x4 (&r)[8]) {
-  const bool real = (t & 15) * 8 < d;
+  const bool real = FULL || (t & 15) * 8 < d;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     int64_t key = kb + i * 16 + (t >> 4);
     if (key > n - 1) key = n - 1;
-    r[i] = (dc_u32x4){0, 0, 0, 0};
-    if (real) r[i] = *reinterpret_cast<const dc_u32x4*>(x + key * stride_n + (t & 15) * 8);
+    if (FULL) {
+      r[i] = *reinterpret_cast<const dc_u32x4*>(x + key * stride_n + (t & 15) * 8);
+    } else {
+      r[i] = (dc_u32x4){0, 0, 0, 0};
+      if (real) r[i] = *reinterpret_cast<const dc_u32x4*>(x + key * stride_n + (t & 15) * 8);
+    }
   }
 }
 
@@ -58,7 +64,7 @@ __device__ static __forceinline__ void dc_store(sp_bf16* tile, int t, const dc_u
 
 // grid (splits, hkv); partial layout: o [hkv][splits][g][128] fp32, ml [hkv][splits][g] float2 (m in log2 units, l)
 // G8 = groups of 8 heads the instance handles (g <= 8 * G8): accumulator rows r < 4 * G8 can belong to real heads
-template <int G8>
+template <int G8, bool FULL>
 __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ v, int64_t n, int g,
     int d, int64_t sq_h, int64_t sk_n, int64_t sk_h, int64_t sv_n, int64_t sv_h, float scale_log2,
@@ -80,7 +86,7 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
     dc_u32x4 raw = {0, 0, 0, 0};
-    if (head_ok && 16 * ks + 8 * hi < d)
+    if (head_ok && (FULL || 16 * ks + 8 * hi < d))
       raw = *reinterpret_cast<const dc_u32x4*>(q + (int64_t)(kvh * g + lh) * sq_h + 16 * ks + 8 * hi);
     qb[ks] = __builtin_bit_cast(dc_bf16x8, raw);
   }
@@ -93,8 +99,8 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
   float m_run = -INFINITY, l_run = 0.f;  // of head lh (every wave keeps the same copy)
   dc_u32x4 kr[8], vr[8];
   if (key_begin < key_end) {
-    dc_fetch(kh, n, sk_n, key_begin, t, d, kr);
-    dc_fetch(vh, n, sv_n, key_begin, t, d, vr);
+    dc_fetch<FULL>(kh, n, sk_n, key_begin, t, d, kr);
+    dc_fetch<FULL>(vh, n, sv_n, key_begin, t, d, vr);
   }
   for (int64_t kb = key_begin; kb < key_end; kb += DC_TILE) {
     __syncthreads();  // the previous tile's operand reads are done
@@ -102,8 +108,8 @@ __global__ __launch_bounds__(DC_THREADS, 2) void sp_decode_partial_kernel(
     dc_store(Vs, t, vr);
     __syncthreads();
     if (kb + DC_TILE < key_end) {  // next tile on its way while this one is used
-      dc_fetch(kh, n, sk_n, kb + DC_TILE, t, d, kr);
-      dc_fetch(vh, n, sv_n, kb + DC_TILE, t, d, vr);
+      dc_fetch<FULL>(kh, n, sk_n, kb + DC_TILE, t, d, kr);
+      dc_fetch<FULL>(vh, n, sv_n, kb + DC_TILE, t, d, vr);
     }
     // ---- S^T for this wave's 32 keys: acc[r] = logit(key 32*wave + 8(r/4) + 4hi + r%4, head lh) ----
     dc_floatx16 acc = {0};
@@ -266,10 +272,17 @@ static int dc_launch(const void* q, const void* k, const void* v, int64_t n, int
   float* o_part = (float*)partials;
   float2* ml_part = (float2*)(o_part + (size_t)splits * hq * DC_D);
   const float scale_log2 = softmax_scale * 1.4426950408889634f;
-#define DC_LAUNCH_PARTIAL(G8)                                                                                         \
-  hipLaunchKernelGGL(sp_decode_partial_kernel<G8>, dim3(splits, hkv), dim3(DC_THREADS), 0, s, (const sp_bf16*)q,      \
+#define DC_LAUNCH_PARTIAL_(G8, FULL)                                                                                  \
+  hipLaunchKernelGGL((sp_decode_partial_kernel<G8, FULL>), dim3(splits, hkv), dim3(DC_THREADS), 0, s, (const sp_bf16*)q, \
                      (const sp_bf16*)k, (const sp_bf16*)v, n, g, (int)d, q_stride_h, k_stride_n, k_stride_h,          \
                      v_stride_n, v_stride_h, scale_log2, keys_per_split, o_part, ml_part)
+#define DC_LAUNCH_PARTIAL(G8)     \
+  do {                            \
+    if (d == DC_D)                \
+      DC_LAUNCH_PARTIAL_(G8, true);  \
+    else                          \
+      DC_LAUNCH_PARTIAL_(G8, false); \
+  } while (0)
   if (g <= 8) {
     DC_LAUNCH_PARTIAL(1);
   } else if (g <= 16) {
@@ -278,6 +291,7 @@ static int dc_launch(const void* q, const void* k, const void* v, int64_t n, int
     DC_LAUNCH_PARTIAL(4);
   }
 #undef DC_LAUNCH_PARTIAL
+#undef DC_LAUNCH_PARTIAL_
   SP_LAUNCH_CHECK();
   hipLaunchKernelGGL(sp_decode_combine_kernel, dim3(hq), dim3(DC_D), 0, s, o_part, ml_part, g, splits, (int)d,
                      (sp_bf16*)out);
