@@ -288,6 +288,23 @@ def test_layer_ragged_length(gpu_device, tmp_path):
     check_outputs(run)
 
 
+@pytest.mark.parametrize("n", [128, 129, 200, 256, 257, 383, 385])
+@pytest.mark.parametrize("qat", [0.1, 10.0])
+def test_layer_of_one_to_four_blocks(gpu_device, tmp_path, n, qat):
+    """The whole selection (not the dense short-prompt shortcut) on prompts of one to four blocks, ragged and not, with
+    the minimum budget at one block; queryaware_threshold 10 sends every head down the query-aware path.  Degenerate
+    sizes for every kernel: one-entry vectors, a single diagonal block, pivots whose map is 1 x 1."""
+    run = run_layers(gpu_device, tmp_path, hq=4, hkv=2, n=n, seed=n, n_clusters=2, min_budget=128,
+                     fallback_threshold=1e9, queryaware_threshold=qat)
+    check_forced(run)
+    if n > 128:
+        # (with a single block both distributions of the query-aware test are [1] up to rounding, and their sqrt-JS is
+        # the square root of rounding noise around zero: 0, 2e-4 or NaN by the last bit of a sum, here as in the
+        # reference -- nothing to compare; every mask is the one block whatever it decides)
+        check_free(run, expect_same_masks=False)
+    check_outputs(run)
+
+
 def test_reference_style_interfaces(gpu_device, tmp_path):
     """get_active_blocks / update_pivotal_attns with the reference's argument layout, and the id-list view."""
     from shareprefill_amd import AttentionSharing, ops
