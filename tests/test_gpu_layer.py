@@ -38,7 +38,7 @@ class FakeAttention:
 
 
 def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_free=True, with_forced=True, d=128,
-               **thr):
+               shared=None, **thr):
     from shareprefill_amd import AttentionSharing, shareprefill_attention_forward, ops
 
     # dense_short_prompts off: these tests compare the selection itself, also where the prompt is so short that every
@@ -47,6 +47,8 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_fre
               fallback_threshold=0.9, queryaware_threshold=0.1, dense_short_prompts=False)
     kw.update(thr)
     table = synthetic.random_cluster_table(hq, n_clusters, n_layers, seed)
+    if shared is not None:  # only these clusters share (the shipped Llama table shares one of its 44)
+        table["shared_clusters"] = list(shared)
     path = synthetic.write_cluster_table(table, str(tmp_path / "table.json"))
     q, k, v = synthetic.planted_qkv(hq, hkv, n, d, seed, q_head_gain=1.0)
     sharing = AttentionSharing(path)
@@ -303,6 +305,24 @@ def test_layer_of_one_to_four_blocks(gpu_device, tmp_path, n, qat):
         # reference -- nothing to compare; every mask is the one block whatever it decides)
         check_free(run, expect_same_masks=False)
     check_outputs(run)
+
+
+@pytest.mark.parametrize("shared", [[], ["1"], ["0", "3"]])
+def test_layer_with_few_or_no_shared_clusters(gpu_device, tmp_path, shared):
+    """Tables in which only some clusters share, or none does (no device slot at all): heads outside the shared
+    clusters never become pivots and never share, whatever the thresholds."""
+    run = run_layers(gpu_device, tmp_path, hq=8, hkv=2, n=3000, seed=77, n_clusters=4, n_layers=3, shared=shared,
+                     fallback_threshold=1e9, min_budget=512)
+    check_forced(run)
+    check_free(run)
+    check_outputs(run)
+    dense_per_layer = [int((L["dec"] == O.DEC_DENSE).sum()) for L in run["layers"]]
+    assert dense_per_layer[0] == len(shared) and sum(dense_per_layer[1:]) == 0
+    member = {h for cid in shared for layer, h in run["table"]["clusters"][cid]}
+    for L in run["layers"]:
+        for h in range(8):
+            if h not in member:
+                assert L["dec"][h] in (O.DEC_VS, O.DEC_QA)
 
 
 def test_reference_style_interfaces(gpu_device, tmp_path):
