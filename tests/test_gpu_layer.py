@@ -325,6 +325,23 @@ def test_layer_with_few_or_no_shared_clusters(gpu_device, tmp_path, shared):
                 assert L["dec"][h] in (O.DEC_VS, O.DEC_QA)
 
 
+@pytest.mark.parametrize("min_budget,max_budget,thr", [(512, 1536, 0.95), (128, 128, 0.99), (2048, 1024, 0.9), (None, None, 0.5),
+                                                       (1, 100000, 0.999)])
+def test_layer_budget_clamps(gpu_device, tmp_path, min_budget, max_budget, thr):
+    """min_budget / max_budget in tokens, converted and clamped as shareprefill_attn.py:112-122 and
+    attention_sharing.py:169-176 do: a maximum below what the threshold asks for, a maximum of one block, a minimum
+    above the maximum (the maximum wins: it is applied last), no limits at all, and limits that never bind."""
+    run = run_layers(gpu_device, tmp_path, hq=8, hkv=2, n=4096, seed=31, n_clusters=2, min_budget=min_budget,
+                     max_budget=max_budget, pattern_threshold=thr, fallback_threshold=1e9)
+    check_forced(run)
+    check_free(run, expect_same_masks=False)
+    check_outputs(run)
+    if max_budget is not None:
+        cap = min(-(-max_budget // 128), run["nb"])
+        for L in run["layers"]:
+            assert int(L["plan"].nv.max()) <= cap and int(L["plan"].ns.max()) <= cap
+
+
 def test_reference_style_interfaces(gpu_device, tmp_path):
     """get_active_blocks / update_pivotal_attns with the reference's argument layout, and the id-list view."""
     from shareprefill_amd import AttentionSharing, ops
