@@ -342,6 +342,17 @@ def test_layer_budget_clamps(gpu_device, tmp_path, min_budget, max_budget, thr):
             assert int(L["plan"].nv.max()) <= cap and int(L["plan"].ns.max()) <= cap
 
 
+@pytest.mark.parametrize("hq,hkv,n_clusters", [(1, 1, 1), (3, 3, 1), (5, 1, 1), (12, 4, 3), (6, 6, 2), (9, 3, 3)])
+def test_layer_head_counts(gpu_device, tmp_path, hq, hkv, n_clusters):
+    """One head, no grouping, odd groups, groups of three: the kv-head mapping of every kernel and the work-item
+    pairing (two adjacent heads only inside one kv group; an odd head pairs its own rows)."""
+    run = run_layers(gpu_device, tmp_path, hq=hq, hkv=hkv, n=1500, seed=10 * hq + hkv, n_clusters=n_clusters,
+                     min_budget=256, fallback_threshold=1e9)
+    check_forced(run)
+    check_free(run, expect_same_masks=False)
+    check_outputs(run)
+
+
 def test_reference_style_interfaces(gpu_device, tmp_path):
     """get_active_blocks / update_pivotal_attns with the reference's argument layout, and the id-list view."""
     from shareprefill_amd import AttentionSharing, ops
