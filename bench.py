@@ -538,6 +538,9 @@ def main():
                                          "constant_operands": round(ops.mfma_probe_tflops(0), 1),
                                          "library_gemm_8192_random_data": round(library_gemm_tflops(dev), 1),
                                          "nominal_peak": PEAK_BF16_TFLOPS}
+        # the attention kernel against what MFMAs alone sustain on this chip under the same power limit
+        sustained = line["mfma_sustained_tflops"]["random_operands_changing_every_instruction"]
+        line["mfma_sustained_tflops"]["attention_kernel_over_sustained"] = round(attn_tflops / sustained, 4)
         if not args.no_sweep:
             sweep = []
             for thr in (0.9, 0.95, 0.99):
