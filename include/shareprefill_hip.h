@@ -60,7 +60,8 @@ typedef struct sp_cluster_state {
   int32_t n_clusters;
   int32_t nb;  /* blocks per side the slabs are sized for */
   int32_t nbw; /* ceil(nb/64) */
-  int32_t reserved;
+  int32_t struct_bytes; /* sizeof(sp_cluster_state) as the caller was compiled.  0 or SP_CLUSTER_STATE_V1_BYTES = the
+                           first layout of this struct, which ended with `accum`: no member behind it is read */
   int32_t* info;     /* [C][8]: 0 pivot head (-1 none), 1 has_pattern, 2 pivot nv, 3 pivot ns, 4 pivot layer,
                         5 rows counted by a running sp_pivot_update (zero between calls) */
   double* ratio;     /* [C]     vs_ratio of the pivot (valid once has_pattern) */
@@ -73,8 +74,9 @@ typedef struct sp_cluster_state {
                         every completed call leaves it zero again: allocate it zero-filled */
   float* avg_map;    /* [C][nb][nb] or NULL: the pivot's block-average attention map, kept by sp_pivot_update for
                         AttentionSharing.get_pivotal_attn (attention_sharing.py:87-99); valid once has_pattern
-                        (since library version 2) */
+                        (since library version 2; read only when struct_bytes >= sizeof(sp_cluster_state)) */
 } sp_cluster_state;
+#define SP_CLUSTER_STATE_V1_BYTES 80 /* 4 x int32 + 8 pointers */
 
 /* ---- library info ------------------------------------------------------------------------- */
 int sp_version(void);
@@ -157,10 +159,13 @@ int sp_build_mask(const sp_cluster_state* state /* host */, const int32_t* head_
 /* ---- query-aware block selection (attention_sharing.py:339-364, attn/utils.py:53-57) --------
  * For heads with decision == SP_DEC_QA: probs[h] = softmax rows of (qbar[h]/sqrt(d)) . kbar^T with the
  * block-causal mask ([nb][nb] fp32, caller scratch [hq][nb][nb]); then the global cumulative-mass
- * selection at pattern_threshold * nb (crossing entry excluded) is OR-ed into mask[h].
+ * selection at pattern_threshold * nb (crossing entry excluded) is OR-ed into mask[h].  pattern_threshold is a
+ * double because the reference forms that product from the Python float before the comparison takes it to fp32:
+ * score = fp32(pattern_threshold * nb) (attention_sharing.py:361, attn/utils.py:56).
  * qbar: bf16 [nb][hq][d] (sp_pool_avg_bf16 of q), kbar: bf16 [nb][hkv][d]. */
+float sp_queryaware_select_score(double pattern_threshold, int32_t nb); /* host arithmetic only: the score above */
 int sp_queryaware_select_bf16(const void* qbar, const void* kbar, const int32_t* decision, int32_t hq,
-                              int32_t hkv, int32_t d, int32_t nb, uint32_t flags, float pattern_threshold,
+                              int32_t hkv, int32_t d, int32_t nb, uint32_t flags, double pattern_threshold,
                               float* probs, uint64_t* mask, void* workspace, size_t workspace_bytes,
                               sp_stream_t stream);
 
@@ -261,7 +266,8 @@ int sp_rope_inplace_bf16(void* q, void* k, const void* cos_t, const void* sin_t,
 /* ---- pivot state update (attention_sharing.py:94-103, attn/utils.py:60-76) ------------------
  * For each head with decision == SP_DEC_DENSE: per-row cumulative-mass selection (>= threshold,
  * crossing entry included) of avg_attn[h] -> state.pattern, the pivot's vs_ratio
- * (attention_sharing.py:278-286, duplicates counted) -> state.ratio, has_pattern = 1. */
+ * (attention_sharing.py:278-286, duplicates counted) -> state.ratio, has_pattern = 1.  When several DENSE heads name
+ * the same cluster, the highest head's map is the one kept (the reference stores them in ascending order). */
 int sp_pivot_update(const sp_cluster_state* state /* host */, const int32_t* head_cluster, const int32_t* decision,
                     const float* avg_attn, int32_t hq, int32_t nb, float pattern_threshold, sp_stream_t stream);
 

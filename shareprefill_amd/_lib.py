@@ -33,7 +33,7 @@ class ClusterStateStruct(C.Structure):
     """struct sp_cluster_state (host struct holding device pointers)."""
 
     _fields_ = [
-        ("n_clusters", C.c_int32), ("nb", C.c_int32), ("nbw", C.c_int32), ("reserved", C.c_int32),
+        ("n_clusters", C.c_int32), ("nb", C.c_int32), ("nbw", C.c_int32), ("struct_bytes", C.c_int32),
         ("info", C.c_void_p), ("ratio", C.c_void_p), ("vert", C.c_void_p), ("slash", C.c_void_p),
         ("cols", C.c_void_p), ("dists", C.c_void_p), ("pattern", C.c_void_p), ("accum", C.c_void_p),
         ("avg_map", C.c_void_p),
@@ -60,7 +60,8 @@ SIGNATURES = {
                                        _P]),
     "sp_share_decide": (_I32, [_ST, _P, _I32, _I32, _P, _P, _P, _P, _P, _I32, _F, _D, _P, _P, _P, _P, _P, _P]),
     "sp_build_mask": (_I32, [_ST, _P, _P, _P, _P, _P, _P, _I32, _I32, _P, _P]),
-    "sp_queryaware_select_bf16": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _U32, _F, _P, _P, _P, _SZ, _P]),
+    "sp_queryaware_select_score": (_F, [_D, _I32]),
+    "sp_queryaware_select_bf16": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _U32, _D, _P, _P, _P, _SZ, _P]),
     "sp_cover_select_workspace_bytes": (_SZ, [_I32]),
     "sp_cover_select_global": (_I32, [_P, _P, _I32, _I32, _F, _P, _P, _SZ, _P]),
     "sp_attn_workspace_bytes": (_SZ, [_I64, _I32, _I32, _I32, _I32]),

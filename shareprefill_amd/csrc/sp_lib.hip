@@ -12,7 +12,7 @@ void sp_set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
-extern "C" int sp_version(void) { return 2; }
+extern "C" int sp_version(void) { return 3; }
 extern "C" const char* sp_arch(void) { return "gfx950"; }
 extern "C" const char* sp_last_error(void) { return g_sp_error; }
 

@@ -12,6 +12,8 @@
 //     three passes over the data building (count, mass) histograms over 11/11/10 key bits;
 //   * rank sort for short vectors (rows of length nb): rank by pairwise comparison in LDS, scatter to
 //     sorted order, integer prefix scan -- a literal sort / cumsum / threshold.
+#include <cstring>
+
 #include "sp_common.h"
 
 #define SEL_THREADS 1024
@@ -1110,8 +1112,23 @@ __global__ __launch_bounds__(DEC_THREADS) void sp_share_keep_kernel(
           st.cols + (int64_t)c * nb, st.dists + (int64_t)c * nb, DEC_THREADS);
 }
 
+// The struct a kernel receives by value.  A caller built against the first layout of the struct (it ended with
+// `accum`; struct_bytes 0 or SP_CLUSTER_STATE_V1_BYTES) has no avg_map member: nothing behind `accum` is read.
+static sp_cluster_state state_by_value(const sp_cluster_state* st) {
+  sp_cluster_state v;
+  memset(&v, 0, sizeof v);
+  const bool full = st->struct_bytes >= (int32_t)sizeof(sp_cluster_state);
+  memcpy(&v, st, full ? sizeof v : (size_t)SP_CLUSTER_STATE_V1_BYTES);
+  if (!full) v.avg_map = nullptr;
+  return v;
+}
+
 static int check_state(const sp_cluster_state* st, int nb, const char* who) {
   SP_REQUIRE(st != nullptr, SP_ERR_INVALID_ARGUMENT, "%s: null cluster state", who);
+  SP_REQUIRE(st->struct_bytes == 0 || st->struct_bytes == (int32_t)SP_CLUSTER_STATE_V1_BYTES ||
+                 st->struct_bytes >= (int32_t)sizeof(sp_cluster_state),
+             SP_ERR_INVALID_ARGUMENT, "%s: cluster state struct_bytes=%d is neither 0, %d nor >= %d", who,
+             st->struct_bytes, (int)SP_CLUSTER_STATE_V1_BYTES, (int)sizeof(sp_cluster_state));
   SP_REQUIRE(st->n_clusters >= 0 && st->nb == nb && st->nbw == (nb + 63) / 64, SP_ERR_INVALID_ARGUMENT,
              "%s: cluster state sized for nb=%d, call uses nb=%d", who, st->nb, nb);
   if (st->n_clusters > 0) {
@@ -1136,14 +1153,14 @@ extern "C" int sp_share_decide(const sp_cluster_state* state, const int32_t* hea
              DEC_MAX_HEADS);
   SP_REQUIRE(state->nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_share_decide: nb=%d exceeds %d", state->nb, RS_MAX);
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_share_similarity_kernel, dim3(hq), dim3(2 * SP_WAVE), 0, s, *state, head_cluster, vert_blk,
+  hipLaunchKernelGGL(sp_share_similarity_kernel, dim3(hq), dim3(2 * SP_WAVE), 0, s, state_by_value(state), head_cluster, vert_blk,
                      slash_blk, use_qa, js_v, js_s);
   SP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sp_share_decide_kernel, dim3(1), dim3(DEC_MAX_HEADS), 0, s, *state, head_cluster, layer_idx, hq, use_qa,
+  hipLaunchKernelGGL(sp_share_decide_kernel, dim3(1), dim3(DEC_MAX_HEADS), 0, s, state_by_value(state), head_cluster, layer_idx, hq, use_qa,
                      nv, ns, min_blocks, similarity_threshold, fallback_threshold, decision, js_v, js_s, nv_final,
                      ns_final);
   SP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sp_share_keep_kernel, dim3(hq), dim3(DEC_THREADS), 0, s, *state, head_cluster, layer_idx, vert_blk,
+  hipLaunchKernelGGL(sp_share_keep_kernel, dim3(hq), dim3(DEC_THREADS), 0, s, state_by_value(state), head_cluster, layer_idx, vert_blk,
                      slash_blk, decision, nv, ns);
   SP_LAUNCH_CHECK();
   return SP_OK;
@@ -1221,9 +1238,8 @@ extern "C" int sp_build_mask(const sp_cluster_state* state, const int32_t* head_
              SP_ERR_INVALID_ARGUMENT, "sp_build_mask: null pointer");
   SP_REQUIRE(hq > 0 && nb > 0 && nb <= RS_MAX, SP_ERR_UNSUPPORTED, "sp_build_mask: nb=%d unsupported (max %d)", nb,
              RS_MAX);
-  hipLaunchKernelGGL(sp_build_mask_kernel, dim3(hq, MASK_SPLIT), dim3(MASK_THREADS), 0, (hipStream_t)stream, *state,
-                     head_cluster,
-                     decision, vert_blk, slash_blk, nv_final, ns_final, nb, (nb + 63) / 64, mask);
+  hipLaunchKernelGGL(sp_build_mask_kernel, dim3(hq, MASK_SPLIT), dim3(MASK_THREADS), 0, (hipStream_t)stream,
+                     state_by_value(state), head_cluster, decision, vert_blk, slash_blk, nv_final, ns_final, nb, (nb + 63) / 64, mask);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
@@ -1295,8 +1311,17 @@ __global__ __launch_bounds__(BP_THREADS) void sp_block_probs_kernel(
   for (int b = threadIdx.x; b < nb; b += BP_THREADS) out[b] = (b <= r) ? logit[b] / gsum : 0.f;
 }
 
+// score = pattern_threshold * nb: the product of the caller's DOUBLE threshold and the block count, evaluated in
+// double as Python evaluates it (attention_sharing.py:361), then taken to fp32 as the comparison with an fp32
+// tensor takes it (utils.py:56).  A threshold that had been rounded to fp32 first would give a score one fp32 ulp
+// away for about a fifth of the block counts.
+extern "C" float sp_queryaware_select_score(double pattern_threshold, int32_t nb) {
+  volatile double product = pattern_threshold * (double)nb;  // one rounding to double, then one to float
+  return (float)product;
+}
+
 extern "C" int sp_queryaware_select_bf16(const void* qbar, const void* kbar, const int32_t* decision, int32_t hq,
-                                         int32_t hkv, int32_t d, int32_t nb, uint32_t flags, float pattern_threshold,
+                                         int32_t hkv, int32_t d, int32_t nb, uint32_t flags, double pattern_threshold,
                                          float* probs, uint64_t* mask, void* workspace, size_t workspace_bytes,
                                          sp_stream_t stream) {
   SP_REQUIRE(qbar && kbar && decision && probs && mask, SP_ERR_INVALID_ARGUMENT,
@@ -1314,8 +1339,7 @@ extern "C" int sp_queryaware_select_bf16(const void* qbar, const void* kbar, con
                        sp_inv_sqrt_dim(flags, d), probs);
     SP_LAUNCH_CHECK();
   }
-  // score = pattern_threshold * nb evaluated in double, then taken to fp32 as a tensor comparison would
-  const float score = (float)((double)pattern_threshold * (double)nb);
+  const float score = sp_queryaware_select_score(pattern_threshold, nb);
   return gsel_run(probs, decision, SP_DEC_QA, hq, nb, score, mask, workspace, workspace_bytes, (hipStream_t)stream,
                   "sp_queryaware_select_bf16");
 }
@@ -1336,8 +1360,8 @@ struct PivotRowShared {
 __global__ __launch_bounds__(RS_THREADS) void sp_pivot_rows_kernel(sp_cluster_state st,
                                                                    const int32_t* __restrict__ head_cluster,
                                                                    const int32_t* __restrict__ decision,
-                                                                   const float* __restrict__ avg_attn, int nb,
-                                                                   int nbw, long long t_lt,
+                                                                   const float* __restrict__ avg_attn, int hq,
+                                                                   int nb, int nbw, long long t_lt,
                                                                    unsigned long long* __restrict__ accum) {
   __shared__ PivotRowShared sh;
   extern __shared__ __attribute__((aligned(16))) char rs_lds[];
@@ -1346,6 +1370,14 @@ __global__ __launch_bounds__(RS_THREADS) void sp_pivot_rows_kernel(sp_cluster_st
   if (decision[h] != SP_DEC_DENSE) return;
   const int c = head_cluster[h];
   if (!sp_slot_ok(st, c)) return;  // a dense head outside every shared cluster keeps no pattern
+  // One head per cluster and call: the election flags one, but a caller's own flags may name several heads of a
+  // cluster.  The reference stores them one after the other, so the highest head's map is what stays
+  // (attention_sharing.py:96-103); here the lower ones leave, or their rows would share the cluster's row counter
+  // and accumulators with the highest head's.
+  bool later = false;
+  for (int h2 = h + 1 + threadIdx.x; h2 < hq; h2 += RS_THREADS)
+    later = later || (decision[h2] == SP_DEC_DENSE && head_cluster[h2] == c);
+  if (__syncthreads_or(later ? 1 : 0)) return;
   const float* row = avg_attn + ((int64_t)h * nb + r) * nb;
   const int keep = rs_row_keep(row, nb, t_lt, rsh);
   uint32_t* prow = reinterpret_cast<uint32_t*>(st.pattern + ((int64_t)c * nb + r) * nbw);
@@ -1426,8 +1458,8 @@ extern "C" int sp_pivot_update(const sp_cluster_state* state, const int32_t* hea
   if (state->n_clusters == 0) return SP_OK;
   unsigned long long* accum = reinterpret_cast<unsigned long long*>(state->accum);
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(sp_pivot_rows_kernel, dim3(nb, hq), dim3(RS_THREADS), rs_lds_bytes(nb), s, *state, head_cluster, decision,
-                     avg_attn, nb, (nb + 63) / 64, (long long)sp_thr_lt(pattern_threshold), accum);
+  hipLaunchKernelGGL(sp_pivot_rows_kernel, dim3(nb, hq), dim3(RS_THREADS), rs_lds_bytes(nb), s, state_by_value(state), head_cluster, decision,
+                     avg_attn, hq, nb, (nb + 63) / 64, (long long)sp_thr_lt(pattern_threshold), accum);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

@@ -172,7 +172,7 @@ class ClusterState:
         self.dists = torch.zeros(c, nb, dtype=torch.uint8, device=device)
         self.pattern = torch.zeros(c, nb, self.nbw, dtype=torch.int64, device=device)
         self.accum = torch.zeros(c, 2, dtype=torch.int64, device=device)
-        self.struct = ClusterStateStruct(n_clusters, nb, self.nbw, 0, self.info.data_ptr(), self.ratio.data_ptr(),
+        self.struct = ClusterStateStruct(n_clusters, nb, self.nbw, C.sizeof(ClusterStateStruct), self.info.data_ptr(), self.ratio.data_ptr(),
                                          self.vert.data_ptr(), self.slash.data_ptr(), self.cols.data_ptr(),
                                          self.dists.data_ptr(), self.pattern.data_ptr(), self.accum.data_ptr(),
                                          self.avg_map.data_ptr() if keep_maps else None)
@@ -182,6 +182,7 @@ class ClusterState:
         """No pivot, no pattern (attention_sharing.py:41-78); enqueued on the current stream."""
         self.info.zero_()
         self.info[:, 0] = -1
+        self.accum.zero_()  # (zero between completed pivot updates anyway; a reset must not depend on that)
 
     def ref(self):
         return C.byref(self.struct)

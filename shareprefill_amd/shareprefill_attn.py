@@ -173,10 +173,12 @@ def shareprefill_attention_core(module, query_states: torch.Tensor, key_states: 
     nb = -(-q_len // block_size)
     sharing = module.attention_sharing
     minb, maxb = budget_blocks(config.min_budget, config.max_budget, block_size)
-    if q_len < block_size or (nb <= minb and getattr(config, "dense_short_prompts", True)):
+    if q_len < block_size or (nb <= minb and nb <= maxb and getattr(config, "dense_short_prompts", True)):
         # (a) Shorter than one block: a single diagonal block, nothing to select (the reference cannot run here).
-        # (b) The prompt has no more blocks than the minimum budget.  Every head's budgets are then clamped to nb
-        # (attention_sharing.py:173-176: raised to min_budget, cut to min(max_budget, nb)), its vertical-slash set is
+        # (b) The prompt has no more blocks than the minimum budget, nor than the maximum.  Every head's budgets are
+        # then raised to min_budget and cut to min(max_budget, nb) = nb (attention_sharing.py:173-176; with a maximum
+        # BELOW nb the cut leaves max_budget columns and distances, a sparse mask, so that case takes the full path),
+        # its vertical-slash set is
         # every column and every distance, and whatever the head's decision (pivot, shared, query-aware, fallback) its
         # mask is the whole lower triangle -- in this layer and, with the same prompt, in every later one.  Nothing the
         # selection computes can change an output, so it is skipped and the attention runs on the dense mask: the

@@ -38,7 +38,9 @@ class FakeAttention:
 
 
 def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_free=True, with_forced=True, d=128,
-               shared=None, **thr):
+               shared=None, table=None, layer_ids=None, reseed=False, **thr):
+    """table: a cluster table to use instead of a random one; layer_ids: the layer indices to run, in order (default
+    0 .. n_layers - 1); reseed: draw new q / k / v for every layer (seed + layer index) instead of one set."""
     from shareprefill_amd import AttentionSharing, shareprefill_attention_forward, ops
 
     # dense_short_prompts off: these tests compare the selection itself, also where the prompt is so short that every
@@ -46,7 +48,8 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_fre
     kw = dict(block_size=128, min_budget=1024, max_budget=None, pattern_threshold=0.95, similarity_threshold=0.5,
               fallback_threshold=0.9, queryaware_threshold=0.1, dense_short_prompts=False)
     kw.update(thr)
-    table = synthetic.random_cluster_table(hq, n_clusters, n_layers, seed)
+    if table is None:
+        table = synthetic.random_cluster_table(hq, n_clusters, n_layers, seed)
     if shared is not None:  # only these clusters share (the shipped Llama table shares one of its 44)
         table["shared_clusters"] = list(shared)
     path = synthetic.write_cluster_table(table, str(tmp_path / "table.json"))
@@ -59,7 +62,10 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_fre
     qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
     nb = -(-n // 128)
     results = []
-    for layer in range(n_layers):
+    for layer in (range(n_layers) if layer_ids is None else layer_ids):
+        if reseed:
+            q, k, v = synthetic.planted_qkv(hq, hkv, n, d, seed + layer, q_head_gain=1.0)
+            qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
         mod = FakeAttention(cfg, sharing, layer, d, hq, hkv)
         out, avg = shareprefill_attention_forward(mod, qg, kg, vg, None, scaling=mod.scaling)
         plan = sharing.plans[-1]
@@ -83,7 +89,7 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_fre
             free = oracle_free.layer(q[0], k[0], v[0], layer, compute_attention=False, **okw)
             oracle_free.update_pivots(layer, free.decision, avg[0].cpu().numpy(), kw["pattern_threshold"])
         results.append(dict(layer=layer, out=out.cpu(), avg=avg.cpu(), plan=plan, mask=gpu_mask, dec=dec,
-                            forced=forced, free=free))
+                            forced=forced, free=free, q=q[0], k=k[0], v=v[0]))
     return dict(q=q[0], k=k[0], v=v[0], table=table, sharing=sharing, oracle_forced=oracle_forced,
                 oracle_free=oracle_free, layers=results, nb=nb, kw=kw, d=d)
 
@@ -154,8 +160,8 @@ def check_free(run, expect_same_masks=True):
 
 
 def check_outputs(run):
-    q, k, v = run["q"], run["k"], run["v"]
     for L in run["layers"]:
+        q, k, v = L["q"], L["k"], L["v"]
         want = L["dec"] == O.DEC_DENSE
         ref, avg_ref = O.masked_attention(q, k, v, L["mask"], 128, run["d"] ** -0.5, want_avg=want)
         out = L["out"][0].transpose(0, 1).float()
@@ -407,3 +413,104 @@ def test_forward_rejects_sliding_window_and_handles_short_and_decode(gpu_device,
     out1, w1 = shareprefill_attention_forward(mod, q[:, :, -1:], k, v, None, scaling=1.0)  # decode step
     assert w1 is None and out1.shape == (1, 1, 4, 128)
     assert (out1[0, 0].float() - ref[0, :, -1].float()).abs().max().item() <= MAX_ABS
+
+
+@pytest.mark.parametrize("nb,thr", [(13, 0.95), (21, 0.95), (37, 0.95), (12, 0.9), (23, 0.9), (14, 0.99), (29, 0.99)])
+def test_layer_all_query_aware_at_block_counts_where_a_float_threshold_would_differ(gpu_device, tmp_path, nb, thr):
+    """Block counts at which fp32(double(pattern_threshold) * nb), the score the reference's query-aware selection
+    compares with (attention_sharing.py:361), differs from what a threshold rounded to fp32 first would give (never the
+    case for powers of two, which every other test of this path uses).  queryaware_threshold 10 sends every head down
+    the query-aware path; the forced comparison holds the masks to the oracle's, which forms the score from the
+    Python float."""
+    assert np.float32(thr * nb) != np.float32(float(np.float32(thr)) * nb)
+    run = run_layers(gpu_device, tmp_path, hq=8, hkv=2, n=nb * 128, seed=nb, n_clusters=2, min_budget=256,
+                     pattern_threshold=thr, fallback_threshold=1e9, queryaware_threshold=10.0)
+    assert all((L["dec"] == O.DEC_QA).all() for L in run["layers"])
+    check_forced(run)
+    check_free(run, expect_same_masks=False)
+    check_outputs(run)
+
+
+def test_short_prompt_shortcut_needs_the_maximum_budget_to_reach_the_prompt_too(gpu_device, tmp_path):
+    """min_budget 2048 tokens (16 blocks) above max_budget 1024 (8 blocks) on a prompt of 12 blocks: the budgets are
+    raised to 16 and then cut to 8 (attention_sharing.py:173-176), so vertical-slash and fallback heads keep 8 of 12
+    columns and distances -- a sparse mask, although the prompt has no more blocks than the minimum budget.  The
+    dense short-prompt shortcut must not be taken: with it enabled the layer gives the full path's decisions, masks
+    (the oracle's) and output bits."""
+    from shareprefill_amd import shareprefill_attention_forward
+
+    kw = dict(hq=8, hkv=2, n=1500, seed=91, n_clusters=2, min_budget=2048, max_budget=1024, fallback_threshold=1e9)
+    full = run_layers(gpu_device, tmp_path, **kw)
+    check_forced(full)
+    check_outputs(full)
+    tri = np.tril(np.ones((12, 12), dtype=bool))
+    assert any(not np.array_equal(L["mask"][h], tri) for L in full["layers"] for h in range(8)), "masks must be sparse"
+    from shareprefill_amd import AttentionSharing
+
+    fast = full
+    sharing = AttentionSharing(synthetic.write_cluster_table(full["table"], str(tmp_path / "same_table.json")))
+    cfg = types.SimpleNamespace(**{**fast["kw"], "dense_short_prompts": True})
+    q, k, v = (fast[x][None].to(gpu_device) for x in ("q", "k", "v"))
+    for layer in range(2):
+        out, avg = shareprefill_attention_forward(FakeAttention(cfg, sharing, layer, 128, 8, 2), q, k, v, None,
+                                                  scaling=128 ** -0.5)
+        assert torch.equal(out.cpu(), full["layers"][layer]["out"]), f"layer {layer}"
+        assert torch.equal(avg.cpu(), full["layers"][layer]["avg"])
+    assert len(sharing.plans) == 2 and sharing.dense_layers == 0
+    # with the maximum at or above the prompt the shortcut is taken again
+    cfg_ok = types.SimpleNamespace(**{**fast["kw"], "dense_short_prompts": True, "max_budget": 1536})
+    sharing.reset_state()
+    shareprefill_attention_forward(FakeAttention(cfg_ok, sharing, 0, 128, 8, 2), q, k, v, None, scaling=128 ** -0.5)
+    assert sharing.plans == [] and sharing.dense_layers == 1
+
+
+def test_layers_of_the_shipped_llama_table_elect_and_reuse_the_pivot_of_its_one_shared_cluster(gpu_device, tmp_path):
+    """The table the reference ships for Llama-3.1-8B-Instruct: 44 clusters over 32 layers x 32 heads of which ONE
+    ("9": 42 heads in layers 14 to 30) is shared (attention_sharing.py:204-295 only ever look at shared clusters).
+    Layers 14, 15, 17, 22 and 30 run with the layer indices of the table on 8192 planted tokens, new q / k / v per
+    layer: the pivot is elected at the cluster's first layer (14, head 17), a layer without members (15) changes
+    nothing, the members of layers 17, 22 (nine of them in one layer) and 30 -- sixteen layers after the election --
+    take the share test against that pivot's stored vectors and reuse its pattern; every head outside the cluster
+    stays on the vertical-slash path.  Decisions, budgets, masks, the pivot's pattern, map and coverage ratio are the
+    oracle's (forced comparison); outputs against the fp32 masked attention for the last layer."""
+    import json
+
+    from shareprefill_amd import SharePrefillConfig, ops
+
+    path = SharePrefillConfig(model_name="Llama-3.1-8B-Instruct").sharing_lookup_path
+    with open(path) as f:
+        table = json.load(f)
+    members = {}
+    for layer, head in table["clusters"]["9"]:
+        members.setdefault(layer, []).append(head)
+    assert table["shared_clusters"] == ["9"] and min(members) == 14 and members[14] == [17] and 15 not in members
+    layer_ids = [14, 15, 17, 22, 30]
+    run = run_layers(gpu_device, tmp_path, hq=32, hkv=8, n=8192, seed=400, n_clusters=0, table=table,
+                     layer_ids=layer_ids, reseed=True, with_free=False, fallback_threshold=1e9)
+    sharing = run["sharing"]
+    assert len(sharing._slot) == 1 and sharing.max_pivots(14, 32) == 1 and sharing.max_pivots(15, 32) == 0
+    check_forced(run)
+    by_layer = {L["layer"]: L for L in run["layers"]}
+    assert np.nonzero(by_layer[14]["dec"] == O.DEC_DENSE)[0].tolist() == [17]
+    summary = sharing.pivot_summary()["9"]
+    assert summary["pivot_head"] == 17 and summary["layer"] == 14 and summary["has_pattern"]
+    shared_heads = 0
+    for layer in layer_ids[1:]:
+        dec = by_layer[layer]["dec"]
+        assert not (dec == O.DEC_DENSE).any()
+        share = set(np.nonzero(dec == O.DEC_SHARE)[0].tolist())
+        assert share <= set(members.get(layer, []))
+        shared_heads += len(share)
+        # a shared head's mask holds the pivot's pattern
+        pat = ops.mask_to_bool(sharing._state.pattern[0], run["nb"]).cpu().numpy()
+        for h in share:
+            assert (by_layer[layer]["mask"][h] & pat == pat).all()
+    assert not (by_layer[15]["dec"] == O.DEC_SHARE).any()
+    assert len(set(np.nonzero(by_layer[22]["dec"] == O.DEC_SHARE)[0].tolist())) >= 2, "several members in one layer"
+    assert (by_layer[30]["dec"] == O.DEC_SHARE).tolist().count(True) == 1 and by_layer[30]["dec"][21] == O.DEC_SHARE
+    assert shared_heads >= 4
+    L = by_layer[30]  # heads 20 .. 23 = the group of kv head 5, with the shared head 21 among them
+    ref, _ = O.masked_attention(L["q"][20:24], L["k"][5:6], L["v"][5:6], L["mask"][20:24], 128, 128 ** -0.5)
+    out = L["out"][0].transpose(0, 1)[20:24].float()
+    assert (out - ref).abs().max().item() <= MAX_ABS
+    assert ((out - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL

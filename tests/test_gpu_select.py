@@ -224,3 +224,101 @@ def test_heads_without_a_cluster_slot_never_touch_the_state(gpu_device):
     assert state.info[:, 1].cpu().tolist() == [1, 1]
     for k, v in bufs.items():
         assert torch.equal(v[0], before[k][0]) and torch.equal(v[-1], before[k][-1]), f"canary of {k} overwritten"
+
+
+def _straddling_threshold(probs: np.ndarray, nb: int):
+    """A double threshold pt for which the score fp32(pt * nb) that the reference forms (attention_sharing.py:361,
+    utils.py:56) and the score fp32(fp32(pt) * nb) that a float argument would give lie on the two sides of one of
+    the running sums of `probs`, so the two scores select different sets.  Returns (pt, kept right, kept wrong)."""
+    order = O.order_desc(probs)
+    sums = np.cumsum(O.to_fixed(probs[order]), dtype=np.uint64)
+    nonzero = int((probs > 0).sum())  # entries above the diagonal are exact zeros: they sort last and add nothing
+    for m in range(nonzero // 3, nonzero - 1):
+        s = int(sums[m]) / float(2 ** 48)
+        lo = np.float32(s)
+        if float(lo) > s:
+            lo = np.nextafter(lo, np.float32(0))
+        hi = np.nextafter(lo, np.float32(np.inf))
+        for u in np.linspace(0.30, 0.70, 161):
+            pt = (float(lo) + u * (float(hi) - float(lo))) / nb
+            right, wrong = np.float32(pt * nb), np.float32(float(np.float32(pt)) * nb)
+            if right != wrong and {float(right), float(wrong)} == {float(lo), float(hi)}:
+                kr, kw = O.prefix_len(probs, O.thr_le(float(right))), O.prefix_len(probs, O.thr_le(float(wrong)))
+                if kr != kw and 0.3 < pt < 1.0:
+                    return pt, kr, kw
+    raise AssertionError("no straddling threshold found")
+
+
+@pytest.mark.parametrize("nb", [13, 21, 100])
+def test_queryaware_select_compares_with_the_double_product_score(gpu_device, nb):
+    """The query-aware selection's score is fp32(double(pattern_threshold) * nb).  The thresholds here are chosen, per
+    head, so that one running sum of the head's own block probabilities lies between that score and the one a
+    threshold rounded to fp32 first would give (one fp32 ulp apart): the selection must keep exactly the entries the
+    oracle keeps with the reference's score, and the negative control shows that the other score keeps a different
+    number of entries."""
+    from shareprefill_amd import _lib, ops
+
+    hq, hkv, d = 4, 2, 128
+    g = torch.Generator().manual_seed(1000 + nb)
+    qbar = (torch.randn(nb, hq, d, generator=g) * 1.5).to(torch.bfloat16).to(gpu_device)
+    kbar = (torch.randn(nb, hkv, d, generator=g) * 1.5).to(torch.bfloat16).to(gpu_device)
+    tri = np.tril(np.ones((nb, nb), dtype=bool))
+    all_qa = torch.full((hq,), _lib.SP_DEC_QA, dtype=torch.int32, device=gpu_device)
+    mask0 = torch.zeros(hq, nb, (nb + 63) // 64, dtype=torch.int64, device=gpu_device)
+    probs = ops.queryaware_select(qbar, kbar, all_qa, mask0, 0.9).cpu().numpy()   # the probabilities do not depend on it
+    for h in range(hq):
+        ph = probs[h].reshape(-1)
+        pt, kept_right, kept_wrong = _straddling_threshold(ph, nb)
+        assert kept_right != kept_wrong
+        only = torch.zeros(hq, dtype=torch.int32, device=gpu_device)
+        only[h] = _lib.SP_DEC_QA
+        mask = torch.zeros(hq, nb, (nb + 63) // 64, dtype=torch.int64, device=gpu_device)
+        ops.queryaware_select(qbar, kbar, only, mask, pt)
+        got = ops.mask_to_bool(mask, nb).cpu().numpy()
+        want = np.zeros(nb * nb, dtype=bool)
+        want[O.cover_keep_le(ph, pt * nb)] = True
+        want = want.reshape(nb, nb) & tri
+        want[0, 0] = True
+        assert np.array_equal(got[h], want), f"head {h}, threshold {pt!r}"
+        assert not got[[x for x in range(hq) if x != h]].any()
+        other = np.zeros(nb * nb, dtype=bool)
+        other[O.cover_keep_le(ph, float(np.float32(float(np.float32(pt)) * nb)))] = True
+        other = other.reshape(nb, nb) & tri
+        other[0, 0] = True
+        assert not np.array_equal(other, want), "negative control: the fp32-rounded threshold must select another set"
+
+
+def test_pivot_update_with_several_dense_heads_of_one_cluster_keeps_the_highest(gpu_device):
+    """A caller's own flags may mark several heads of one cluster dense.  The reference stores their maps one after
+    the other (attention_sharing.py:96-103), so the highest head's stays; here the rows of the lower heads leave
+    at once instead of sharing the cluster's row counter and accumulators.  The state after the call is exactly that
+    of a call with the highest head alone, and counter and accumulators are zero again."""
+    from shareprefill_amd import ops
+
+    hq, nb = 6, 48
+    g = torch.Generator().manual_seed(23)
+    tri = torch.tril(torch.ones(nb, nb, dtype=torch.bool))
+    avg = torch.softmax((torch.randn(hq, nb, nb, generator=g) * 2).masked_fill(~tri, float("-inf")), -1)
+    avg = avg.to(gpu_device).contiguous()
+    hc = torch.tensor([0, 0, 1, 0, -1, 1], dtype=torch.int32, device=gpu_device)
+
+    def run(decision):
+        state = ops.ClusterState(2, nb, gpu_device, keep_maps=True)
+        state.info[0, 0], state.info[1, 0] = 3, 5
+        state.cols[:, :3] = 1
+        state.dists[:, :2] = 1
+        ops.pivot_update(state, hc, torch.tensor(decision, dtype=torch.int32, device=gpu_device), avg, 0.9)
+        torch.cuda.synchronize()
+        return state
+
+    many = run([1, 1, 1, 1, 1, 1])
+    last = run([0, 0, 0, 1, 0, 1])
+    for name in ("info", "ratio", "pattern", "accum", "avg_map"):
+        assert torch.equal(getattr(many, name), getattr(last, name)), name
+    assert many.info[:, 1].cpu().tolist() == [1, 1] and many.info[:, 5].cpu().tolist() == [0, 0]
+    assert int(many.accum.abs().sum()) == 0
+    for slot, h in ((0, 3), (1, 5)):
+        want = O.cover_keep_rows_ge(avg[h].cpu().numpy(), 0.9) & tri.numpy()
+        want[0, 0] = True
+        assert np.array_equal(ops.mask_to_bool(many.pattern[slot], nb).cpu().numpy(), want)
+        assert torch.equal(many.avg_map[slot], avg[h])

@@ -64,6 +64,48 @@ def test_cluster_state_struct_matches_header_layout():
     assert names == [f[0] for f in ClusterStateStruct._fields_]
 
 
+def test_cluster_state_struct_size_guards_the_members_added_later():
+    """struct_bytes tells the library which layout the caller was compiled against: the first one ended with `accum`
+    (80 bytes), so avg_map is read only from a struct that declares itself long enough; any other size is refused
+    (argument checks run on the host, before any GPU call)."""
+    from shareprefill_amd import _lib
+    from shareprefill_amd._lib import ClusterStateStruct
+
+    lib = _lib.load()
+    assert ctypes.sizeof(ClusterStateStruct) == 88
+    header = open(HEADER).read()
+    assert "#define SP_CLUSTER_STATE_V1_BYTES 80" in header
+    one = ctypes.c_void_p(16)  # never dereferenced: the calls below fail their checks before any launch
+    for size, ok in ((0, True), (80, True), (88, True), (96, True), (84, False), (40, False), (-1, False)):
+        st = ClusterStateStruct(1, 4, 1, size, one, one, one, one, one, one, one, one, None)
+        rc = lib.sp_pivot_update(ctypes.byref(st), None, None, None, 1, 4, 0.9, None)
+        msg = lib.sp_last_error()
+        assert rc == -1
+        assert (b"struct_bytes" not in msg) == ok, (size, msg)
+
+
+def test_queryaware_selection_score_is_the_double_product_taken_to_fp32():
+    """attention_sharing.py:361 forms pattern_threshold * num_blocks from the Python float (double) and utils.py:56
+    compares the fp32 running sums with it, i.e. with fp32(double(pt) * nb).  The entry point takes the threshold as a
+    double and must form exactly that value -- for every block count the kernels accept.  Rounding the threshold to
+    fp32 first (what a `float` argument does) gives another value for hundreds of block counts: the negative control."""
+    import numpy as np
+
+    from shareprefill_amd import _lib
+
+    lib = _lib.load()
+    for pt in (0.5, 0.9, 0.95, 0.99, 0.999, 0.1, 1.0 / 3.0):
+        differs_when_rounded_first = 0
+        for nb in range(1, 4097):
+            want = float(np.float32(pt * nb))
+            assert lib.sp_queryaware_select_score(pt, nb) == want, (pt, nb)
+            differs_when_rounded_first += float(np.float32(float(np.float32(pt)) * nb)) != want
+        if pt in (0.9, 0.95, 0.99):
+            assert differs_when_rounded_first > 400  # 1326 / 818 / 497 of 4096
+    # the binding hands the Python float over unrounded
+    assert _lib.SIGNATURES["sp_queryaware_select_bf16"][1][8] is ctypes.c_double
+
+
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     from shareprefill_amd import _lib
 
