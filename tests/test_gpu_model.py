@@ -194,3 +194,60 @@ def test_llama31_8b_architecture_at_131072_tokens(gpu_device):
         stock = getattr(modeling_llama.apply_rotary_pos_emb, "_shareprefill_original", None)
         if stock is not None:
             modeling_llama.apply_rotary_pos_emb = stock
+
+
+def test_llama31_8b_architecture_all_32_layers_at_131072_tokens(gpu_device):
+    """The end-to-end configuration as stated: the whole Llama-3.1-8B architecture (32 layers, hidden 4096, Hq32 Hkv8,
+    head_dim 128, intermediate 14336, RoPE theta 5e5, vocab 128256, random-init bf16, 16 GB of weights), 131072
+    uniform-random token ids, SharePrefill in every layer with the shipped Llama-3.1-8B-Instruct table (44 clusters,
+    one shared, its members in layers 14 to 30) and the thresholds of the reference's latency script
+    (eval/efficiency/run_latency.sh:12).  One prefill forward: finite last-token logits, all 32 x 32 heads decided,
+    every layer's block density within (0, 1], and a second forward (state reset in between) gives the same logits
+    bit for bit."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from shareprefill_amd import SharePrefill
+
+    n = 131072
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, vocab_size=128256, max_position_embeddings=n,
+                      rope_parameters={"rope_type": "default", "rope_theta": 500000.0}, rms_norm_eps=1e-5,
+                      tie_word_embeddings=False)
+    torch.manual_seed(1238)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(gpu_device):
+            model = LlamaForCausalLM(cfg)
+    finally:
+        torch.set_default_dtype(old)
+    model.eval()
+    gen = torch.Generator(device=gpu_device).manual_seed(1238)
+    ids = torch.randint(0, cfg.vocab_size, (1, n), generator=gen, device=gpu_device)
+    SharePrefill(model_name="meta-llama/Llama-3.1-8B-Instruct", pattern_threshold=0.95, similarity_threshold=0.5,
+                 fallback_threshold=0.95, block_size=128, min_budget=1024)(model)
+    sharing = model.attention_sharing
+    assert len(sharing.clusters) == 44 and len(sharing._slot) == 1
+    sharing.keep_plans = True
+    print("C4 test: 32-layer patched forward", flush=True)
+    with torch.no_grad():
+        out = model(ids, use_cache=False, logits_to_keep=1).logits.float()
+    assert out.shape == (1, 1, cfg.vocab_size) and torch.isfinite(out).all()
+    assert [p.layer_idx for p in sharing.plans] == list(range(32))
+    hist = sharing.decision_histogram()
+    assert sum(hist.values()) == 1024
+    for p in sharing.plans:
+        d = p.density().cpu()
+        assert d.shape == (32,) and (d > 0).all() and (d <= 1).all()
+        assert int(p.decision.min()) >= 0 and int(p.decision.max()) <= 3
+    # heads outside the one shared cluster can neither become pivots nor share
+    members = {(l, h) for l, h in sharing.clusters["9"]}
+    for p in sharing.plans:
+        for h in torch.nonzero((p.decision == 1) | (p.decision == 2)).reshape(-1).cpu().tolist():
+            assert (p.layer_idx, h) in members
+    print("C4 test: second forward", flush=True)
+    sharing.keep_plans = False
+    with torch.no_grad():
+        out2 = model(ids, use_cache=False, logits_to_keep=1).logits.float()
+    assert torch.equal(out, out2)
+    assert len(sharing.plans) == 32
