@@ -219,6 +219,23 @@ def c4_line(args):
                        "fuse_rope": bool(args.fuse_rope)},
             "tokens_per_s": round(args.seq_len / sec, 1), "mean_block_density": round(dens, 4),
             "decisions": sharing.decision_histogram(), "finite_logits": bool(torch.isfinite(out).all())}
+    if getattr(args, "both_rope", False):
+        # the same model and prompt with the other rotary-embedding setting (the fused one-pass kernel is bit-identical
+        # to the model's elementwise evaluation): 1 warm-up + the same number of timed forwards
+        from shareprefill_amd import unpatch_model
+
+        unpatch_model(model)
+        model = SharePrefill(model_name="meta-llama/Llama-3.1-8B-Instruct", pattern_threshold=0.95,
+                             similarity_threshold=0.5, fallback_threshold=0.95, block_size=128, min_budget=1024,
+                             fuse_rope=not args.fuse_rope)(model)
+        fwd()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fwd()
+        torch.cuda.synchronize()
+        line["other_rope_setting"] = {"fuse_rope": not args.fuse_rope, "value": round((time.perf_counter() - t0) / steps, 3),
+                                      "unit": "s", "steps": steps, "warmup": 1}
     if args.length_sweep:
         # the reference's latency protocol (eval/efficiency/latency.py:21-108): same model, growing prompts,
         # sparse path against the stock dense causal attention
@@ -349,6 +366,65 @@ def sharing_layer_variant(args, w, pt, q, k, v, table):
     stage["pivot_update_layer0_pivots"] = event_ms(lambda: ops.pivot_update(state, hc0, plan0.decision, avg0[0], pt))
     out["stage_ms"] = {a: round(b, 3) for a, b in stage.items()}
     out["n_pivots_layer0"] = int((plan0.decision == _lib.SP_DEC_DENSE).sum())
+    return out
+
+
+def timed_layer_point(w, q, k, v, table, pt, steps=5, n_tokens=None, with_stages=False):
+    """Layer 0 once (pivot election), one warm-up and `steps` timed calls of layer 1 at pattern_threshold pt on the
+    workload's inputs (cut to their first n_tokens tokens when given): kept blocks, layer and attention-launch time,
+    fractions of the bf16 peak on kept blocks; with_stages adds the time of every stage outside the attention launch."""
+    import torch
+
+    from shareprefill_amd import AttentionSharing, ops, shareprefill_attention_forward, synthetic
+
+    if n_tokens is not None:
+        q, k, v = q[:, :, :n_tokens], k[:, :, :n_tokens], v[:, :, :n_tokens]
+    n = q.shape[2]
+    nb = -(-n // w.block_size)
+    tri = w.hq * nb * (nb + 1) // 2
+    scale = w.head_dim ** -0.5
+    with tempfile.TemporaryDirectory() as tmp:
+        sh = AttentionSharing(synthetic.write_cluster_table(table, os.path.join(tmp, "table.json")))
+    cfg = types.SimpleNamespace(block_size=w.block_size, min_budget=w.min_budget, max_budget=None, pattern_threshold=pt,
+                                similarity_threshold=w.similarity_threshold, fallback_threshold=w.fallback_threshold,
+                                queryaware_threshold=w.queryaware_threshold)
+
+    def run(layer):
+        mod = types.SimpleNamespace(config=cfg, attention_sharing=sh, layer_idx=layer, scaling=scale)
+        return shareprefill_attention_forward(mod, q, k, v, None, scaling=scale)
+
+    run(0)
+    run(1)
+    torch.cuda.synchronize()
+    tm = ops.KernelTimer()
+    ops.kernel_timer = tm
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run(1)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    ops.kernel_timer = None
+    ams = sum(tm.durations_ms("attn")) / steps
+    plan = sh.plans[-1]
+    kept = int(ops.mask_row_pointers(plan.mask)[:, -1].sum())
+    out = {"pattern_threshold": pt, "tokens": n, "kept_blocks": kept, "density": round(kept / tri, 4),
+           "layer_ms": round(ms, 3), "attn_ms": round(ams, 3),
+           "attn_tflops": round(kept * FLOP_PER_BLOCK / ams / 1e9, 1),
+           "attn_frac_of_peak": round(kept * FLOP_PER_BLOCK / ams / 1e9 / PEAK_BF16_TFLOPS, 4),
+           "layer_frac_of_peak": round(kept * FLOP_PER_BLOCK / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    if with_stages:
+        qh, kh, vh = q[0], k[0], v[0]
+        minb = math.ceil(w.min_budget / w.block_size)
+        st = {}
+        st["lastq_scores"] = event_ms(lambda: ops.lastq_scores(qh, kh, w.block_size))
+        vt, st_, vb, sb = ops.lastq_scores(qh, kh, w.block_size)
+        st["cover_budgets"] = event_ms(lambda: ops.cover_budgets(vt, st_, w.block_size, pt, minb, nb))
+        st["pool_k"] = event_ms(lambda: ops.pool_avg(kh, w.block_size))
+        kbar = ops.pool_avg(kh, w.block_size)
+        st["queryaware_test"] = event_ms(lambda: ops.queryaware_test(qh, kbar, vb, w.block_size, w.queryaware_threshold))
+        st["attention_launch"] = ams
+        st["everything_else"] = max(0.0, ms - sum(st.values()))
+        out["stage_ms"] = {a: round(b, 3) for a, b in st.items()}
     return out
 
 
@@ -562,6 +638,22 @@ def main():
                               "attn_frac_of_peak": round(kb * FLOP_PER_BLOCK / ams / 1e9 / PEAK_BF16_TFLOPS, 4),
                               "layer_frac_of_peak": round(kb * FLOP_PER_BLOCK / ms / 1e9 / PEAK_BF16_TFLOPS, 4)})
             line["threshold_sweep"] = sweep
+            # The regime the method exists for: the reference's minimum mask is 8 vertical + 8 slash blocks per row
+            # (attention_sharing.py:169-176), which a pattern_threshold near zero leaves alone (every budget clamps to
+            # min_budget); 0.65 gives about a tenth of the blocks with this generator.  Same layer, same inputs.
+            line["low_density"] = [timed_layer_point(w, q, k, v, table, thr, steps=5, with_stages=True)
+                                   for thr in (0.01, 0.65)]
+            # shorter prompts of the same workload (the lengths most of the reference's latency protocol covers,
+            # eval/efficiency/latency.py:90-108): its first 16384 and 32768 tokens, and the 32768-token configuration
+            line["shorter_prompts"] = [timed_layer_point(w, q, k, v, table, pt, steps=10, n_tokens=t, with_stages=True)
+                                       for t in (16384, 32768)]
+            w2 = synthetic.WORKLOADS["C2"]
+            q2, k2, v2 = synthetic.workload_inputs(w2, device=dev)
+            c2 = timed_layer_point(w2, q2, k2, v2, synthetic.random_cluster_table(w2.hq, w2.n_clusters, 2, w2.seed),
+                                   w2.pattern_threshold, steps=10, with_stages=True)
+            c2["workload"] = "C2: B1 Hq32 Hkv8 D128 N32768 bf16, seed %d" % w2.seed
+            line["c2_layer"] = c2
+            del q2, k2, v2
         line["sharing_layer"] = sharing_layer_variant(args, w, pt, q, k, v, table)
 
     if not args.no_cpu_baseline:
@@ -575,13 +667,16 @@ def main():
         ops.release_workspaces()
         torch.cuda.empty_cache()
         targs = argparse.Namespace(**vars(args))
-        targs.seq_len, targs.warmup, targs.steps = 131072, 1, 1
+        targs.seq_len, targs.warmup, targs.steps = 131072, 1, 3  # 1 warm-up, mean of 3 timed forwards
         targs.length_sweep = "1024,4096,16384"
+        targs.both_rope = True
+        targs.fuse_rope = True  # bit-identical to the model's own rotary embedding; the other setting is timed as well
         c4 = c4_line(targs)
         line["ttft"] = {"value": c4["value"], "unit": "s", "steps": c4["steps"], "warmup": c4["warmup"],
                         "tokens_per_s": c4["tokens_per_s"], "mean_block_density": c4["mean_block_density"],
                         "decisions": c4["decisions"], "finite_logits": c4["finite_logits"],
                         "workload": c4["config"]["workload"], "fuse_rope": c4["config"]["fuse_rope"],
+                        "other_rope_setting": c4.get("other_rope_setting"),
                         "length_sweep": c4.get("length_sweep")}
     print(json.dumps(line))
 
