@@ -339,9 +339,13 @@ __device__ __forceinline__ void at_mfma_first(floatx4& d, bf16x8 a, bf16x8 b) { 
 __device__ __forceinline__ void at_mfma_acc(floatx4& d, bf16x8 a, bf16x8 b) {  // d += a . b
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
 }
-// 16 wait states (a 16x16x32 MFMA takes 4 passes), tied to the registers so that nothing that reads them moves up
-__device__ __forceinline__ void at_settle_s(floatx4 (&s)[2][2]) {
-  asm volatile("s_nop 15" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]));
+// ... and the same with the wait states that let vector instructions read the results of this and every earlier MFMA
+// INSIDE the statement.  A separate settling statement tied to the result registers is not enough where the reader
+// follows closely: to satisfy the tie the register allocator may first copy a result into other registers -- with a
+// vector move that reads the result while the MFMA is still in flight -- and put the wait states behind that copy
+// (seen in the generated code of the pivot instantiation: a copy of the row sums five wait states behind their MFMA).
+__device__ __forceinline__ void at_mfma_acc_settled(floatx4& d, bf16x8 a, bf16x8 b) {  // d += a . b, then 16 wait states
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\ts_nop 15" : "+v"(d) : "v"(a), "v"(b));
 }
 __device__ __forceinline__ void at_settle_o(floatx4 (&o)[9][2]) {
   asm volatile("s_nop 15"
@@ -405,7 +409,9 @@ __device__ __forceinline__ void at_prefetch_qk(const AtAddr& ad, bf16x8 (&pre)[2
 // read from LDS since).  NEXT >= 0: the stage ends by fetching the first two operands of the next one, quarter NEXT.
 // HALF: q, k and v are zero beyond channel 64 (a head_dim of at most 64 padded to the tiles' 128): the S product takes the
 // first two of its four channel steps and O the first four of its eight channel tiles -- half the operand slots.
-template <bool DO_QK, bool DO_PV, int KQ, int VB, int KT, bool PRE, int NEXT, bool HALF>
+// SETTLE: the stage's last MFMA carries the wait states after which vector instructions may read every MFMA result
+// (a run's first stage, whose S the next stage's softmax reads at once; a pivot head's stage in front of the block sums).
+template <bool DO_QK, bool DO_PV, int KQ, int VB, int KT, bool PRE, int NEXT, bool HALF, bool SETTLE>
 __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2][4], floatx4 (&s_out)[2][2],
                                          const floatx4 (&s_in)[2][2], const bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
                                          floatx4 (&o)[9][2], float sc, const float (&neg_m)[2], uint32_t (&det)[2],
@@ -444,11 +450,14 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
     constexpr int in_flight_after = (NP - 1 - k) < (AHEAD - 1) ? (NP - 1 - k) : (AHEAD - 1);
     AT_WAIT_LGKM(in_flight_after);  // operand k has landed
     AT_PIN();
-    auto mfma = [&](auto qc) {
+    auto mfma = [&](auto qc, auto lastc) {
       constexpr int qt = decltype(qc)::value;
+      constexpr bool settle = decltype(lastc)::value;  // the stage's last MFMA, and results are read right behind it
       if constexpr (qk) {
         if constexpr ((i >> 1) == 0)
           at_mfma_first(s_out[i & 1][qt], opnd[k], qb[qt][0]);
+        else if constexpr (settle)
+          at_mfma_acc_settled(s_out[i & 1][qt], opnd[k], qb[qt][i >> 1]);
         else
           at_mfma_acc(s_out[i & 1][qt], opnd[k], qb[qt][i >> 1]);
       } else {
@@ -457,7 +466,7 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
     };
     // the two query tiles take turns at going first: across a slot boundary the B operand (Q or P of one query tile)
     // stays the same for two MFMAs in a row, as the A operand does inside a slot (+0.5 % under the power cap)
-    mfma(std::integral_constant<int, (k & 1)>{});
+    mfma(std::integral_constant<int, (k & 1)>{}, std::false_type{});
     if constexpr (k + AHEAD < NP) fetch(std::integral_constant<int, k + AHEAD>{});
 #pragma unroll
     for (int u = 0; u < EPS; ++u) {
@@ -490,10 +499,13 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
       }
     }
     AT_PIN();
-    mfma(std::integral_constant<int, 1 - (k & 1)>{});
+    mfma(std::integral_constant<int, 1 - (k & 1)>{}, std::integral_constant<bool, SETTLE && !DO_PV && k == NP - 1>{});
     if constexpr (DO_PV && k == NP - 1) {  // row sums of P(j-1) as rounded for the P.V product: ones . P
       at_mfma_acc(o[8][0], ones, p_prev[0]);
-      at_mfma_acc(o[8][1], ones, p_prev[1]);
+      if constexpr (SETTLE)
+        at_mfma_acc_settled(o[8][1], ones, p_prev[1]);
+      else
+        at_mfma_acc(o[8][1], ones, p_prev[1]);
     }
     AT_PIN();
   });
@@ -504,9 +516,7 @@ __device__ __forceinline__ void at_fused(const AtAddr& ad, const bf16x8 (&qb)[2]
   e[15] = __builtin_amdgcn_exp2f(x[15]);
   pk[7] = at_pack2(e[14], e[15]);
   det[1] |= pk[7];
-  // start of a run: S_out's last accumulation is only a few cycles old and the next stage reads it with vector
-  // instructions right away
-  if constexpr (DO_QK && !DO_PV) at_settle_s(s_out);
+  static_assert(!(DO_QK && !DO_PV) || SETTLE, "a run's first stage: the next stage's softmax reads S_out at once");
   at_u32x4 w0, w1;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -532,12 +542,13 @@ __device__ __forceinline__ void at_qk_only(const char* kb, int koff, const bf16x
     for (int qt = 0; qt < 2; ++qt) {
       if ((i >> 1) == 0)
         at_mfma_first(s_out[i & 1][qt], a[i], qb[qt][0]);
+      else if (i == QS - 1 && qt == 1)  // the last one: the softmax of the next stage reads S_out right away
+        at_mfma_acc_settled(s_out[i & 1][qt], a[i], qb[qt][i >> 1]);
       else
         at_mfma_acc(s_out[i & 1][qt], a[i], qb[qt][i >> 1]);
     }
     AT_PIN();
   }
-  at_settle_s(s_out);
 }
 
 template <int KT, bool HALF>
@@ -556,7 +567,7 @@ __device__ __forceinline__ void at_pv_only(const char* vb, int voff, const bf16x
     AT_PIN();
   }
   at_mfma_acc(o[8][0], ones, p[0]);
-  at_mfma_acc(o[8][1], ones, p[1]);
+  at_mfma_acc_settled(o[8][1], ones, p[1]);  // the end of a run: the block sums and the epilogue read O next
 }
 
 // causal predicate inside the diagonal block; key_base = offset of the half-tile's first key inside the block
@@ -663,8 +674,11 @@ __device__ __forceinline__ void at_step(const AtAddr& ad, const bf16x8 (&qb)[2][
   if (HAVE_PREV) at_commit<MODE>(s_out, p_prev, det, o, scale_log2, m_run, l_mark);
   if (diag) at_causal(s_in, key_base, t);
   const float neg_m[2] = {-m_run[0], -m_run[1]};
-  at_fused<DO_QK, HAVE_PREV, KQ, VB, KT, PRE, NEXT, (MODE & 2) != 0>(ad, qb, s_out, s_in, p_prev, p_out, o, scale_log2,
-                                                                      neg_m, det, ones, pre);
+  // wait states inside the stage's last MFMA: a run's first stage (S read at once), and for pivot heads the stage
+  // behind which the block sums are taken (emit in the kernel: the second stage of a block in the steady state)
+  constexpr bool SETTLE = (DO_QK && !HAVE_PREV) || ((MODE & 1) != 0 && DO_QK && HAVE_PREV && KQ == 1);
+  at_fused<DO_QK, HAVE_PREV, KQ, VB, KT, PRE, NEXT, (MODE & 2) != 0, SETTLE>(ad, qb, s_out, s_in, p_prev, p_out, o,
+                                                                              scale_log2, neg_m, det, ones, pre);
 }
 
 // PIVOT = false: every head except the pivots that have a slot in the scheduler area's table (when skip_slotted).
@@ -817,7 +831,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     float* const pu = PIVOT ? pivot_u + tri_row * AT_BS : nullptr;
     auto emit = [&](int c) {
       if constexpr (PIVOT) {
-        asm volatile("s_nop 15" : "+v"(o[8][0]), "+v"(o[8][1]));  // the sums' last MFMAs have written
+        // (the sums' last MFMA carried its wait states: at_fused<SETTLE> / at_pv_only)
         AT_LANE_VIEW(tq);
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
