@@ -82,14 +82,13 @@ typedef struct sp_cluster_state {
 int sp_version(void);
 const char* sp_arch(void);       /* "gfx950" */
 const char* sp_last_error(void); /* host string, valid until the next failing call on this thread */
-/* Measurement aid (no counterpart in the reference): runs `iters` x 4 back-to-back bf16 32x32x16 MFMAs per wave on
- * every CU (8 waves per CU).  random_operands 0: one constant in every operand element; 1: random values per lane,
- * the same registers for every instruction (operand inputs never toggle); 2: four different random operand pairs in
- * rotation, so both operands change with every instruction as in a real product.  The caller times it; flops =
- * sp_diag_mfma_flops(iters).  Used to calibrate the sustained matrix-core rate under the board's power limit, which
- * depends on how much the operand bits toggle.  out: 512 floats of device scratch. */
-int sp_diag_mfma_bf16(int32_t iters, int32_t random_operands, float* out, sp_stream_t stream);
-double sp_diag_mfma_flops(int32_t iters);
+
+/* pool types of sp_pool_bf16, numbered as in the reference's kernel (attn/utils.py:135, 255) */
+#define SP_POOL_AVG 0
+#define SP_POOL_MAX 1
+#define SP_POOL_MIN 2
+#define SP_POOL_MAXABS 3 /* max of absolute values */
+#define SP_POOL_SUM 4
 
 /* ---- (a) block average pooling --------------------------------------------------------------
  * Replaces triton_bnhd_pool / bnhd_pool_kernel (attn/utils.py:131-261, "avg" mode) and the torch
@@ -99,6 +98,13 @@ double sp_diag_mfma_flops(int32_t iters);
 int sp_pool_avg_bf16(const void* x, void* y, int64_t n, int32_t h, int32_t d, int64_t x_stride_n,
                      int64_t x_stride_h, int32_t bs, int32_t tail_mode, const int32_t* head_enable,
                      sp_stream_t stream);
+/* The other pool types of bnhd_pool_kernel (attn/utils.py:180-191; nothing in the selection uses them): per block of
+ * bs tokens the maximum, the minimum, the maximum of the absolute values or the sum (SP_POOL_*; SP_POOL_AVG = the
+ * call above with SP_POOL_TAIL_TRUE_LENGTH).  As in the reference's kernel, tokens of a ragged last block that lie
+ * beyond the sequence count as zeros (its masked load, utils.py:168-179): that block's maximum is at least 0 and its
+ * minimum at most 0.  Sums accumulate in fp32 and are rounded to bf16 once. */
+int sp_pool_bf16(const void* x, void* y, int64_t n, int32_t h, int32_t d, int64_t x_stride_n, int64_t x_stride_h,
+                 int32_t bs, int32_t pool_type, sp_stream_t stream);
 
 /* ---- last-block scores -> vertical / slash --------------------------------------------------
  * Replaces attention_sharing.py:127-167 + sum_all_diagonal_matrix (attn/utils.py:79-86) +
@@ -201,19 +207,6 @@ size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, in
  * and their block-average maps (shareprefill_attn.py:425-457) are made from those instead of a second pass over
  * Q.K^T; further pivots, or all of them with the base size, take that second pass.  Same results to rounding. */
 size_t sp_attn_pivot_scratch_bytes(int64_t n, int32_t bs);
-/* Measurement aid (no counterpart in the reference): shader-clock cycles and 100 MHz wall ticks that workgroup 0
- * of the LAST sp_block_sparse_attn_fwd_bf16 launch on this workspace spent in the kernel; cycles / (ticks / 100)
- * is the average shader clock in MHz under that load.  Copies two int64 to host memory after synchronising the
- * stream. */
-int sp_attn_last_launch_clocks(const void* workspace, int64_t n, int32_t hkv, int32_t d, int32_t bs,
-                               int64_t* cycles_and_ticks, sp_stream_t stream);
-/* Test / measurement aid (no counterpart in the reference): how the LAST sp_block_sparse_attn_fwd_bf16 launch on
- * this workspace paired query blocks into work items, one byte per two adjacent heads (2i, 2i+1): 0 = rows 2p and
- * 2p+1 of each head share an item, 1 = the same row of the two heads does (chosen when it makes the unions of the
- * paired masks smaller; only inside a kv group).  Copies (hq + 1) / 2 bytes to host memory after synchronising the
- * stream.  The pairing changes how the work is scheduled, never the result. */
-int sp_attn_last_launch_pairing(const void* workspace, int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs,
-                                uint8_t* by_heads, sp_stream_t stream);
 int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int32_t d, int64_t v_stride_n, int64_t v_stride_h,
                           int32_t bs, void* workspace, size_t workspace_bytes, sp_stream_t stream);
 int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const void* v, int64_t n, int32_t hq, int32_t hkv,

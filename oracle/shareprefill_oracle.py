@@ -23,6 +23,7 @@ Canonical arithmetic (where the reference leaves behaviour to the backend):
 
 Parity pins (what each function is checked against, besides the HIP path):
   pool_avg ........... float64 mean, constant/linearity invariants
+  pool ............... torch's max_pool1d / avg_pool1d library routines on the zero-filled sequence; one-hot cases
   diagonal_sums ...... brute-force double loop; sums to the matrix total
   cover_count ........ literal torch sort+cumsum formula; one-hot / uniform closed forms
   cover_keep_le ...... literal torch formula; brute force on tiny inputs; "excludes crossing entry"
@@ -176,6 +177,33 @@ def pool_avg(x: torch.Tensor, bs: int) -> torch.Tensor:
     cnt = torch.full((nb,), float(bs))
     cnt[-1] = float(n - (nb - 1) * bs)
     return (s / cnt[:, None, None]).to(x.dtype)
+
+
+def pool(x: torch.Tensor, bs: int, pool_type: str) -> torch.Tensor:
+    """utils.py:131-261 triton_bnhd_pool for x[N,H,D] -> [nb,H,D] in x.dtype, pool types "max", "min", "maxabs", "sum"
+    ("avg": pool_avg).  Plain loops over the blocks.
+
+    The reference's kernel loads the tokens of a ragged last block beyond the sequence as zeros (utils.py:168-179,
+    other=0) and reduces over all bs slots (:180-191), so the tail's maximum is at least 0 and its minimum at most 0.
+    Sums accumulate in fp32 here (the reference's kernel adds in the input dtype)."""
+    n, h, d = x.shape
+    nb = -(-n // bs)
+    out = torch.zeros(nb, h, d, dtype=torch.float32)
+    for b in range(nb):
+        blk = x[b * bs:(b + 1) * bs].float()
+        if blk.shape[0] < bs:
+            blk = torch.cat([blk, torch.zeros(bs - blk.shape[0], h, d)])
+        if pool_type == "max":
+            out[b] = blk.amax(0)
+        elif pool_type == "min":
+            out[b] = blk.amin(0)
+        elif pool_type == "maxabs":
+            out[b] = blk.abs().amax(0)
+        elif pool_type == "sum":
+            out[b] = blk.sum(0)
+        else:
+            raise KeyError(pool_type)
+    return out.to(x.dtype)
 
 
 def diagonal_sums(p: torch.Tensor) -> torch.Tensor:

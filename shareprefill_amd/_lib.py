@@ -23,6 +23,7 @@ def SP_FLAG_SCALE_DIM(head_dim: int) -> int:
 
 
 SP_POOL_TAIL_TRUE_LENGTH, SP_POOL_TAIL_RESCALE = 0, 1
+SP_POOL_TYPES = {"avg": 0, "max": 1, "min": 2, "maxabs": 3, "sum": 4}  # attn/utils.py:255
 SP_ATTN_V_REPACKED = 1
 SP_ATTN_PAIR_ROWS = 2
 SP_ATTN_HALF_CHANNELS = 4
@@ -51,6 +52,7 @@ SIGNATURES = {
     "sp_diag_mfma_bf16": (_I32, [_I32, _I32, _P, _P]),
     "sp_diag_mfma_flops": (_D, [_I32]),
     "sp_pool_avg_bf16": (_I32, [_P, _P, _I64, _I32, _I32, _I64, _I64, _I32, _I32, _P, _P]),
+    "sp_pool_bf16": (_I32, [_P, _P, _I64, _I32, _I32, _I64, _I64, _I32, _I32, _P]),
     "sp_lastq_scores_workspace_bytes": (_SZ, [_I64, _I32, _I32]),
     "sp_lastq_scores_bf16": (_I32, [_P, _P, _I64, _I32, _I32, _I32, _I64, _I64, _I64, _I64, _I32, _U32, _P, _SZ,
                                     _P, _P, _P, _P, _P]),

@@ -6,6 +6,7 @@
 #include <stdio.h>
 
 #include "shareprefill_hip.h"
+#include "shareprefill_hip_diag.h"
 
 #define SP_WAVE 64
 

@@ -67,6 +67,22 @@ def pool_avg(x: torch.Tensor, block_size: int, tail_mode: int = _lib.SP_POOL_TAI
     return out
 
 
+def pool(x: torch.Tensor, block_size: int, pool_type: str) -> torch.Tensor:
+    """x: bf16 [H, N, D] view -> bf16 [nb, H, D], one of the reference kernel's pool types "avg", "max", "min",
+    "maxabs", "sum" per block of block_size tokens (bnhd_pool_kernel, attn/utils.py:131-208)."""
+    lib = _lib.load()
+    _check_hnd(x, "x")
+    if pool_type not in _lib.SP_POOL_TYPES:
+        raise KeyError(pool_type)
+    h, n, d = x.shape
+    nb = -(-n // block_size)
+    out = torch.empty(nb, h, d, dtype=torch.bfloat16, device=x.device)
+    st = lib.sp_pool_bf16(_ptr(x), _ptr(out), n, h, d, x.stride(1), x.stride(0), block_size,
+                          _lib.SP_POOL_TYPES[pool_type], _stream(x.device))
+    _lib.check(st, "sp_pool_bf16")
+    return out
+
+
 _workspaces = {}
 
 

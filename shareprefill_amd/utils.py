@@ -8,20 +8,24 @@ from . import ops
 
 
 def triton_bnhd_pool(x: torch.Tensor, kernel_size: int, pool_type: str = "avg") -> torch.Tensor:
-    """x bf16 [B, N, H, D] -> [B, ceil(N / kernel_size), H, D]: the mean of every run of kernel_size tokens, the last
-    run divided by its true length (attn/utils.py:211-261; nothing here is Triton).
+    """x bf16 [B, N, H, D] -> [B, ceil(N / kernel_size), H, D]: every run of kernel_size tokens reduced by pool_type
+    (attn/utils.py:211-261; nothing here is Triton): "avg" (the last run divided by its true length; the one the
+    selection uses, attention_sharing.py:194-196), "max", "min", "maxabs", "sum", or the slicing mode "last".
 
-    Of the reference's pool types only "avg", the one its selection uses (attention_sharing.py:194-196), and the
-    slicing mode "last" are built.  The sum is kept in fp32 and rounded once (the reference's kernel adds in bf16)."""
+    As in the reference's kernel a ragged last run is filled up with zeros, which a maximum / minimum then sees.  Sums
+    are kept in fp32 and rounded once (the reference's kernel adds in bf16); an unknown pool_type is a KeyError, as
+    from the reference's own dictionary (attn/utils.py:254-256)."""
     if x.dim() != 4:
         raise ValueError("x must be [batch_size, seq_len, num_heads, head_dim]")
     if pool_type == "last":
         if x.shape[1] % kernel_size == 0:
             return x[:, kernel_size - 1::kernel_size, ...]
         return torch.cat((x[:, kernel_size - 1::kernel_size, ...], x[:, -1:, ...]), dim=1)
-    if pool_type != "avg":
-        raise NotImplementedError(f"pool_type {pool_type!r}: only 'avg' and 'last' are built")
-    return torch.stack([ops.pool_avg(x[b].transpose(0, 1), kernel_size) for b in range(x.shape[0])])
+    assert x.shape[-1] in {16, 32, 64, 128}
+    assert kernel_size in {16, 32, 64, 128, 256, 512}
+    if pool_type == "avg":
+        return torch.stack([ops.pool_avg(x[b].transpose(0, 1), kernel_size) for b in range(x.shape[0])])
+    return torch.stack([ops.pool(x[b].transpose(0, 1), kernel_size, pool_type) for b in range(x.shape[0])])
 
 
 def score_cover_topk(x: torch.Tensor, score: float) -> torch.Tensor:

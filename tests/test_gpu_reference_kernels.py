@@ -210,8 +210,18 @@ def test_bnhd_pool_reference_signature(gpu_device, b, n, h, d, ks):
     last = triton_bnhd_pool(x.to(gpu_device), ks, "last").cpu()
     rows = list(range(ks - 1, n, ks)) + ([n - 1] if n % ks else [])
     assert torch.equal(last, x[:, rows])
-    with pytest.raises(NotImplementedError):
-        triton_bnhd_pool(x.to(gpu_device), ks, "max")
+    # the other pool types (attn/utils.py:180-191): max / min / maxabs are exact, the sum within one bf16 rounding
+    for kind in ("max", "min", "maxabs", "sum"):
+        got = triton_bnhd_pool(x.to(gpu_device), ks, kind).cpu()
+        assert got.shape == (b, m, h, d) and got.dtype == torch.bfloat16
+        for i in range(b):
+            want = O.pool(x[i], ks, kind)
+            if kind == "sum":
+                assert ((got[i].float() - want.float()).abs() <= want.float().abs() * 2.0 ** -7 + 1e-30).all()
+            else:
+                assert torch.equal(got[i], want), kind
+    with pytest.raises(KeyError):
+        triton_bnhd_pool(x.to(gpu_device), ks, "median")
 
 
 def test_score_cover_topk_reference_signature(gpu_device):
@@ -252,10 +262,30 @@ def test_block_wise_prefill_attention_small_head_dims(gpu_device, d):
             assert (avg[0, h].cpu() - ref_avg[h]).abs().max().item() <= 2e-3
 
 
+def _reference_side_binding():
+    """The ctypes stub that the integration notes at the repository root show to a maintainer of the reference (the
+    module they would add as shareprefill/attn/hip_backend.py), taken from the notes themselves -- their first Python
+    block -- and executed against the in-tree library, so that the text shown there is the code tested here."""
+    import types
+
+    from shareprefill_amd import _lib
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "INTEGRATION.md")).read()
+    blocks = [b[:b.index("```")] for b in text.split("```python")[1:]]
+    code = next(b for b in blocks if 'C.CDLL("libshareprefill_hip.so")' in b)
+    code = code.replace('C.CDLL("libshareprefill_hip.so")', f"C.CDLL({_lib.LIB_PATH!r})")
+    mod = types.ModuleType("hip_backend")
+    exec(compile(code, "hip_backend.py", "exec"), mod.__dict__)
+    return mod
+
+
 def test_ctypes_binding_for_the_reference(gpu_device):
-    """shareprefill_amd/reference_binding.py -- the self-contained ctypes stub a maintainer of the reference would add
-    -- gives the results of the package's own front ends."""
-    from shareprefill_amd import ops, reference_binding as rb
+    """The self-contained ctypes stub a maintainer of the reference would add gives the results of the package's own
+    front ends."""
+    from shareprefill_amd import ops
+
+    rb = _reference_side_binding()
 
     hq, hkv, n = 4, 2, 1100
     g = torch.Generator().manual_seed(8)

@@ -13,12 +13,15 @@ import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "shareprefill_hip.h")
+DIAG_HEADER = os.path.join(ROOT, "include", "shareprefill_hip_diag.h")  # measurement aids, not the drop-in boundary
 
 
-def header_functions():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(sp_[a-z0-9_]+)\s*\(", text)) - {"sp_cluster_state"})
+def header_functions(paths=(HEADER, DIAG_HEADER)):
+    names = set()
+    for path in paths:
+        text = re.sub(r"/\*.*?\*/", "", open(path).read(), flags=re.S)
+        names |= set(re.findall(r"\b(sp_[a-z0-9_]+)\s*\(", text))
+    return sorted(names - {"sp_cluster_state"})
 
 
 def test_library_exports_every_declared_symbol():
@@ -31,6 +34,10 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signature table and header disagree"
+    # the measurement aids live in a header of their own: the boundary header declares none of them
+    diag = {"sp_diag_mfma_bf16", "sp_diag_mfma_flops", "sp_attn_last_launch_clocks", "sp_attn_last_launch_pairing"}
+    assert set(header_functions((DIAG_HEADER,))) == diag
+    assert not diag & set(header_functions((HEADER,)))
 
 
 def test_library_identity_and_error_string():

@@ -88,6 +88,41 @@ def test_pool_avg_constant_and_linear():
     assert torch.allclose(O.pool_avg(a + 2 * b, 128), O.pool_avg(a, 128) + 2 * O.pool_avg(b, 128), atol=1e-5)
 
 
+@pytest.mark.parametrize("n,ks", [(256, 128), (300, 128), (100, 16), (1000, 512), (33, 32)])
+def test_pool_types_against_the_library_pooling_routines(n, ks):
+    """The reference kernel's other pool types (attn/utils.py:180-191) against torch's own pooling routines run on the
+    sequence filled up with zeros to a whole number of blocks, which is what the kernel's masked load does to a ragged
+    last block (utils.py:168-179) -- so a negative tail has maximum 0, a positive tail minimum 0."""
+    g = torch.Generator().manual_seed(n + ks)
+    x = (torch.randn(n, 2, 16, generator=g) * 3).to(torch.bfloat16)
+    nb = -(-n // ks)
+    seq = torch.nn.functional.pad(x.float(), (0, 0, 0, 0, 0, nb * ks - n)).permute(1, 2, 0).reshape(1, 32, nb * ks)
+    F = torch.nn.functional
+    lib = {"max": F.max_pool1d(seq, ks, ks), "min": -F.max_pool1d(-seq, ks, ks), "maxabs": F.max_pool1d(seq.abs(), ks, ks),
+           "sum": F.avg_pool1d(seq, ks, ks) * ks}
+    for kind, want in lib.items():
+        got = O.pool(x, ks, kind)
+        assert got.shape == (nb, 2, 16) and got.dtype == torch.bfloat16
+        want = want.reshape(2, 16, nb).permute(2, 0, 1)
+        if kind == "sum":
+            assert torch.allclose(got.float(), want, rtol=2 ** -7, atol=1e-3)
+        else:
+            assert torch.equal(got.float(), want), kind
+    with pytest.raises(KeyError):
+        O.pool(x, ks, "median")
+
+
+def test_pool_types_see_the_zero_fill_of_a_ragged_tail():
+    x = torch.full((40, 1, 16), -2.0, dtype=torch.bfloat16)
+    assert float(O.pool(x, 32, "max")[0].max()) == -2.0 and float(O.pool(x, 32, "max")[1].max()) == 0.0
+    assert float(O.pool(-x, 32, "min")[1].min()) == 0.0 and float(O.pool(x, 32, "min")[1].min()) == -2.0
+    assert float(O.pool(x, 32, "maxabs")[1].max()) == 2.0 and float(O.pool(x, 32, "sum")[1].max()) == -16.0
+    one = torch.zeros(64, 1, 16, dtype=torch.bfloat16)
+    one[37, 0, 5] = -7.0
+    assert float(O.pool(one, 32, "min")[1, 0, 5]) == -7.0 and float(O.pool(one, 32, "maxabs")[1, 0, 5]) == 7.0
+    assert float(O.pool(one, 32, "max").abs().max()) == 0.0
+
+
 def test_pool_q_head_tail_rescale():
     g = torch.Generator().manual_seed(3)
     x = torch.randn(300, 16, generator=g)
