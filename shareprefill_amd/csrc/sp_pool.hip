@@ -136,19 +136,19 @@ extern "C" int sp_pool_bf16(const void* x, void* y, int64_t n, int32_t h, int32_
 static int pool_launch(int pool_type, const void* x, void* y, int64_t n, int32_t h, int32_t d, int64_t x_stride_n,
                        int64_t x_stride_h, int32_t bs, int32_t tail_mode, const int32_t* head_enable,
                        sp_stream_t stream) {
-  SP_REQUIRE(x && y, SP_ERR_INVALID_ARGUMENT, "sp_pool_avg_bf16: null tensor pointer");
-  SP_REQUIRE(n > 0 && h > 0 && d > 0, SP_ERR_INVALID_ARGUMENT, "sp_pool_avg_bf16: n, h, d must be positive");
-  SP_REQUIRE(d % 8 == 0, SP_ERR_UNSUPPORTED, "sp_pool_avg_bf16: head_dim %d is not a multiple of 8", d);
+  SP_REQUIRE(x && y, SP_ERR_INVALID_ARGUMENT, "sp_pool_avg_bf16 / sp_pool_bf16: null tensor pointer");
+  SP_REQUIRE(n > 0 && h > 0 && d > 0, SP_ERR_INVALID_ARGUMENT, "sp_pool_avg_bf16 / sp_pool_bf16: n, h, d must be positive");
+  SP_REQUIRE(d % 8 == 0, SP_ERR_UNSUPPORTED, "sp_pool_avg_bf16 / sp_pool_bf16: head_dim %d is not a multiple of 8", d);
   SP_REQUIRE(bs >= POOL_SPLIT && bs % POOL_SPLIT == 0, SP_ERR_UNSUPPORTED,
-             "sp_pool_avg_bf16: block size %d is not a multiple of %d", bs, POOL_SPLIT);
+             "sp_pool_avg_bf16 / sp_pool_bf16: block size %d is not a multiple of %d", bs, POOL_SPLIT);
   SP_REQUIRE(x_stride_n % 8 == 0 && x_stride_h % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0,
-             SP_ERR_UNSUPPORTED, "sp_pool_avg_bf16: tensors must be 16-byte aligned with strides multiple of 8");
+             SP_ERR_UNSUPPORTED, "sp_pool_avg_bf16 / sp_pool_bf16: tensors must be 16-byte aligned with strides multiple of 8");
   SP_REQUIRE(tail_mode == SP_POOL_TAIL_TRUE_LENGTH || tail_mode == SP_POOL_TAIL_RESCALE, SP_ERR_INVALID_ARGUMENT,
-             "sp_pool_avg_bf16: unknown tail_mode %d", tail_mode);
+             "sp_pool_avg_bf16 / sp_pool_bf16: unknown tail_mode %d", tail_mode);
   const int64_t nb = sp_ceil_div(n, bs);
   const int chunks_per_block = h * (d / 8);
   const int groups = (int)sp_ceil_div(chunks_per_block, POOL_CHUNKS);
-  SP_REQUIRE(nb * groups < (1ll << 31), SP_ERR_UNSUPPORTED, "sp_pool_avg_bf16: grid too large");
+  SP_REQUIRE(nb * groups < (1ll << 31), SP_ERR_UNSUPPORTED, "sp_pool_avg_bf16 / sp_pool_bf16: grid too large");
   dim3 grid((unsigned)(nb * groups));
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(POOL_CHUNKS * POOL_SPLIT), 0, (hipStream_t)stream, (const sp_bf16*)x,
