@@ -111,6 +111,8 @@ int sp_pool_bf16(const void* x, void* y, int64_t n, int32_t h, int32_t d, int64_
  * torch_bhn_sumpool (attn/utils.py:33-44): softmax over all keys of the last bs queries
  * (scaled by 1/sqrt(d), causal inside the last bs columns), column mean -> vert_tok[hq][n],
  * anti-diagonal mean -> slash_tok[hq][n], and their block sums vert_blk / slash_blk [hq][nb].
+ * bs: 16, 32, 64 or 128 (attention_sharing.py:127 takes any; shareprefill_attn.py:509-516 allows these); d 128;
+ * n >= 128 whatever bs (the kernels work on the last 128 tokens' queries and drop the rows a smaller block lacks).
  * workspace: sp_lastq_scores_workspace_bytes(...) bytes of device scratch. */
 size_t sp_lastq_scores_workspace_bytes(int64_t n, int32_t hq, int32_t bs);
 int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int32_t hq, int32_t hkv, int32_t d,
@@ -190,6 +192,11 @@ int sp_cover_select_global(const float* x, const int32_t* enable, int32_t n_vec,
  * mask (and c <= r) are computed.  For heads with decision == SP_DEC_DENSE the block-averaged attention
  * map avg_attn[h][nb][nb] (fp32, pre-zeroed by the caller) is written as well (:425-457); decision and
  * avg_attn may both be NULL.
+ * bs: 16, 32, 64 or 128 (:509-516); mask [hq][nb][ceil(nb / 64)] and avg_attn are on the grid nb = ceil(n / bs) <= 4096.
+ * The kernels are built on 128-token blocks: for a smaller bs they visit every 128-token block that holds a kept
+ * block and drop the others' keys per 16 x 16 sub-tile, like the keys the causal predicate hides (exact; the work is
+ * that of the 128-token blocks), the maps of DENSE heads come from the recomputing pass only, and
+ * SP_ATTN_HALF_CHANNELS is accepted and ignored (all 128 channels of out are written).
  * workspace: sp_attn_workspace_bytes(...) bytes of device scratch (key-major repack of V, a work counter and
  * the pivot heads' softmax row statistics).
  * sp_attn_repack_v_bf16 fills it; sp_block_sparse_attn_fwd_bf16 calls it first unless flags has

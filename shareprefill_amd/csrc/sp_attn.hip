@@ -584,6 +584,18 @@ __device__ __forceinline__ void at_causal(floatx4 (&s)[2][2], int key_base, int 
       }
 }
 
+// Block sizes below 128: the 16 x 16 sub-tiles of a half-tile whose fine block the mask does not keep are taken out
+// like the keys the causal predicate hides.  kq: bit 8 * qt + c16 = keep the fine block that holds keys 16 c16 .. 16 c16
+// + 15 of the 128-key block for the queries of tile qt (wave-uniform).
+__device__ __forceinline__ void at_keep(floatx4 (&s)[2][2], uint32_t kq, int key_base) {
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+      if (((kq >> (8 * qt + (key_base >> 4) + kt)) & 1u) == 0u)
+        s[kt][qt] = (floatx4){-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+}
+
 // max over the lane's 8 keys of each query tile
 __device__ __forceinline__ void at_lanemax(const floatx4 (&s)[2][2], float (&mx)[2]) {
 #pragma unroll
@@ -621,7 +633,7 @@ __device__ __forceinline__ float at_groupmax(float mx) {
 // s_prev = S(j-1) (causal predicate applied), p = P(j-1), det = OR of its packed words.  On return p is safe to use.
 // PIVOT: l_mark (the row sums at the start of the current key block, see the block sums of pivot heads in the
 // kernel) follows every rescale.
-// MODE: bit 0 = PIVOT, bit 1 = HALF (see at_fused)
+// MODE: bit 0 = PIVOT, bit 1 = HALF (see at_fused), bit 2 = FINE (see at_keep)
 template <int MODE>
 __device__ __forceinline__ void at_commit(const floatx4 (&s_prev)[2][2], bf16x8 (&p)[2], uint32_t (&det)[2],
                                           floatx4 (&o)[9][2], float scale_log2, float (&m_run)[2],
@@ -670,9 +682,10 @@ __device__ __forceinline__ void at_step(const AtAddr& ad, const bf16x8 (&qb)[2][
                                         floatx4 (&s_in)[2][2], bf16x8 (&p_prev)[2], bf16x8 (&p_out)[2],
                                         floatx4 (&o)[9][2], float scale_log2, float (&m_run)[2], uint32_t (&det)[2],
                                         const bf16x8& ones, bool diag, int key_base, int t, float (&l_mark)[2],
-                                        bf16x8 (&pre)[2]) {
+                                        bf16x8 (&pre)[2], uint32_t kq = 0xffffu) {
   if (HAVE_PREV) at_commit<MODE>(s_out, p_prev, det, o, scale_log2, m_run, l_mark);
   if (diag) at_causal(s_in, key_base, t);
+  if constexpr ((MODE & 4) != 0) at_keep(s_in, kq, key_base);
   const float neg_m[2] = {-m_run[0], -m_run[1]};
   // wait states inside the stage's last MFMA: a run's first stage (S read at once), and for pivot heads the stage
   // behind which the block sums are taken (emit in the kernel: the second stage of a block in the steady state)
@@ -686,16 +699,19 @@ __device__ __forceinline__ void at_step(const AtAddr& ad, const bf16x8 (&qb)[2][
 // block relative to the running max at that time as u = log2(sum) + max, from which at_avg_from_block_sums (sp_attn_avg_kernel) makes
 // the block-average map without recomputing any logit.  pivot_u: fp32 [slot][r*(r+1)/2 + c][128 queries].
 // HALF: q, k and v are zero beyond channel 64 (see at_fused); channels 64..127 of out are then not written.
-template <bool PIVOT, bool HALF>
+// FINE: a block size f = 128 >> fshift below 128.  `mask` is then the OR of the caller's fine mask over 128-token
+// blocks (sp_attn_coarsen_kernel) and decides which 128-key blocks a row visits; fine_mask [hq][nbf][nbfw] decides, per
+// 16 x 16 sub-tile, what survives of a visited block (at_keep).  Exact, at the cost of computing whole 128 x 128 blocks.
+template <bool PIVOT, bool HALF, bool FINE = false>
 __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const sp_bf16* __restrict__ vt,
     const uint64_t* __restrict__ mask, const int32_t* __restrict__ decision, sp_bf16* __restrict__ out,
     float2* __restrict__ rowstat, int64_t n, int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n,
     int64_t sk_h, int nb, int nbw, float scale_log2, int* __restrict__ sched, int skip_slotted,
-    float* __restrict__ pivot_u) {
+    float* __restrict__ pivot_u, const uint64_t* __restrict__ fine_mask, int fshift, int nbf, int nbfw) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // K ring (4 x 16 KiB) | V^T ring (4 x 16 KiB)
   __shared__ int s_queue, s_ticket;
-  constexpr int MODE = (PIVOT ? 1 : 0) | (HALF ? 2 : 0);
+  constexpr int MODE = (PIVOT ? 1 : 0) | (HALF ? 2 : 0) | (FINE ? 4 : 0);
   if (PIVOT && sched[AT_NPIV_SLOT] == 0) return;  // no pivot in this layer
   const uint8_t* const slots = reinterpret_cast<const uint8_t*>(sched + AT_SLOT_TABLE);
   const uint8_t* const pair_table = reinterpret_cast<const uint8_t*>(sched + AT_PAIR_TABLE);
@@ -814,6 +830,46 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       }
     }
 
+    // FINE: the two fine mask rows of this wave's query tiles, and the keep bits (at_keep) of a block from them
+    const uint64_t* frow[2] = {fine_mask, fine_mask};
+    if constexpr (FINE) {
+      const int w4 = wave & 3;
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        int fr = (r * AT_BS + 32 * w4 + 16 * qt) >> (7 - fshift);
+        if (fr > nbf - 1) fr = nbf - 1;  // (queries beyond the sequence: computed, never stored)
+        frow[qt] = fine_mask + ((int64_t)h * nbf + fr) * nbfw;
+      }
+    }
+    // the two 64-bit mask words are requested a block ahead of their use (fine_issue at the top of block b for block
+    // b + 1, fine_take when the walk moves on)
+    uint64_t fw_next[2] = {~0ull, ~0ull};
+    auto fine_issue = [&](int c) {
+      if constexpr (FINE) {
+        const int fc0 = c << fshift;  // first fine column of the 128-key block; its 1 << fshift bits share a word
+        fw_next[0] = frow[0][fc0 >> 6];
+        fw_next[1] = frow[1][fc0 >> 6];
+      }
+    };
+    auto fine_take = [&](int c) -> uint32_t {  // kq of column c from the words fine_issue(c) requested
+      uint32_t kq = 0xffffu;
+      if constexpr (FINE) {
+        const int fc0 = c << fshift;
+        kq = 0u;
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+          const uint32_t fb = (uint32_t)(fw_next[qt] >> (fc0 & 63));
+          uint32_t k16 = 0u;
+#pragma unroll
+          for (int c16 = 0; c16 < 8; ++c16) k16 |= ((fb >> (c16 >> (3 - fshift))) & 1u) << c16;
+          kq |= k16 << (8 * qt);
+        }
+        kq = __builtin_amdgcn_readfirstlane(kq);
+      }
+      return kq;
+    };
+    uint32_t kq_cur = 0xffffu;
+
     floatx4 o[9][2];  // [channel tile][query tile]; o[8]: the row sums (ones . P)
 #pragma unroll
     for (int dt = 0; dt < 9; ++dt)
@@ -880,6 +936,8 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       issue_k(c_cur, 0, 0);
       issue_k(c_cur, 1, 1);
       issue_v(c_cur, 0, 0);
+      fine_issue(c_cur);
+      kq_cur = fine_take(c_cur);
     }
 
     // The compute walk.  Per block every wave passes `top` exactly once (wait, barrier, issue), whatever its row
@@ -897,6 +955,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       // (hidden loop invariance: no precomputed copies of these lane constants that could be spilled)
       asm volatile("" : "+v"(lo.k), "+v"(lo.v));
       c_next = (int)(e_next & AT_COL_MASK);
+      fine_issue(c_next);
       {
         const int ba = b + 2 < n_blk ? b + 2 : n_blk - 1;
         asm volatile("ds_read_b32 %0, %1" : "=v"(e_ahead) : "v"(blist_addr + 4u * (uint32_t)ba));
@@ -926,6 +985,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       if (b < n_blk) {
         c_cur = (int)(e_next & AT_COL_MASK);
         mine = (e_next & my_flag) != 0u;
+        kq_cur = fine_take(c_cur);
       } else {
         c_cur = -1;
         mine = false;
@@ -949,14 +1009,15 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
       at_qk_only<0, HALF>(kb, koff, qb, sa);
       feed(1);
       at_step<true, false, 1, 0, 0, MODE, false, 2>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
-                                                     c_cur == r, 0, tq, l_mark, pre);
+                                                     c_cur == r, 0, tq, l_mark, pre, kq_cur);
       feed(2);
       at_step<true, true, 2, 1, 0, MODE, true, 3>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
-                                                   c_cur == r, 32, tq, l_mark, pre);
+                                                   c_cur == r, 32, tq, l_mark, pre, kq_cur);
       feed(3);
       at_step<true, true, 3, 1, 1, MODE, true, -1>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
-                                                    c_cur == r, AT_SUB, tq, l_mark, pre);
+                                                    c_cur == r, AT_SUB, tq, l_mark, pre, kq_cur);
       int c_prev = c_cur;
+      uint32_t kq_prev = kq_cur;
       step_walk();
       // ---- steady state: four half-tile steps per block ----
       while (mine) {  // (mine implies c_cur >= 0)
@@ -968,20 +1029,21 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         if (grp) __builtin_amdgcn_s_setprio(1);
         // S(previous block, keys 96..127) -> P;  S(keys 0..31) on the matrix core;  O += V^T(2b-1, keys 0..31) . P
         at_step<true, true, 0, 0, 0, MODE, true, 1>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
-                                                     c_prev == r, AT_SUB + 32, tq, l_mark, pre);
+                                                     c_prev == r, AT_SUB + 32, tq, l_mark, pre, kq_prev);
         feed(0);
         at_step<true, true, 1, 0, 1, MODE, true, 2>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
-                                                     c_cur == r, 0, tq, l_mark, pre);
+                                                     c_cur == r, 0, tq, l_mark, pre, kq_cur);
         emit(c_prev);  // the previous block's last half-tile went into O (and the sums) in this step
         if (grp) __builtin_amdgcn_s_setprio(0);
         feed(1);
         feed(2);
         at_step<true, true, 2, 1, 0, MODE, true, 3>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
-                                                     c_cur == r, 32, tq, l_mark, pre);
+                                                     c_cur == r, 32, tq, l_mark, pre, kq_cur);
         feed(3);
         at_step<true, true, 3, 1, 1, MODE, true, -1>(ad, qb, sb, sa, pb, pa, o, scale_log2, m_run, det, ones,
-                                                      c_cur == r, AT_SUB, tq, l_mark, pre);
+                                                      c_cur == r, AT_SUB, tq, l_mark, pre, kq_cur);
         c_prev = c_cur;
+        kq_prev = kq_cur;
         step_walk();
       }
       // ---- drain: the run's last half-tile and its P.V (V^T of sub-tile 2b-1) ----
@@ -997,7 +1059,7 @@ __global__ __launch_bounds__(AT_FWD_THREADS, 1) void sp_attn_fwd_kernel(
         at_block_addr(ad, kb, vb, vb, koff, voff);
       }
       at_step<false, true, 0, 0, 0, MODE>(ad, qb, sa, sb, pa, pb, o, scale_log2, m_run, det, ones,
-                                           c_prev == r, AT_SUB + 32, tq, l_mark, pre);
+                                           c_prev == r, AT_SUB + 32, tq, l_mark, pre, kq_prev);
       at_commit<MODE>(sb, pb, det, o, scale_log2, m_run, l_mark);
       at_pv_only<1, HALF>(vb, voff, pb, o, ones);
       emit(c_prev);
@@ -1285,23 +1347,161 @@ __global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_kernel(
     arow_out[c_done] = ((wred[par ^ 1][0] + wred[par ^ 1][1]) + (wred[par ^ 1][2] + wred[par ^ 1][3])) * inv_q;
 }
 
+// ---- block sizes below 128 ----------------------------------------------------------------------------
+// The caller's mask has one bit per f x f block (f = 128 >> fshift).  The forward kernel walks 128-key blocks: its
+// block mask is the OR over every group of (128 / f)^2 fine blocks.  One thread per 64-bit word of the coarse mask.
+__global__ __launch_bounds__(256) void sp_attn_coarsen_kernel(const uint64_t* __restrict__ fine, uint64_t* __restrict__ coarse,
+                                                              int hq, int nb, int nbw, int nbf, int nbfw, int fshift) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)hq * nb * nbw) return;
+  const int wc = (int)(i % nbw), r = (int)((i / nbw) % nb), h = (int)(i / ((int64_t)nbw * nb));
+  const int per = 1 << fshift;  // fine blocks per 128 tokens
+  uint64_t out = 0ull;
+  for (int fi = 0; fi < per; ++fi) {
+    const int fr = r * per + fi;
+    if (fr >= nbf) break;
+    const uint64_t* row = fine + ((int64_t)h * nbf + fr) * nbfw;
+    for (int t = 0; t < per; ++t) {  // fine word wc * per + t holds the coarse columns 64 wc + t (64 / per) ...
+      const int fw = wc * per + t;
+      if (fw >= nbfw) break;
+      const uint64_t w = row[fw];
+      for (int cb = 0; cb < (64 >> fshift); ++cb)
+        if ((w >> (cb << fshift)) & ((1ull << per) - 1ull)) out |= 1ull << (t * (64 >> fshift) + cb);
+    }
+  }
+  coarse[i] = out;
+}
+
+// Block-average maps of dense heads at a block size below 128 (shareprefill_attn.py:425-457): the recomputing pass of
+// sp_attn_avg_kernel with the sums kept per 16 x 16 cell of a 128 x 128 block, folded to f x f blocks at the end.
+// One workgroup per (128-query block, head); only fine blocks the mask keeps are computed into and written.
+__global__ __launch_bounds__(AT_THREADS) void sp_attn_avg_fine_kernel(
+    const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, const uint64_t* __restrict__ mask,
+    const uint64_t* __restrict__ fine_mask, const int32_t* __restrict__ decision, const float2* __restrict__ rowstat,
+    float* __restrict__ avg_attn, int64_t n, int hq, int hkv, int64_t sq_n, int64_t sq_h, int64_t sk_n, int64_t sk_h,
+    int nb, int nbw, int nbf, int nbfw, int fshift, float scale_log2) {
+  __shared__ __attribute__((aligned(16))) sp_bf16 Ks[AT_BS * AT_PITCH];
+  __shared__ float cell[AT_THREADS][8];  // per thread: its query's mass in the eight 16-key groups of the block
+  __shared__ float sum16[8][8];          // [16-query group][16-key group]
+  const int r = nb - 1 - blockIdx.x, h = blockIdx.y;
+  if (decision[h] != SP_DEC_DENSE) return;
+  const int kvh = h / (hq / hkv);
+  const int t = threadIdx.x;
+  const int wave = t >> 6, lane = t & 63;
+  const int lq = lane & 31, g = lane >> 5;
+  const int q_off = wave * 32 + lq;
+  const int lf = 7 - fshift;   // log2 of the block size
+  const int f = 1 << lf, per = 1 << fshift;
+  const int64_t rem = n - (int64_t)r * AT_BS;
+  const int valid_q = rem < AT_BS ? (int)rem : AT_BS;
+  const bool q_valid = q_off < valid_q;
+  int64_t qrow = (int64_t)r * AT_BS + q_off;
+  if (qrow > n - 1) qrow = n - 1;
+  bf16x8 qb[8];
+  {
+    const sp_bf16* src = q + (int64_t)h * sq_h + qrow * sq_n + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qb[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 16 * ks));
+  }
+  const float2 st = rowstat[(int64_t)h * n + qrow];
+  const float m_row = st.x, inv_l = 1.0f / st.y;
+  const sp_bf16* kh = k + (int64_t)kvh * sk_h;
+  const int fr_q = (int)(qrow >> lf);  // this thread's fine row
+  const uint64_t* frow = fine_mask + ((int64_t)h * nbf + fr_q) * nbfw;
+  AtBlocks it;
+  it.init(mask + ((int64_t)h * nb + r) * nbw, r);
+  for (int c = it.next(); c >= 0; c = it.next()) {
+    __syncthreads();  // the previous block's tile and cells are consumed
+    for (int i8 = 0; i8 < 8; ++i8) {
+      int64_t key = (int64_t)c * AT_BS + i8 * 16 + (t >> 4);
+      if (key > n - 1) key = n - 1;
+      *reinterpret_cast<at_u32x4*>(&Ks[(i8 * 16 + (t >> 4)) * AT_PITCH + (t & 15) * 8]) =
+          *reinterpret_cast<const at_u32x4*>(kh + key * sk_n + (t & 15) * 8);
+    }
+    __syncthreads();
+    const int fc0 = c << fshift;
+    const uint32_t rowbits = (uint32_t)(frow[fc0 >> 6] >> (fc0 & 63)) & ((1u << per) - 1u);  // this query's kept fine columns
+    float part[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      floatx16 acc = (floatx16){0};
+      const sp_bf16* arow = &Ks[(kt * 32 + lq) * AT_PITCH + 8 * g];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(arow + 16 * ks));
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qb[ks], acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key_off = kt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+        const bool ok = q_valid && (c < r || key_off <= q_off) && ((int64_t)c * AT_BS + key_off < n) &&
+                        ((rowbits >> (key_off >> lf)) & 1u);
+        const float pv = ok ? __builtin_amdgcn_exp2f(__builtin_fmaf(acc[i], scale_log2, -m_row)) : 0.f;
+        part[2 * kt + (i >> 3)] += pv;  // keys 8 (i / 4) + 4 g + i % 4 of the 32: below 16 for i < 8
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) cell[t][j] = part[j] * inv_l;
+    __syncthreads();
+    if (t < 64) {  // cell (16-query group t / 8, 16-key group t % 8): its 16 queries in ascending order
+      const int qg = t >> 3, kg = t & 7;
+      float sacc = 0.f;
+      for (int i = 0; i < 16; ++i) {
+        const int qo = 16 * qg + i;  // q_off of the thread that holds it: wave qo / 32, lq qo % 32, both g
+        const int tb = (qo >> 5) * 64 + (qo & 31);
+        sacc += cell[tb][kg] + cell[tb + 32][kg];
+      }
+      sum16[qg][kg] = sacc;
+    }
+    __syncthreads();
+    if (t < per * per) {  // fine block (fi, fj) of this 128 x 128 block
+      const int fi = t >> fshift, fj = t & (per - 1);
+      const int fr = r * per + fi, fc = fc0 + fj;
+      if (fr < nbf && fc < nbf && fc <= fr) {
+        const uint64_t* rw = fine_mask + ((int64_t)h * nbf + fr) * nbfw;
+        if ((rw[fc >> 6] >> (fc & 63)) & 1ull) {
+          const int cells = f >> 4;  // 16-wide cells per fine block side
+          float tot = 0.f;
+          for (int a = 0; a < cells; ++a)
+            for (int b2 = 0; b2 < cells; ++b2) tot += sum16[fi * cells + a][fj * cells + b2];
+          const int64_t left = n - (int64_t)fr * f;
+          const int rows = left < f ? (int)left : f;
+          avg_attn[((int64_t)h * nbf + fr) * nbf + fc] = tot / (float)rows;
+        }
+      }
+    }
+  }
+}
+
 // ---- host ---------------------------------------------------------------------------------------------
 // workspace layout: [ repacked V^T : hkv*nb*128*128 bf16 | scheduler area : 1 KiB of slots + 2 KiB order table |
 //                     row statistics : hq*n float2 ]
+// (the tiles are 128 keys wide whatever the caller's block size)
 static size_t at_vt_bytes(int64_t n, int32_t hkv, int32_t d, int32_t bs) {
-  return (size_t)hkv * (size_t)sp_ceil_div(n, bs) * bs * d * sizeof(sp_bf16);
+  (void)bs;
+  return (size_t)hkv * (size_t)sp_ceil_div(n, AT_BS) * AT_BS * d * sizeof(sp_bf16);
+}
+static inline bool at_block_size_ok(int32_t bs) { return bs == 128 || bs == 64 || bs == 32 || bs == 16; }
+static inline int at_fshift(int32_t bs) { return bs == 64 ? 1 : bs == 32 ? 2 : bs == 16 ? 3 : 0; }
+// block sizes below 128: the 128-block mask the kernels walk, behind the row statistics
+static size_t at_coarse_mask_bytes(int64_t n, int32_t hq, int32_t bs) {
+  if (bs == AT_BS) return 0;
+  const size_t nb = (size_t)sp_ceil_div(n, AT_BS);
+  return (size_t)hq * nb * ((nb + 63) / 64) * sizeof(uint64_t);
 }
 
 extern "C" size_t sp_attn_workspace_bytes(int64_t n, int32_t hq, int32_t hkv, int32_t d, int32_t bs) {
   if (n <= 0 || hq <= 0 || hkv <= 0 || d <= 0 || bs <= 0) return 0;
-  return at_vt_bytes(n, hkv, d, bs) + AT_SCHED_BYTES + (size_t)hq * (size_t)n * sizeof(float2);
+  return at_vt_bytes(n, hkv, d, bs) + AT_SCHED_BYTES + (size_t)hq * (size_t)n * sizeof(float2) +
+         at_coarse_mask_bytes(n, hq, bs);
 }
 
-// block sums of one pivot head: fp32 [nb*(nb+1)/2 lower-triangular blocks][128 queries]
+// block sums of one pivot head: fp32 [nb*(nb+1)/2 lower-triangular blocks][128 queries] (128-token blocks; a call
+// with a smaller block size keeps no block sums and ignores workspace beyond the base size)
 extern "C" size_t sp_attn_pivot_scratch_bytes(int64_t n, int32_t bs) {
   if (n <= 0 || bs <= 0) return 0;
-  const size_t nb = (size_t)sp_ceil_div(n, bs);
-  return nb * (nb + 1) / 2 * (size_t)bs * sizeof(float);
+  const size_t nb = (size_t)sp_ceil_div(n, AT_BS);
+  return nb * (nb + 1) / 2 * (size_t)AT_BS * sizeof(float);
 }
 
 extern "C" int sp_attn_last_launch_clocks(const void* workspace, int64_t n, int32_t hkv, int32_t d, int32_t bs,
@@ -1329,14 +1529,14 @@ extern "C" int sp_attn_repack_v_bf16(const void* v, int64_t n, int32_t hkv, int3
                                      sp_stream_t stream) {
   SP_REQUIRE(v && workspace, SP_ERR_INVALID_ARGUMENT, "sp_attn_repack_v_bf16: null pointer");
   SP_REQUIRE(n > 0 && hkv > 0, SP_ERR_INVALID_ARGUMENT, "sp_attn_repack_v_bf16: bad shape");
-  SP_REQUIRE(bs == AT_BS && d == AT_D, SP_ERR_UNSUPPORTED,
-             "sp_attn_repack_v_bf16: block size %d / head_dim %d unsupported (only 128 / 128)", bs, d);
+  SP_REQUIRE(at_block_size_ok(bs) && d == AT_D, SP_ERR_UNSUPPORTED,
+             "sp_attn_repack_v_bf16: block size %d / head_dim %d unsupported (16, 32, 64 or 128 / 128)", bs, d);
   SP_REQUIRE(v_stride_n % 8 == 0 && v_stride_h % 8 == 0 && ((uintptr_t)v % 16) == 0 &&
                  ((uintptr_t)workspace % 16) == 0,
              SP_ERR_UNSUPPORTED, "sp_attn_repack_v_bf16: v must be 16-byte aligned, strides multiple of 8");
   SP_REQUIRE(workspace_bytes >= at_vt_bytes(n, hkv, d, bs), SP_ERR_WORKSPACE,
              "sp_attn_repack_v_bf16: workspace too small");
-  const int64_t nb = sp_ceil_div(n, bs);
+  const int64_t nb = sp_ceil_div(n, AT_BS);
   hipLaunchKernelGGL(sp_repack_v_kernel, dim3((unsigned)nb, hkv), dim3(AT_THREADS), 0, (hipStream_t)stream,
                      (const sp_bf16*)v, (sp_bf16*)workspace, n, v_stride_n, v_stride_h, nb);
   SP_LAUNCH_CHECK();
@@ -1357,8 +1557,8 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   SP_REQUIRE(hq <= AT_MAX_HEADS, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: more than %d query heads",
              AT_MAX_HEADS);
   SP_REQUIRE(softmax_scale > 0.f, SP_ERR_INVALID_ARGUMENT, "sp_block_sparse_attn_fwd_bf16: softmax_scale must be > 0");
-  SP_REQUIRE(bs == AT_BS, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: block size %d unsupported (only 128)",
-             bs);
+  SP_REQUIRE(at_block_size_ok(bs), SP_ERR_UNSUPPORTED,
+             "sp_block_sparse_attn_fwd_bf16: block size %d unsupported (16, 32, 64 or 128)", bs);
   SP_REQUIRE(d == AT_D, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: head_dim %d unsupported (only 128)", d);
   SP_REQUIRE(q_stride_n % 8 == 0 && q_stride_h % 8 == 0 && k_stride_n % 8 == 0 && k_stride_h % 8 == 0 &&
                  ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)out % 16) == 0,
@@ -1367,7 +1567,12 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
              "sp_block_sparse_attn_fwd_bf16: key token stride %lld too large", (long long)k_stride_n);
   SP_REQUIRE(workspace_bytes >= sp_attn_workspace_bytes(n, hq, hkv, d, bs), SP_ERR_WORKSPACE,
              "sp_block_sparse_attn_fwd_bf16: workspace too small");
-  const int64_t nb = sp_ceil_div(n, bs);
+  // nb: 128-token blocks, what the kernels walk; nbf: blocks of the caller's size, what `mask` and `avg_attn` index
+  const int64_t nb = sp_ceil_div(n, AT_BS), nbf = sp_ceil_div(n, bs);
+  const bool fine = bs != AT_BS;
+  const int fshift = at_fshift(bs);
+  SP_REQUIRE(nbf <= 4096, SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: %lld blocks of %d tokens exceed 4096",
+             (long long)nbf, bs);
   SP_REQUIRE(nb * hq < (1ll << 31), SP_ERR_UNSUPPORTED, "sp_block_sparse_attn_fwd_bf16: grid too large");
   SP_REQUIRE(nb <= AT_LIST_MAX, SP_ERR_UNSUPPORTED,
              "sp_block_sparse_attn_fwd_bf16: %lld key blocks exceed the supported %d (sequence too long)", (long long)nb,
@@ -1382,6 +1587,17 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   float2* rowstat = reinterpret_cast<float2*>(ws + at_vt_bytes(n, hkv, d, bs) + AT_SCHED_BYTES);
   const bool want_avg = decision != nullptr && avg_attn != nullptr;
   hipStream_t s = (hipStream_t)stream;
+  const uint64_t* const fine_mask = mask;  // the caller's mask, at the caller's block size
+  const int nbfw = (int)((nbf + 63) / 64);
+  if (fine) {
+    uint64_t* coarse = reinterpret_cast<uint64_t*>(ws + at_vt_bytes(n, hkv, d, bs) + AT_SCHED_BYTES +
+                                                   (size_t)hq * (size_t)n * sizeof(float2));
+    const int64_t words = (int64_t)hq * nb * ((nb + 63) / 64);
+    hipLaunchKernelGGL(sp_attn_coarsen_kernel, dim3((unsigned)sp_ceil_div(words, 256)), dim3(256), 0, s, fine_mask,
+                       coarse, (int)hq, (int)nb, (int)((nb + 63) / 64), (int)nbf, nbfw, fshift);
+    SP_LAUNCH_CHECK();
+    mask = coarse;  // from here on `mask` is the 128-block mask
+  }
   // Workspace beyond the base size holds the block sums of pivot heads, one slab per pivot: those heads run in a
   // launch of their own that keeps the sums, and their block-average maps are made from them; pivots beyond the
   // slabs (or all of them, with a base-size workspace) take the recomputing pass.
@@ -1389,7 +1605,7 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   const size_t base_aligned = (base_bytes + 255) & ~(size_t)255;
   const size_t slab = sp_attn_pivot_scratch_bytes(n, bs);
   int max_pivots = 0;
-  if (want_avg && workspace_bytes > base_aligned) {
+  if (want_avg && workspace_bytes > base_aligned && !fine) {
     const size_t fit = (workspace_bytes - base_aligned) / slab;
     max_pivots = fit > (size_t)(AT_NO_SLOT - 1) ? AT_NO_SLOT - 1 : (int)fit;
   }
@@ -1422,8 +1638,9 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
   if (cu_of_device[dev] == 0) {
     hipDeviceProp_t prop;
     SP_HIP(hipGetDeviceProperties(&prop, dev));
-    const void* fwd_kernels[4] = {(const void*)sp_attn_fwd_kernel<false, false>, (const void*)sp_attn_fwd_kernel<true, false>,
-                                  (const void*)sp_attn_fwd_kernel<false, true>, (const void*)sp_attn_fwd_kernel<true, true>};
+    const void* fwd_kernels[5] = {(const void*)sp_attn_fwd_kernel<false, false>, (const void*)sp_attn_fwd_kernel<true, false>,
+                                  (const void*)sp_attn_fwd_kernel<false, true>, (const void*)sp_attn_fwd_kernel<true, true>,
+                                  (const void*)sp_attn_fwd_kernel<false, false, true>};
     for (const void* f : fwd_kernels)
       SP_HIP(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     cu_of_device[dev] = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
@@ -1437,9 +1654,11 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(AT_FWD_THREADS), lds_bytes, s, (const sp_bf16*)q, (const sp_bf16*)k,
                        (const sp_bf16*)workspace, mask, decision, (sp_bf16*)out, stats, n, hq, hkv, q_stride_n,
                        q_stride_h, k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, counter,
-                       skip_slotted, block_sums);
+                       skip_slotted, block_sums, fine_mask, fshift, (int)nbf, nbfw);
   };
-  if (half)
+  if (fine)  // (one instance: a head_dim below 128 computes its zero channels here)
+    launch_fwd(sp_attn_fwd_kernel<false, false, true>, 0, (float*)nullptr);
+  else if (half)
     launch_fwd(sp_attn_fwd_kernel<false, true>, max_pivots > 0 ? 1 : 0, (float*)nullptr);
   else
     launch_fwd(sp_attn_fwd_kernel<false, false>, max_pivots > 0 ? 1 : 0, (float*)nullptr);
@@ -1451,7 +1670,13 @@ extern "C" int sp_block_sparse_attn_fwd_bf16(const void* q, const void* k, const
       launch_fwd(sp_attn_fwd_kernel<true, false>, 0, pivot_u);
     SP_LAUNCH_CHECK();
   }
-  if (want_avg) {
+  if (want_avg && fine) {
+    hipLaunchKernelGGL(sp_attn_avg_fine_kernel, dim3((unsigned)nb, hq), dim3(AT_THREADS), 0, s, (const sp_bf16*)q,
+                       (const sp_bf16*)k, mask, fine_mask, decision, rowstat, avg_attn, n, hq, hkv, q_stride_n,
+                       q_stride_h, k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), (int)nbf, nbfw, fshift,
+                       scale_log2);
+    SP_LAUNCH_CHECK();
+  } else if (want_avg) {
     hipLaunchKernelGGL(sp_attn_avg_kernel, dim3((unsigned)nb, hq), dim3(AT_THREADS), 0, s, (const sp_bf16*)q,
                        (const sp_bf16*)k, mask, decision, rowstat, avg_attn, n, hq, hkv, q_stride_n, q_stride_h,
                        k_stride_n, k_stride_h, (int)nb, (int)((nb + 63) / 64), scale_log2, (const int*)counter,

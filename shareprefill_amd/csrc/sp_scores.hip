@@ -319,7 +319,7 @@ __global__ __launch_bounds__(LQ_WG_THREADS, 2) void sp_lastq_probs_kernel(
     const sp_bf16* __restrict__ q, const sp_bf16* __restrict__ k, int64_t n, int hkv, int group, int64_t sq_n,
     int64_t sq_h, int64_t sk_n, int64_t sk_h, float inv_sqrt_d, uint32_t flags, const float2* __restrict__ rowstat,
     float* __restrict__ vert_tok, float* __restrict__ slash_tok, float* __restrict__ vert_blk,
-    float* __restrict__ slash_blk, int64_t nb, int tiles_per_wg) {
+    float* __restrict__ slash_blk, int64_t nb, int tiles_per_wg, int bs) {
   extern __shared__ __attribute__((aligned(1024))) char lqp_lds[];
   char* R2 = lqp_lds;  // [2][LQ_KSW_BYTES]
   const int pairs = lq_pairs(group);
@@ -338,15 +338,19 @@ __global__ __launch_bounds__(LQ_WG_THREADS, 2) void sp_lastq_probs_kernel(
   lq_load_q<true>(qh, n, sq_n, wave, lane, inv_sqrt_d, qa);
   // per row: max + log2(sum), so that a probability is exp2(logit * log2 e - rm): the normalisation rides in the
   // exponent instead of costing a multiplication per element
+  // A block size below 128 has its last block's queries in the tail of the 128 rows: the rows in front of them get
+  // rm = +inf, so that every probability of theirs is exp2(-inf) = 0, and the means divide by bs.
   float rm[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const float2 st = rowstat[h * LQ_ROWS + (LQ_ROWS - 1 - lq_row_of(wave, lane, r))];
-    rm[r] = st.x - __builtin_amdgcn_logf(st.y);  // st.y = 1 / sum; v_log_f32 is log2
+    const int qi = LQ_ROWS - 1 - lq_row_of(wave, lane, r);  // query index inside the last 128 tokens
+    const float2 st = rowstat[h * LQ_ROWS + qi];
+    rm[r] = qi >= LQ_ROWS - bs ? st.x - __builtin_amdgcn_logf(st.y) : INFINITY;  // st.y = 1 / sum; v_log_f32 is log2
   }
   const int64_t n_tiles = sp_ceil_div(n, LQ_TILE);
   const int64_t first = (int64_t)blockIdx.x * tiles_per_wg;
-  const float inv_rows = 1.0f / (float)LQ_ROWS;
+  const float inv_rows = 1.0f / (float)bs;
+  const bool write_blk = bs == LQ_ROWS;  // the block sums of smaller blocks come from sp_lastq_block_sums_kernel
   const int64_t t_begin = first > 0 ? first - 1 : 0;
   const int64_t t_end = first + tiles_per_wg < n_tiles ? first + tiles_per_wg : n_tiles;
   float* Dm = L.D;
@@ -367,7 +371,7 @@ __global__ __launch_bounds__(LQ_WG_THREADS, 2) void sp_lastq_probs_kernel(
     __syncthreads();  // ... and everyone's; the previous tile's K reads and digest reads are done
     if (tile + 1 < t_end)  // the next K tile, into the buffer the previous tile has left
       lq_issue_k_direct<2>(kh, n, sk_n, kb + LQ_TILE, R2 + (par ^ 1) * LQ_KSW_BYTES, wave8, lane, kl);
-    if (tid == 0 && tile > first && has_head) {  // the previous tile's block sums: its parts were complete one barrier ago
+    if (tid == 0 && tile > first && has_head && write_blk) {  // the previous tile's block sums: its parts were complete one barrier ago
       const float* bp = &L.bpart[par ^ 1][0][0];
       slash_blk[(int64_t)h * nb + tile - 1] = bp[0] + bp[1];
       vert_blk[(int64_t)h * nb + tile - 1] = (bp[4] + bp[5]) + (bp[6] + bp[7]);
@@ -506,11 +510,31 @@ __global__ __launch_bounds__(LQ_WG_THREADS, 2) void sp_lastq_probs_kernel(
     }
   }
   __syncthreads();
-  if (tid == 0 && t_end > first && has_head) {  // the last tile's block sums
+  if (tid == 0 && t_end > first && has_head && write_blk) {  // the last tile's block sums
     const float* bp = &L.bpart[(t_end - 1) & 1][0][0];
     slash_blk[(int64_t)h * nb + t_end - 1] = bp[0] + bp[1];
     vert_blk[(int64_t)h * nb + t_end - 1] = (bp[4] + bp[5]) + (bp[6] + bp[7]);
   }
+}
+
+// Block sums of the token vectors for block sizes below 128 (torch_bhn_sumpool, utils.py:33-44): one thread per
+// (head, block) adds its bs tokens in ascending order; tokens beyond the sequence count as zero.
+__global__ __launch_bounds__(256) void sp_lastq_block_sums_kernel(const float* __restrict__ vert_tok,
+                                                                  const float* __restrict__ slash_tok, int64_t n,
+                                                                  int64_t nb, int bs, int64_t total,
+                                                                  float* __restrict__ vert_blk,
+                                                                  float* __restrict__ slash_blk) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // h * nb + block
+  if (i >= total) return;
+  const int64_t h = i / nb, b = i % nb;
+  const int64_t t0 = b * bs, t1 = t0 + bs < n ? t0 + bs : n;
+  float sv = 0.f, ss = 0.f;
+  for (int64_t t = t0; t < t1; ++t) {
+    sv += vert_tok[h * n + t];
+    ss += slash_tok[h * n + t];
+  }
+  vert_blk[i] = sv;
+  slash_blk[i] = ss;
 }
 
 // ---- pooled block probabilities of query-aware heads (attention_sharing.py:350-360) -------------------------------
@@ -744,10 +768,15 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
              "sp_lastq_scores_bf16: null pointer");
   SP_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0, SP_ERR_INVALID_ARGUMENT,
              "sp_lastq_scores_bf16: hq=%d must be a positive multiple of hkv=%d", hq, hkv);
-  SP_REQUIRE(bs == LQ_ROWS, SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: block size %d unsupported (only 128)", bs);
+  SP_REQUIRE(bs == 128 || bs == 64 || bs == 32 || bs == 16, SP_ERR_UNSUPPORTED,
+             "sp_lastq_scores_bf16: block size %d unsupported (16, 32, 64 or 128)", bs);
   SP_REQUIRE(d == LQ_D, SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: head_dim %d unsupported (only 128)", d);
   SP_REQUIRE(n >= bs, SP_ERR_INVALID_ARGUMENT, "sp_lastq_scores_bf16: seq_len %lld is shorter than one block",
              (long long)n);
+  // the kernels always work on the last 128 tokens' queries and drop the rows a smaller block does not have
+  SP_REQUIRE(n >= LQ_ROWS, SP_ERR_UNSUPPORTED,
+             "sp_lastq_scores_bf16: seq_len %lld is shorter than %d tokens (needed for block sizes below 128 too)",
+             (long long)n, LQ_ROWS);
   SP_REQUIRE(q_stride_n % 8 == 0 && q_stride_h % 8 == 0 && k_stride_n % 8 == 0 && k_stride_h % 8 == 0 &&
                  ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0,
              SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: q/k must be 16-byte aligned with strides multiple of 8");
@@ -755,7 +784,8 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
              "sp_lastq_scores_bf16: workspace too small");
   const int tiles_per_wg = lq_tiles_per_wg(n, hq);
   const int n_chunks = (int)sp_ceil_div(sp_ceil_div(n, LQ_TILE), tiles_per_wg);
-  const int64_t nb = sp_ceil_div(n, bs);
+  const int64_t nb = sp_ceil_div(n, bs);          // blocks of the caller's size: the length of vert_blk / slash_blk
+  const int64_t nb_tiles = sp_ceil_div(n, LQ_TILE);  // 128-token tiles the kernels walk
   float2* partial = (float2*)workspace;
   float2* rowstat = partial + (size_t)hq * lq_chunks(n, hq) * LQ_ROWS;
   const float inv_sqrt_d = sp_inv_sqrt_dim(flags, d);
@@ -778,11 +808,17 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
                                (int)LQP_LDS_BYTES));
     attr_set[dev] = true;
   }
-  const int tiles_probs = lq_probs_tiles_per_wg(nb, wg_rows);
-  const int grid_x = (int)sp_ceil_div(nb, tiles_probs);
+  const int tiles_probs = lq_probs_tiles_per_wg(nb_tiles, wg_rows);
+  const int grid_x = (int)sp_ceil_div(nb_tiles, tiles_probs);
   hipLaunchKernelGGL(sp_lastq_probs_kernel, dim3(grid_x, wg_rows), dim3(LQ_WG_THREADS), LQP_LDS_BYTES, s, (const sp_bf16*)q,
                      (const sp_bf16*)k, n, hkv, group, q_stride_n, q_stride_h, k_stride_n, k_stride_h, inv_sqrt_d,
-                     flags, rowstat, vert_tok, slash_tok, vert_blk, slash_blk, nb, tiles_probs);
+                     flags, rowstat, vert_tok, slash_tok, vert_blk, slash_blk, nb_tiles, tiles_probs, (int)bs);
   SP_LAUNCH_CHECK();
+  if (bs != LQ_ROWS) {
+    const int64_t total = (int64_t)hq * nb;
+    hipLaunchKernelGGL(sp_lastq_block_sums_kernel, dim3((unsigned)sp_ceil_div(total, 256)), dim3(256), 0, s, vert_tok,
+                       slash_tok, n, nb, (int)bs, total, vert_blk, slash_blk);
+    SP_LAUNCH_CHECK();
+  }
   return SP_OK;
 }

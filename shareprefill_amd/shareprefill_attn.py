@@ -86,13 +86,16 @@ def triton_block_wise_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: tor
     heads_need_blockwise_attn_mask bool [B, Hq]: the heads whose block-average attention map is wanted.
     Returns (out [B, N, Hq, D] bf16, avg_attn fp32 [B, Hq, nb, nb], zero for the other heads).
     gqa_interleave: query head h reads kv head h % Hkv instead of h // (Hq / Hkv) (shareprefill_attn.py:333-336).
-    Only grid_offset == 0 and block_size 128 are built; head_dim 16 / 32 / 64 run zero-padded to 128 (pad_head_dim)."""
+    block_size 16 / 32 / 64 / 128 as in the reference (:509-516); below 128 the kernel walks the 128-token blocks that
+    hold an activated block and drops the rest of each per 16 x 16 sub-tile: exact, not tuned.  Only grid_offset == 0
+    is built; head_dim 16 / 32 / 64 run zero-padded to 128 (pad_head_dim)."""
     batch_size, q_len, num_q_heads, model_dim = q.shape
     _, k_len, num_kv_heads, _ = k.shape
     assert q.dtype == torch.bfloat16
     assert q_len == k_len
     assert num_q_heads % num_kv_heads == 0
     assert model_dim in PADDED_HEAD_DIMS + (KERNEL_HEAD_DIM,), "only support head_dim in {16, 32, 64, 128}"
+    assert block_size in (16, 32, 64, 128), "only support block_size in {16, 32, 64, 128}"
     if model_dim != KERNEL_HEAD_DIM:
         q, k, v = pad_head_dim(q, k, v)
     head_dim = q.shape[-1]

@@ -60,7 +60,8 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_fre
     oracle_forced = O.OracleSharing(O.ClusterTable(table["clusters"], table["shared_clusters"]))
     oracle_free = O.OracleSharing(O.ClusterTable(table["clusters"], table["shared_clusters"]))
     qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
-    nb = -(-n // 128)
+    bs = kw["block_size"]
+    nb = -(-n // bs)
     results = []
     for layer in (range(n_layers) if layer_ids is None else layer_ids):
         if reseed:
@@ -77,7 +78,7 @@ def run_layers(gpu, tmp_path, hq, hkv, n, seed, n_clusters, n_layers=2, with_fre
                       slash_blk=plan.slash_blk.cpu(), avg_qk=plan.avg_qk.cpu(), js_qa=plan.js_qa.cpu(),
                       js_v=plan.js_v.cpu().numpy(), js_s=plan.js_s.cpu().numpy(),
                       qa_probs={h: plan.qa_probs[h].cpu() for h in range(hq)})
-        okw = dict(bs=128, min_budget=kw["min_budget"], max_budget=kw["max_budget"],
+        okw = dict(bs=bs, min_budget=kw["min_budget"], max_budget=kw["max_budget"],
                    pattern_threshold=kw["pattern_threshold"], similarity_threshold=kw["similarity_threshold"],
                    fallback_threshold=kw["fallback_threshold"], queryaware_threshold=kw["queryaware_threshold"])
         forced = None
@@ -163,7 +164,7 @@ def check_outputs(run):
     for L in run["layers"]:
         q, k, v = L["q"], L["k"], L["v"]
         want = L["dec"] == O.DEC_DENSE
-        ref, avg_ref = O.masked_attention(q, k, v, L["mask"], 128, run["d"] ** -0.5, want_avg=want)
+        ref, avg_ref = O.masked_attention(q, k, v, L["mask"], run["kw"]["block_size"], run["d"] ** -0.5, want_avg=want)
         out = L["out"][0].transpose(0, 1).float()
         assert (out - ref).abs().max().item() <= MAX_ABS
         assert ((out - ref).abs().mean() / ref.abs().mean()).item() <= MEAN_REL
@@ -181,6 +182,33 @@ def test_layer_default_thresholds_small(gpu_device, tmp_path):
     check_outputs(run)
     d0 = run["layers"][0]["dec"]
     assert (d0 == O.DEC_DENSE).sum() == 2  # one pivot per shared cluster in the first layer
+
+
+@pytest.mark.parametrize("bs,n,hq,hkv", [(64, 2048, 8, 2), (64, 1100, 6, 2), (32, 1536, 8, 2), (32, 999, 4, 4),
+                                         (16, 1024, 8, 2), (16, 777, 7, 1)])
+def test_layer_smaller_block_sizes(gpu_device, tmp_path, bs, n, hq, hkv):
+    """block_size 64 / 32 / 16 (shareprefill_attn.py:509-516): the selection runs on N / bs blocks, the attention
+    kernel walks the 128-token blocks that hold a kept block and drops the rest of them per 16 x 16 sub-tile.  Three
+    layers (pivot election, sharing tests, pivot update), budgets / decisions / masks / pivot state forced against
+    the oracle, float stages and outputs to the bars of the 128 case, with thresholds under which heads share and go
+    query-aware."""
+    n_clusters = 2 if hq % 2 == 0 else 1
+    seen = []
+    for qa_thr in (0.0, 1e9):  # nobody query-aware: pivots and their sharers; then every head query-aware
+        run = run_layers(gpu_device, tmp_path, hq=hq, hkv=hkv, n=n, seed=500 + bs + n, n_clusters=n_clusters,
+                         n_layers=3, block_size=bs, min_budget=4 * bs, fallback_threshold=1e9,
+                         similarity_threshold=0.9, queryaware_threshold=qa_thr)
+        assert run["nb"] == -(-n // bs)
+        check_forced(run)
+        check_free(run, expect_same_masks=False)
+        check_outputs(run)
+        seen.append(np.concatenate([L["dec"] for L in run["layers"]]))
+    assert (seen[0] == O.DEC_DENSE).any() and (seen[0] == O.DEC_SHARE).any() and (seen[1] == O.DEC_QA).any()
+    # default thresholds as well
+    run = run_layers(gpu_device, tmp_path, hq=hq, hkv=hkv, n=n, seed=600 + bs + n, n_clusters=n_clusters,
+                     block_size=bs, min_budget=8 * bs)
+    check_forced(run)
+    check_outputs(run)
 
 
 @pytest.mark.parametrize("d,n", [(64, 2048), (32, 1100), (16, 1536)])

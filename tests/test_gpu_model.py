@@ -103,6 +103,41 @@ def test_patched_model_with_head_dim_64(gpu_device, tmp_path):
     assert torch.equal(gen, want)
 
 
+@pytest.mark.parametrize("block_size,head_dim", [(64, 128), (32, 128), (16, 64)])
+def test_patched_model_with_smaller_block_sizes(gpu_device, tmp_path, block_size, head_dim):
+    """block_size 64 / 32 / 16 through SharePrefill(...)(model) (shareprefill_configurations.py:37,
+    shareprefill_attn.py:509-516), the last together with a head_dim of 64: with budgets that keep every block the
+    patched model matches the eager one; with sparse budgets the selection runs on the finer grid, and the dense
+    short-prompt shortcut and decode work."""
+    from shareprefill_amd import SharePrefill
+
+    ids = torch.randint(0, 512, (1, 1100), generator=torch.Generator().manual_seed(block_size)).to(gpu_device)
+    ref_model = small_llama(head_dim=head_dim).to(gpu_device, torch.bfloat16)
+    ref_model.config._attn_implementation = "eager"
+    with torch.no_grad():
+        ref = ref_model(ids).logits.float()
+    for shortcut in (True, False):
+        model = SharePrefill(sharing_lookup_path=table(tmp_path, 2, 4), min_budget=8192, block_size=block_size,
+                             dense_short_prompts=shortcut)(small_llama(head_dim=head_dim).to(gpu_device, torch.bfloat16))
+        with torch.no_grad():
+            out = model(ids, use_cache=False).logits.float()
+        assert (out - ref).abs().max().item() < 0.15 and ((out - ref).abs().mean() / ref.abs().mean()).item() < 2e-2
+    assert sum(model.attention_sharing.decision_histogram().values()) == 8
+    sparse = SharePrefill(sharing_lookup_path=table(tmp_path, 2, 4), pattern_threshold=0.9, min_budget=2 * block_size,
+                          block_size=block_size)(small_llama(head_dim=head_dim).to(gpu_device, torch.bfloat16))
+    sparse.attention_sharing.keep_plans = True
+    with torch.no_grad():
+        logits = sparse(ids, use_cache=False, logits_to_keep=1).logits
+    assert torch.isfinite(logits).all()
+    nb = -(-1100 // block_size)
+    plans = sparse.attention_sharing.plans
+    assert len(plans) == 2 and all(p.mask.shape[1] == nb for p in plans)
+    assert all((p.density().cpu() < 1).any() for p in plans)
+    with torch.no_grad():
+        gen = sparse.generate(ids[:, :block_size + 5], max_new_tokens=3, do_sample=False)
+    assert gen.shape == (1, block_size + 8)
+
+
 def test_patched_qwen2_model_prefill_and_generate(gpu_device, tmp_path):
     """The patch is model-agnostic (any module with ALL_ATTENTION_FUNCTIONS): Qwen2's attention layer passes
     sliding_window=None for its full-attention layers and has q/k/v biases."""

@@ -97,6 +97,41 @@ def test_block_idx_to_mask_round_trip(gpu_device):
             assert torch.equal(back[h].cpu(), lists[h])
 
 
+@pytest.mark.parametrize("bs", [64, 32, 16])
+@pytest.mark.parametrize("hq,hkv,n,density", [(4, 2, 1024, 0.3), (6, 2, 1111, 0.6), (4, 4, 333, 0.1), (7, 1, 640, 1.0)])
+def test_block_wise_prefill_attention_smaller_block_sizes(gpu_device, bs, hq, hkv, n, density):
+    """The wrapper's other block sizes (shareprefill_attn.py:509-516): ids on the N / bs grid, outputs and the wanted
+    heads' block-average maps [nb, nb] against the oracle at that block size; a fully masked stretch of a visited
+    128-token block must contribute nothing."""
+    from shareprefill.attn.shareprefill_attn import triton_block_wise_prefill_attention
+
+    g = torch.Generator().manual_seed(n + bs)
+    mk = lambda h: torch.randn(1, n, h, 128, generator=g).to(torch.bfloat16)
+    q, k, v = mk(hq), mk(hkv), mk(hkv)
+    nb = -(-n // bs)
+    mask = _random_mask(hq, nb, n + bs, density)
+    need = torch.zeros(1, hq, dtype=torch.bool)
+    need[0, 0] = True
+    need[0, hq - 1] = True
+    block_idx = [[t.to(gpu_device) for t in _ids_from_mask(mask)]]
+    out, avg = triton_block_wise_prefill_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), block_idx,
+                                                   need.to(gpu_device), bs)
+    assert out.shape == (1, n, hq, 128) and avg.shape == (1, hq, nb, nb)
+    qh, kh, vh = (t[0].transpose(0, 1) for t in (q, k, v))
+    ref, ref_avg = O.masked_attention(qh, kh, vh, mask, bs, 1.0 / math.sqrt(128), want_avg=need[0].numpy())
+    o = out[0].cpu().float().transpose(0, 1)
+    assert (o - ref).abs().max().item() <= 2e-2
+    assert ((o - ref).abs().mean() / ref.abs().mean()).item() <= 2.5e-3
+    a = avg[0].cpu()
+    for h in range(hq):
+        if need[0, h]:
+            assert (a[h] - ref_avg[h]).abs().max().item() <= 2e-3
+            np.testing.assert_allclose(a[h].sum(-1).numpy(), 1.0, atol=2e-3)
+            assert (a[h][~torch.from_numpy(mask[h])] == 0).all()
+        else:
+            assert a[h].abs().max().item() == 0.0
+
+
 @pytest.mark.parametrize("hq,hkv,n,as_tensor", [(4, 2, 1024, False), (8, 2, 1500, True), (4, 4, 640, False)])
 def test_block_wise_prefill_attention_reference_signature(gpu_device, hq, hkv, n, as_tensor):
     from shareprefill.attn.shareprefill_attn import triton_block_wise_prefill_attention
@@ -189,8 +224,8 @@ def test_block_wise_prefill_attention_rejects_what_is_not_built(gpu_device):
         triton_block_wise_prefill_attention(q, q, q, idx, need, 128, grid_offset=64)
     with pytest.raises(AssertionError):
         triton_block_wise_prefill_attention(q.float(), q.float(), q.float(), idx, need, 128)
-    with pytest.raises(NotImplementedError, match="block size"):
-        triton_block_wise_prefill_attention(q, q, q, idx, need, 64)
+    with pytest.raises(AssertionError, match="block_size"):  # (the reference asserts the same set, :509-516)
+        triton_block_wise_prefill_attention(q, q, q, idx, need, 48)
 
 
 @pytest.mark.parametrize("b,n,h,d,ks", [(1, 1000, 4, 128, 128), (2, 300, 3, 64, 64), (1, 128, 8, 128, 128)])

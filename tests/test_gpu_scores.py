@@ -61,6 +61,31 @@ def test_lastq_scores_seeded_random_shapes(gpu_device):
         assert torch.allclose(sb, O.block_sum(st, 128), rtol=1e-5, atol=1e-9), tag
 
 
+@pytest.mark.parametrize("bs", [64, 32, 16])
+@pytest.mark.parametrize("hq,hkv,n", [(4, 2, 1024), (6, 2, 1000), (7, 1, 389), (2, 1, 128), (4, 4, 2100)])
+def test_lastq_scores_smaller_block_sizes(gpu_device, bs, hq, hkv, n):
+    """Block sizes below 128 (attention_sharing.py:127: the last bs queries): the same kernels with the rows in front
+    of the last bs masked out; token vectors against the oracle with fp32 logits, block sums of bs tokens."""
+    from shareprefill_amd import ops
+
+    q, k = _inputs(hq, hkv, n, 77 + n + bs)
+    vref, sref = O.lastq_scores(q, k, bs, logits_in_input_dtype=False)
+    vt, st, vb, sb = [x.cpu() for x in ops.lastq_scores(q.to(gpu_device), k.to(gpu_device), bs, 0)]
+    nb = -(-n // bs)
+    assert vb.shape == (hq, nb) and sb.shape == (hq, nb)
+    assert torch.allclose(vt, vref, rtol=2e-4, atol=1e-8)
+    assert torch.allclose(st, sref, rtol=2e-4, atol=1e-8)
+    assert torch.allclose(vt.sum(-1), torch.ones(hq), atol=1e-4)
+    assert torch.allclose(vb, O.block_sum(vt, bs), rtol=1e-5, atol=1e-9)
+    assert torch.allclose(sb, O.block_sum(st, bs), rtol=1e-5, atol=1e-9)
+    # the reference's bf16 logits as well: a logit on the other side of a bf16 rounding boundary (one ulp of a logit
+    # of magnitude 8 is 0.03) moves its probability by 3 %, and a slash bin near the end holds few elements
+    vref, sref = O.lastq_scores(q, k, bs, logits_in_input_dtype=True)
+    vt, st, _, _ = [x.cpu() for x in ops.lastq_scores(q.to(gpu_device), k.to(gpu_device), bs)]
+    assert torch.allclose(vt, vref, rtol=8e-2, atol=1e-6)
+    assert torch.allclose(st, sref, rtol=8e-2, atol=1e-6)
+
+
 def test_lastq_scores_head_major_layout_and_determinism(gpu_device):
     from shareprefill_amd import ops
 
