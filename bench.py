@@ -407,11 +407,12 @@ def timed_layer_point(w, q, k, v, table, pt, steps=5, n_tokens=None, with_stages
     ams = sum(tm.durations_ms("attn")) / steps
     plan = sh.plans[-1]
     kept = int(ops.mask_row_pointers(plan.mask)[:, -1].sum())
+    flop_per_block = 4.0 * w.block_size * w.block_size * w.head_dim  # (FLOP_PER_BLOCK at the path's block size 128)
     out = {"pattern_threshold": pt, "tokens": n, "kept_blocks": kept, "density": round(kept / tri, 4),
            "layer_ms": round(ms, 3), "attn_ms": round(ams, 3),
-           "attn_tflops": round(kept * FLOP_PER_BLOCK / ams / 1e9, 1),
-           "attn_frac_of_peak": round(kept * FLOP_PER_BLOCK / ams / 1e9 / PEAK_BF16_TFLOPS, 4),
-           "layer_frac_of_peak": round(kept * FLOP_PER_BLOCK / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+           "attn_tflops": round(kept * flop_per_block / ams / 1e9, 1),
+           "attn_frac_of_peak": round(kept * flop_per_block / ams / 1e9 / PEAK_BF16_TFLOPS, 4),
+           "layer_frac_of_peak": round(kept * flop_per_block / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
     if with_stages:
         qh, kh, vh = q[0], k[0], v[0]
         minb = math.ceil(w.min_budget / w.block_size)
@@ -653,6 +654,18 @@ def main():
                                    w2.pattern_threshold, steps=10, with_stages=True)
             c2["workload"] = "C2: B1 Hq32 Hkv8 D128 N32768 bf16, seed %d" % w2.seed
             line["c2_layer"] = c2
+            # the reference's other block sizes (shareprefill_attn.py:509-516) on the same inputs: a compatibility path
+            # on the 128-token kernels, timed so that its cost is on record (TFLOP/s counted on the kept fine blocks)
+            import dataclasses
+
+            small = []
+            for bs in (64, 32, 16):
+                wb = dataclasses.replace(w2, block_size=bs)
+                pnt = timed_layer_point(wb, q2, k2, v2, synthetic.random_cluster_table(w2.hq, w2.n_clusters, 2, w2.seed),
+                                        w2.pattern_threshold, steps=5)
+                pnt["block_size"] = bs
+                small.append(pnt)
+            line["c2_smaller_block_sizes"] = small
             del q2, k2, v2
         line["sharing_layer"] = sharing_layer_variant(args, w, pt, q, k, v, table)
 

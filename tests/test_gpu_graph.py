@@ -20,14 +20,15 @@ class _Module:
         self.training, self.attention_dropout = False, 0.0
 
 
-def test_two_layers_replay_from_a_graph(gpu_device, tmp_path):
+@pytest.mark.parametrize("block_size,n", [(128, 4096), (32, 1536)])  # (the second: the path of the smaller block sizes)
+def test_two_layers_replay_from_a_graph(gpu_device, tmp_path, block_size, n):
     from shareprefill_amd import AttentionSharing, shareprefill_attention_forward
 
-    hq, hkv, n = 8, 2, 4096
+    hq, hkv = 8, 2
     table = synthetic.random_cluster_table(hq, 2, 2, 3)
     path = synthetic.write_cluster_table(table, str(tmp_path / "table.json"))
     # fallback_threshold lifted: layer 1 shares the patterns layer 0's pivots left in the state
-    cfg = types.SimpleNamespace(block_size=128, min_budget=1024, max_budget=None, pattern_threshold=0.95,
+    cfg = types.SimpleNamespace(block_size=block_size, min_budget=8 * block_size, max_budget=None, pattern_threshold=0.95,
                                 similarity_threshold=0.5, fallback_threshold=1e9, queryaware_threshold=0.1,
                                 dense_short_prompts=False)
     sharing = AttentionSharing(path)
