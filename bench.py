@@ -130,7 +130,7 @@ def cpu_baseline(w, q, k, v, mask_bool, decision, kept_blocks, pt):
 # reported only while shareprefill_amd/csrc/sp_attn.hip still has that hash, and is null (with a note) after any
 # change to the kernel until the profile is taken again.
 MEASURED_ATTN_TRAFFIC = {
-    ("C3", 0.95): {"bytes": int((102.5 + 1.0) * 2 ** 30), "sp_attn_hip_sha256_16": "cec1d4a79675deff",
+    ("C3", 0.95): {"bytes": int((102.5 + 1.0) * 2 ** 30), "sp_attn_hip_sha256_16": "8d0a005a12007b26",
                    "profile": "profiles/attention_layer_C3_hbm_traffic.txt"},
 }
 
