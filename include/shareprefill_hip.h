@@ -112,7 +112,8 @@ int sp_pool_bf16(const void* x, void* y, int64_t n, int32_t h, int32_t d, int64_
  * (scaled by 1/sqrt(d), causal inside the last bs columns), column mean -> vert_tok[hq][n],
  * anti-diagonal mean -> slash_tok[hq][n], and their block sums vert_blk / slash_blk [hq][nb].
  * bs: 16, 32, 64 or 128 (attention_sharing.py:127 takes any; shareprefill_attn.py:509-516 allows these); d 128;
- * n >= 128 whatever bs (the kernels work on the last 128 tokens' queries and drop the rows a smaller block lacks).
+ * n >= bs (the kernels work on the last 128 token positions' queries and drop the rows a smaller block, or a
+ * shorter prompt, lacks).
  * workspace: sp_lastq_scores_workspace_bytes(...) bytes of device scratch. */
 size_t sp_lastq_scores_workspace_bytes(int64_t n, int32_t hq, int32_t bs);
 int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int32_t hq, int32_t hkv, int32_t d,

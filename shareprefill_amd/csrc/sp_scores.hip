@@ -36,7 +36,11 @@ template <bool REVERSED>
 __device__ static __forceinline__ void lq_load_q(const sp_bf16* __restrict__ q, int64_t n, int64_t sq_n, int wave, int lane,
                                         float inv_sqrt_d, bf16x8 (&qa)[8]) {
   const int row = REVERSED ? LQ_ROWS - 1 - (wave * 32 + (lane & 31)) : wave * 32 + (lane & 31);
-  const sp_bf16* src = q + (n - LQ_ROWS + row) * sq_n + 8 * (lane >> 5);
+  // (a prompt shorter than 128 tokens, possible with a block size below 128: the rows in front of its first token
+  // read token 0 and are dropped by the probabilities kernel like every row in front of the last block)
+  int64_t tok = n - LQ_ROWS + row;
+  if (tok < 0) tok = 0;
+  const sp_bf16* src = q + tok * sq_n + 8 * (lane >> 5);
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
     uint4 raw = *reinterpret_cast<const uint4*>(src + 16 * ks);
@@ -773,10 +777,6 @@ extern "C" int sp_lastq_scores_bf16(const void* q, const void* k, int64_t n, int
   SP_REQUIRE(d == LQ_D, SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: head_dim %d unsupported (only 128)", d);
   SP_REQUIRE(n >= bs, SP_ERR_INVALID_ARGUMENT, "sp_lastq_scores_bf16: seq_len %lld is shorter than one block",
              (long long)n);
-  // the kernels always work on the last 128 tokens' queries and drop the rows a smaller block does not have
-  SP_REQUIRE(n >= LQ_ROWS, SP_ERR_UNSUPPORTED,
-             "sp_lastq_scores_bf16: seq_len %lld is shorter than %d tokens (needed for block sizes below 128 too)",
-             (long long)n, LQ_ROWS);
   SP_REQUIRE(q_stride_n % 8 == 0 && q_stride_h % 8 == 0 && k_stride_n % 8 == 0 && k_stride_h % 8 == 0 &&
                  ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0,
              SP_ERR_UNSUPPORTED, "sp_lastq_scores_bf16: q/k must be 16-byte aligned with strides multiple of 8");

@@ -185,7 +185,7 @@ def test_layer_default_thresholds_small(gpu_device, tmp_path):
 
 
 @pytest.mark.parametrize("bs,n,hq,hkv", [(64, 2048, 8, 2), (64, 1100, 6, 2), (32, 1536, 8, 2), (32, 999, 4, 4),
-                                         (16, 1024, 8, 2), (16, 777, 7, 1)])
+                                         (16, 1024, 8, 2), (16, 777, 7, 1), (16, 100, 4, 2), (32, 127, 4, 2)])
 def test_layer_smaller_block_sizes(gpu_device, tmp_path, bs, n, hq, hkv):
     """block_size 64 / 32 / 16 (shareprefill_attn.py:509-516): the selection runs on N / bs blocks, the attention
     kernel walks the 128-token blocks that hold a kept block and drops the rest of them per 16 x 16 sub-tile.  Three

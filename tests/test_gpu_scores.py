@@ -62,7 +62,8 @@ def test_lastq_scores_seeded_random_shapes(gpu_device):
 
 
 @pytest.mark.parametrize("bs", [64, 32, 16])
-@pytest.mark.parametrize("hq,hkv,n", [(4, 2, 1024), (6, 2, 1000), (7, 1, 389), (2, 1, 128), (4, 4, 2100)])
+@pytest.mark.parametrize("hq,hkv,n", [(4, 2, 1024), (6, 2, 1000), (7, 1, 389), (2, 1, 128), (4, 4, 2100), (4, 2, 100),
+                                      (2, 2, 64), (3, 1, 127)])  # the last three: prompts shorter than 128 tokens
 def test_lastq_scores_smaller_block_sizes(gpu_device, bs, hq, hkv, n):
     """Block sizes below 128 (attention_sharing.py:127: the last bs queries): the same kernels with the rows in front
     of the last bs masked out; token vectors against the oracle with fp32 logits, block sums of bs tokens."""
