@@ -299,8 +299,8 @@ def test_block_wise_prefill_attention_small_head_dims(gpu_device, d):
 
 def _reference_side_binding():
     """The ctypes stub that the integration notes at the repository root show to a maintainer of the reference (the
-    module they would add as shareprefill/attn/hip_backend.py), taken from the notes themselves -- their first Python
-    block -- and executed against the in-tree library, so that the text shown there is the code tested here."""
+    module they would add as shareprefill/attn/hip_backend.py), taken from the notes themselves -- the Python block
+    that opens the library -- and executed against the in-tree library, so that the text shown there is the code tested here."""
     import types
 
     from shareprefill_amd import _lib
